@@ -1,0 +1,449 @@
+// extern "C" surface of libatex_norms_hip.so (declared in include/atex_norms.h).
+//
+// Kernel level: argument validation + routing to the row / channels-last launchers.
+// Op level: the host logic of the reference's OpKernel::Compute methods
+// (cc/kernels/fused_layer_norm_op.cc:295-352, :370-458;
+//  cc/kernels/fused_instance_norm_op.cc:328-406, :430-534) minus tensor allocation,
+// which stays with the caller.
+#include <algorithm>
+#include <cstring>
+#include <vector>
+
+#include "plan.h"
+#include "status.h"
+
+using namespace atexn;
+
+namespace {
+
+constexpr int kAbiVersion = 1;
+constexpr int64_t kMaxInt = 2147483647;
+
+bool dtype_ok(int dtype) { return dtype == ATEXN_F32 || dtype == ATEXN_F16 || dtype == ATEXN_BF16; }
+bool ws_aligned(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 255u) == 0; }
+
+int64_t num_elements(const atexn_tensor* t) {
+  int64_t n = 1;
+  for (int i = 0; i < t->rank; ++i) n *= t->dims[i];
+  return n;
+}
+
+bool same_shape(const atexn_tensor* a, const atexn_tensor* b) {
+  if (a->rank != b->rank) return false;
+  for (int i = 0; i < a->rank; ++i)
+    if (a->dims[i] != b->dims[i]) return false;
+  return true;
+}
+
+int check_tensor(const atexn_tensor* t, const char* name) {
+  ATEXN_REQUIRE(t != nullptr, "%s is NULL", name);
+  ATEXN_REQUIRE(t->rank >= 0 && t->rank <= ATEXN_MAX_RANK, "%s has unsupported rank %d", name, t->rank);
+  for (int i = 0; i < t->rank; ++i)
+    ATEXN_REQUIRE(t->dims[i] >= 0, "%s has negative dim %lld", name, (long long)t->dims[i]);
+  ATEXN_REQUIRE(num_elements(t) == 0 || t->data != nullptr, "%s has elements but a NULL data pointer", name);
+  return ATEXN_OK;
+}
+
+#define ATEXN_TRY(expr)             \
+  do {                              \
+    int s_ = (expr);                \
+    if (s_ != ATEXN_OK) return s_;  \
+  } while (0)
+
+}  // namespace
+
+extern "C" {
+
+const char* atexn_status_string(int status) {
+  switch (status) {
+    case ATEXN_OK: return "OK";
+    case ATEXN_INVALID_ARGUMENT: return "INVALID_ARGUMENT";
+    case ATEXN_LAUNCH_ERROR: return "LAUNCH_ERROR";
+    default: return "UNKNOWN";
+  }
+}
+
+const char* atexn_last_error(void) { return last_error(); }
+int atexn_abi_version(void) { return kAbiVersion; }
+
+/* Benchmark / tuning hook, not part of the drop-in contract: sets a launch-planning
+ * parameter by name for the whole process.  Returns ATEXN_INVALID_ARGUMENT for an unknown
+ * name or a value < 1. */
+int atexn_set_tuning(const char* name, int value) {
+  ATEXN_REQUIRE(name != nullptr && value >= 1, "bad tuning request");
+  Tuning& t = tuning();
+  if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
+  else if (!strcmp(name, "bwd_ln_threads")) {
+    ATEXN_REQUIRE(value == 256 || value == 512 || value == 1024, "bwd_ln_threads must be 256, 512 or 1024");
+    t.bwd_ln_threads = value;
+  } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
+  else if (!strcmp(name, "split_items_per_cu")) t.split_items_per_cu = value;
+  else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
+  else if (!strcmp(name, "colgrad_items_per_cu")) t.colgrad_items_per_cu = value;
+  else if (!strcmp(name, "bwd_stage_mask")) {
+    ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
+    t.bwd_stage_mask = value;
+  }
+  else return set_error(ATEXN_INVALID_ARGUMENT, "unknown tuning parameter '%s'", name);
+  return ATEXN_OK;
+}
+
+/* ------------------------------------------------------------------ kernel level */
+
+size_t atexn_layer_norm_fwd_workspace_bytes(int dtype, int64_t N, int64_t D) {
+  if (!dtype_ok(dtype)) return 0;
+  return rows_fwd_ws(dtype, false, N, D, 1);
+}
+
+int atexn_layer_norm_fwd(int dtype, const void* x, const float* gamma, const float* beta,
+                         int64_t N, int64_t D, float epsilon, void* y, float* mean,
+                         float* inv_std, void* workspace, size_t workspace_bytes,
+                         void* stream) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
+  if (N == 0 || D == 0) return ATEXN_OK;
+  ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
+  ATEXN_REQUIRE(workspace == nullptr || ws_aligned(workspace), "workspace must be 256-byte aligned");
+  return rows_fwd(dtype, false, x, gamma, beta, N, D, 1, epsilon, y, mean, inv_std, workspace,
+                  workspace_bytes, static_cast<hipStream_t>(stream));
+}
+
+size_t atexn_layer_norm_bwd_workspace_bytes(int dtype, int64_t N, int64_t D) {
+  if (!dtype_ok(dtype)) return 0;
+  return rows_bwd_ws(dtype, false, N, D, 1);
+}
+
+int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* gamma,
+                         const float* mean, const float* inv_std, int64_t N, int64_t D,
+                         void* dx, float* dgamma, float* dbeta, void* workspace,
+                         size_t workspace_bytes, void* stream) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (N == 0 || D == 0) {
+    if (D > 0) {
+      ATEXN_REQUIRE(dgamma && dbeta, "NULL pointer argument");
+      ATEXN_TRY(fill_zero(dgamma, D, st));
+      ATEXN_TRY(fill_zero(dbeta, D, st));
+    }
+    return ATEXN_OK;
+  }
+  ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
+  ATEXN_REQUIRE(dx != dy && dx != x, "dx must not alias dy or x");
+  ATEXN_REQUIRE(workspace != nullptr && ws_aligned(workspace), "workspace must be non-NULL and 256-byte aligned");
+  return rows_bwd(dtype, false, dy, x, gamma, mean, inv_std, N, D, 1, dx, dgamma, dbeta, workspace,
+                  workspace_bytes, st);
+}
+
+size_t atexn_instance_norm_fwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
+                                               int64_t D) {
+  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt) return 0;
+  return layout == ATEXN_LAYOUT_NC_ ? rows_fwd_ws(dtype, true, N * C, D, static_cast<int>(C))
+                                    : cl_fwd_ws(dtype, N, C, D);
+}
+
+int atexn_instance_norm_fwd(int dtype, int layout, const void* x, const float* gamma,
+                            const float* beta, int64_t N, int64_t C, int64_t D,
+                            float epsilon, void* y, float* mean, float* inv_std,
+                            void* workspace, size_t workspace_bytes, void* stream) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
+  ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
+  ATEXN_REQUIRE(C <= kMaxInt, "C=%lld too large", (long long)C);
+  if (N == 0 || C == 0 || D == 0) return ATEXN_OK;
+  ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
+  ATEXN_REQUIRE(workspace == nullptr || ws_aligned(workspace), "workspace must be 256-byte aligned");
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (layout == ATEXN_LAYOUT_NC_) {
+    return rows_fwd(dtype, true, x, gamma, beta, N * C, D, static_cast<int>(C), epsilon, y, mean,
+                    inv_std, workspace, workspace_bytes, st);
+  }
+  return cl_fwd(dtype, x, gamma, beta, N, C, D, epsilon, y, mean, inv_std, workspace,
+                workspace_bytes, st);
+}
+
+size_t atexn_instance_norm_bwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
+                                               int64_t D) {
+  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt) return 0;
+  return layout == ATEXN_LAYOUT_NC_ ? rows_bwd_ws(dtype, true, N * C, D, static_cast<int>(C))
+                                    : cl_bwd_ws(dtype, N, C, D);
+}
+
+int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x,
+                            const float* gamma, const float* mean, const float* inv_std,
+                            int64_t N, int64_t C, int64_t D, void* dx, float* dgamma,
+                            float* dbeta, void* workspace, size_t workspace_bytes,
+                            void* stream) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
+  ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
+  ATEXN_REQUIRE(C <= kMaxInt, "C=%lld too large", (long long)C);
+  hipStream_t st = static_cast<hipStream_t>(stream);
+  if (N == 0 || C == 0 || D == 0) {
+    if (C > 0) {
+      ATEXN_REQUIRE(dgamma && dbeta, "NULL pointer argument");
+      ATEXN_TRY(fill_zero(dgamma, C, st));
+      ATEXN_TRY(fill_zero(dbeta, C, st));
+    }
+    return ATEXN_OK;
+  }
+  ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
+  ATEXN_REQUIRE(dx != dy && dx != x, "dx must not alias dy or x");
+  ATEXN_REQUIRE(workspace != nullptr && ws_aligned(workspace), "workspace must be non-NULL and 256-byte aligned");
+  if (layout == ATEXN_LAYOUT_NC_) {
+    return rows_bwd(dtype, true, dy, x, gamma, mean, inv_std, N * C, D, static_cast<int>(C), dx,
+                    dgamma, dbeta, workspace, workspace_bytes, st);
+  }
+  return cl_bwd(dtype, dy, x, gamma, mean, inv_std, N, C, D, dx, dgamma, dbeta, workspace,
+                workspace_bytes, st);
+}
+
+/* ---------------------------------------------------------------------- op level */
+
+int atexn_layer_norm_resolve_axes(int rank, const int64_t* dims, const int* axis, int n_axis,
+                                  int64_t* N, int64_t* D) {
+  ATEXN_REQUIRE(rank >= 1 && rank <= ATEXN_MAX_RANK, "input must be at least 1-dimensional (rank %d)", rank);
+  ATEXN_REQUIRE(dims != nullptr && N != nullptr && D != nullptr, "NULL pointer argument");
+  /* an empty axis list is undefined behaviour in the reference (it indexes element 0 of an
+   * empty vector, norm_ops.cc:38); rejected here */
+  ATEXN_REQUIRE(axis != nullptr && n_axis >= 1, "axis must not be empty");
+  std::vector<int> ax;
+  for (int i = 0; i < n_axis; ++i) {
+    const int a = axis[i] < 0 ? rank + axis[i] : axis[i];
+    ATEXN_REQUIRE(a >= 0 && a < rank, "axis contains invalid value: %d", axis[i]);
+    ax.push_back(a);
+  }
+  std::sort(ax.begin(), ax.end());
+  ax.erase(std::unique(ax.begin(), ax.end()), ax.end());
+  ATEXN_REQUIRE(ax[0] == rank - static_cast<int>(ax.size()), "axis is not packed from last dim.");
+  int64_t n = 1, d = 1;
+  for (int i = 0; i < rank; ++i) {
+    ATEXN_REQUIRE(dims[i] >= 0, "negative dim");
+    if (i >= ax[0]) d *= dims[i]; else n *= dims[i];
+  }
+  *N = n;
+  *D = d;
+  return ATEXN_OK;
+}
+
+int atexn_instance_norm_resolve_format(int rank, const int64_t* dims, const char* data_format,
+                                       int* layout, int64_t* N, int64_t* C, int64_t* D) {
+  ATEXN_REQUIRE(dims != nullptr && layout && N && C && D, "NULL pointer argument");
+  ATEXN_REQUIRE(rank >= 4 && rank <= ATEXN_MAX_RANK, "input must be at least 4-dimensional (rank %d)", rank);
+  bool channel_first = false;
+  if (data_format != nullptr) {
+    const size_t n = strlen(data_format);
+    const bool ok = n > 2 && data_format[0] == 'N' && (data_format[1] == 'C' || data_format[n - 1] == 'C');
+    ATEXN_REQUIRE(ok, "We only accept 'NC...' or 'N...C' data format, but got %s", data_format);
+    channel_first = data_format[1] == 'C';
+  }
+  int64_t d = 1;
+  const int c_dim = channel_first ? 1 : rank - 1;
+  const int first = channel_first ? 2 : 1;
+  const int last = channel_first ? rank : rank - 1;
+  for (int i = first; i < last; ++i) d *= dims[i];
+  *layout = channel_first ? ATEXN_LAYOUT_NC_ : ATEXN_LAYOUT_N_C;
+  *N = dims[0];
+  *C = dims[c_dim];
+  *D = d;
+  return ATEXN_OK;
+}
+
+size_t atexn_fused_layer_norm_workspace_bytes(const atexn_tensor* x, const int* axis, int n_axis) {
+  int64_t N, D;
+  if (!x || atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D) != ATEXN_OK) return 0;
+  return atexn_layer_norm_fwd_workspace_bytes(x->dtype, N, D);
+}
+
+int atexn_fused_layer_norm(const atexn_tensor* x, const atexn_tensor* scale,
+                           const atexn_tensor* offset, float epsilon, const int* axis,
+                           int n_axis, atexn_tensor* y, atexn_tensor* reserve_space_1,
+                           atexn_tensor* reserve_space_2, void* workspace,
+                           size_t workspace_bytes, void* stream) {
+  ATEXN_TRY(check_tensor(x, "x"));
+  ATEXN_TRY(check_tensor(scale, "scale"));
+  ATEXN_TRY(check_tensor(offset, "offset"));
+  ATEXN_TRY(check_tensor(y, "y"));
+  ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
+  ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && offset->dtype == ATEXN_F32 &&
+                    reserve_space_1->dtype == ATEXN_F32 && reserve_space_2->dtype == ATEXN_F32,
+                "scale, offset and the reserve spaces must be float32");
+  ATEXN_REQUIRE(x->rank > 0, "input must be at least 1-dimensional");
+  int64_t N, D;
+  ATEXN_TRY(atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D));
+  ATEXN_REQUIRE(num_elements(scale) == D,
+                "scale must have the same number of elements as the features of x, got %lld and %lld",
+                (long long)num_elements(scale), (long long)D);
+  ATEXN_REQUIRE(num_elements(offset) == D,
+                "offset must have the same number of elements as the features of x, got %lld and %lld",
+                (long long)num_elements(offset), (long long)D);
+  ATEXN_REQUIRE(y->dtype == x->dtype && same_shape(x, y), "y must have the dtype and shape of x");
+  ATEXN_REQUIRE(reserve_space_1->rank == 1 && reserve_space_1->dims[0] == N &&
+                    reserve_space_2->rank == 1 && reserve_space_2->dims[0] == N,
+                "reserve spaces must be rank 1 with %lld elements", (long long)N);
+  return atexn_layer_norm_fwd(x->dtype, x->data, static_cast<const float*>(scale->data),
+                              static_cast<const float*>(offset->data), N, D, epsilon, y->data,
+                              static_cast<float*>(reserve_space_1->data),
+                              static_cast<float*>(reserve_space_2->data), workspace,
+                              workspace_bytes, stream);
+}
+
+size_t atexn_fused_layer_norm_grad_workspace_bytes(const atexn_tensor* x, const int* axis,
+                                                   int n_axis) {
+  int64_t N, D;
+  if (!x || atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D) != ATEXN_OK) return 0;
+  return atexn_layer_norm_bwd_workspace_bytes(x->dtype, N, D);
+}
+
+int atexn_fused_layer_norm_grad(const atexn_tensor* y_backprop, const atexn_tensor* x,
+                                const atexn_tensor* scale, const atexn_tensor* reserve_space_1,
+                                const atexn_tensor* reserve_space_2, const int* axis,
+                                int n_axis, atexn_tensor* x_backprop,
+                                atexn_tensor* scale_backprop, atexn_tensor* offset_backprop,
+                                void* workspace, size_t workspace_bytes, void* stream) {
+  ATEXN_TRY(check_tensor(y_backprop, "y_backprop"));
+  ATEXN_TRY(check_tensor(x, "x"));
+  ATEXN_TRY(check_tensor(scale, "scale"));
+  ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
+  ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_TRY(check_tensor(x_backprop, "x_backprop"));
+  ATEXN_TRY(check_tensor(scale_backprop, "scale_backprop"));
+  ATEXN_TRY(check_tensor(offset_backprop, "offset_backprop"));
+  ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && reserve_space_1->dtype == ATEXN_F32 &&
+                    reserve_space_2->dtype == ATEXN_F32 && scale_backprop->dtype == ATEXN_F32 &&
+                    offset_backprop->dtype == ATEXN_F32,
+                "scale, the reserve spaces and the scale/offset gradients must be float32");
+  ATEXN_REQUIRE(y_backprop->rank > 0 && x->rank > 0, "input must be at least 1-dimensional");
+  ATEXN_REQUIRE(reserve_space_1->rank == 1, "saved mean must be 1-dimensional");
+  ATEXN_REQUIRE(reserve_space_2->rank == 1, "saved inverted variance must be 1-dimensional");
+  ATEXN_REQUIRE(same_shape(x, y_backprop) && x->dtype == y_backprop->dtype,
+                "x and y_backprop must have same shape");
+  int64_t N, D;
+  ATEXN_TRY(atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D));
+  ATEXN_REQUIRE(num_elements(scale) == D,
+                "scale must have the same number of elements as the features of x, got %lld and %lld",
+                (long long)num_elements(scale), (long long)D);
+  ATEXN_REQUIRE(reserve_space_1->dims[0] == N,
+                "reserve_space_1 must have the same number of elements as the batches of x, got %lld and %lld",
+                (long long)reserve_space_1->dims[0], (long long)N);
+  ATEXN_REQUIRE(reserve_space_2->dims[0] == N,
+                "reserve_space_2 must have the same number of elements as the batches of x, got %lld and %lld",
+                (long long)reserve_space_2->dims[0], (long long)N);
+  ATEXN_REQUIRE(x_backprop->dtype == x->dtype && same_shape(x, x_backprop),
+                "x_backprop must have the dtype and shape of x");
+  ATEXN_REQUIRE(num_elements(scale_backprop) == D && num_elements(offset_backprop) == D,
+                "scale_backprop / offset_backprop must have %lld elements", (long long)D);
+  return atexn_layer_norm_bwd(x->dtype, y_backprop->data, x->data,
+                              static_cast<const float*>(scale->data),
+                              static_cast<const float*>(reserve_space_1->data),
+                              static_cast<const float*>(reserve_space_2->data), N, D,
+                              x_backprop->data, static_cast<float*>(scale_backprop->data),
+                              static_cast<float*>(offset_backprop->data), workspace,
+                              workspace_bytes, stream);
+}
+
+size_t atexn_fused_instance_norm_workspace_bytes(const atexn_tensor* x, const char* data_format) {
+  int layout;
+  int64_t N, C, D;
+  if (!x || atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D) != ATEXN_OK) return 0;
+  return atexn_instance_norm_fwd_workspace_bytes(x->dtype, layout, N, C, D);
+}
+
+int atexn_fused_instance_norm(const atexn_tensor* x, const atexn_tensor* scale,
+                              const atexn_tensor* offset, float epsilon,
+                              const char* data_format, atexn_tensor* y,
+                              atexn_tensor* reserve_space_1, atexn_tensor* reserve_space_2,
+                              void* workspace, size_t workspace_bytes, void* stream) {
+  ATEXN_TRY(check_tensor(x, "x"));
+  ATEXN_TRY(check_tensor(scale, "scale"));
+  ATEXN_TRY(check_tensor(offset, "offset"));
+  ATEXN_TRY(check_tensor(y, "y"));
+  ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
+  ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && offset->dtype == ATEXN_F32 &&
+                    reserve_space_1->dtype == ATEXN_F32 && reserve_space_2->dtype == ATEXN_F32,
+                "scale, offset and the reserve spaces must be float32");
+  ATEXN_REQUIRE(x->rank > 3, "input must be at least 4-dimensional");
+  ATEXN_REQUIRE(scale->rank == 1, "scale must be 1-dimensional");
+  ATEXN_REQUIRE(offset->rank == 1, "offset must be 1-dimensional");
+  int layout;
+  int64_t N, C, D;
+  ATEXN_TRY(atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D));
+  ATEXN_REQUIRE(scale->dims[0] == C,
+                "scale must have the same number of elements as the channels of x, got %lld and %lld",
+                (long long)scale->dims[0], (long long)C);
+  ATEXN_REQUIRE(offset->dims[0] == C,
+                "offset must have the same number of elements as the channels of x, got %lld and %lld",
+                (long long)offset->dims[0], (long long)C);
+  ATEXN_REQUIRE(y->dtype == x->dtype && same_shape(x, y), "y must have the dtype and shape of x");
+  ATEXN_REQUIRE(reserve_space_1->rank == 2 && reserve_space_1->dims[0] == N && reserve_space_1->dims[1] == C &&
+                    reserve_space_2->rank == 2 && reserve_space_2->dims[0] == N && reserve_space_2->dims[1] == C,
+                "reserve spaces must have shape [%lld, %lld]", (long long)N, (long long)C);
+  return atexn_instance_norm_fwd(x->dtype, layout, x->data, static_cast<const float*>(scale->data),
+                                 static_cast<const float*>(offset->data), N, C, D, epsilon, y->data,
+                                 static_cast<float*>(reserve_space_1->data),
+                                 static_cast<float*>(reserve_space_2->data), workspace,
+                                 workspace_bytes, stream);
+}
+
+size_t atexn_fused_instance_norm_grad_workspace_bytes(const atexn_tensor* x,
+                                                      const char* data_format) {
+  int layout;
+  int64_t N, C, D;
+  if (!x || atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D) != ATEXN_OK) return 0;
+  return atexn_instance_norm_bwd_workspace_bytes(x->dtype, layout, N, C, D);
+}
+
+int atexn_fused_instance_norm_grad(const atexn_tensor* y_backprop, const atexn_tensor* x,
+                                   const atexn_tensor* scale,
+                                   const atexn_tensor* reserve_space_1,
+                                   const atexn_tensor* reserve_space_2,
+                                   const char* data_format, atexn_tensor* x_backprop,
+                                   atexn_tensor* scale_backprop,
+                                   atexn_tensor* offset_backprop, void* workspace,
+                                   size_t workspace_bytes, void* stream) {
+  ATEXN_TRY(check_tensor(y_backprop, "y_backprop"));
+  ATEXN_TRY(check_tensor(x, "x"));
+  ATEXN_TRY(check_tensor(scale, "scale"));
+  ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
+  ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_TRY(check_tensor(x_backprop, "x_backprop"));
+  ATEXN_TRY(check_tensor(scale_backprop, "scale_backprop"));
+  ATEXN_TRY(check_tensor(offset_backprop, "offset_backprop"));
+  ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && reserve_space_1->dtype == ATEXN_F32 &&
+                    reserve_space_2->dtype == ATEXN_F32 && scale_backprop->dtype == ATEXN_F32 &&
+                    offset_backprop->dtype == ATEXN_F32,
+                "scale, the reserve spaces and the scale/offset gradients must be float32");
+  ATEXN_REQUIRE(y_backprop->rank > 3, "input must be at least 4-dimensional");
+  ATEXN_REQUIRE(scale->rank == 1, "scale must be 1-dimensional");
+  ATEXN_REQUIRE(reserve_space_1->rank == 2, "saved mean must be 2-dimensional");
+  ATEXN_REQUIRE(reserve_space_2->rank == 2, "saved inverted variance must be 2-dimensional");
+  ATEXN_REQUIRE(same_shape(x, y_backprop) && x->dtype == y_backprop->dtype,
+                "x and y_backprop must have same shape");
+  int layout;
+  int64_t N, C, D;
+  ATEXN_TRY(atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D));
+  ATEXN_REQUIRE(scale->dims[0] == C,
+                "scale must have the same number of elements as the channels of x, got %lld and %lld",
+                (long long)scale->dims[0], (long long)C);
+  ATEXN_REQUIRE(num_elements(reserve_space_1) == N * C,
+                "reserve_space_1 must have the same number of elements as the batches*channels of x, got %lld and %lld",
+                (long long)num_elements(reserve_space_1), (long long)(N * C));
+  ATEXN_REQUIRE(num_elements(reserve_space_2) == N * C,
+                "reserve_space_2 must have the same number of elements as the batches*channels of x, got %lld and %lld",
+                (long long)num_elements(reserve_space_2), (long long)(N * C));
+  ATEXN_REQUIRE(x_backprop->dtype == x->dtype && same_shape(x, x_backprop),
+                "x_backprop must have the dtype and shape of x");
+  ATEXN_REQUIRE(num_elements(scale_backprop) == C && num_elements(offset_backprop) == C,
+                "scale_backprop / offset_backprop must have %lld elements", (long long)C);
+  return atexn_instance_norm_bwd(x->dtype, layout, y_backprop->data, x->data,
+                                 static_cast<const float*>(scale->data),
+                                 static_cast<const float*>(reserve_space_1->data),
+                                 static_cast<const float*>(reserve_space_2->data), N, C, D,
+                                 x_backprop->data, static_cast<float*>(scale_backprop->data),
+                                 static_cast<float*>(offset_backprop->data), workspace,
+                                 workspace_bytes, stream);
+}
+
+}  // extern "C"

@@ -1,0 +1,82 @@
+// Launchers for the channels-last InstanceNorm kernels, templated on the storage type.
+#pragma once
+
+#include "cl_kernels.cuh"
+#include "plan.h"
+#include "status.h"
+
+namespace atexn {
+
+template <typename T, int V>
+int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64_t C, int64_t D,
+             float eps, T* y, float* mean, float* rstd, void* ws, size_t ws_bytes,
+             hipStream_t st) {
+  const ClPlan p = plan_cl(false, V, N, C, D, cu_count());
+  ATEXN_REQUIRE(ws != nullptr && ws_bytes >= p.ws_bytes,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  float* pmean = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
+  float* pm2 = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_b);
+  const int Ci = static_cast<int>(C);
+  cl_fwd_stats<T, V><<<p.grid, kClThreads, 0, st>>>(x, pmean, pm2, p.n_work, D, Ci, p.S, p.CT,
+                                                   p.TPP, p.slab_len);
+  ATEXN_CHECK_LAUNCH("cl_fwd_stats");
+  cl_fwd_apply<T, V><<<p.grid, kClThreads, 0, st>>>(x, pmean, pm2, gamma, beta, y, mean, rstd,
+                                                   p.n_work, D, Ci, p.S, p.CT, p.TPP, p.slab_len,
+                                                   eps);
+  ATEXN_CHECK_LAUNCH("cl_fwd_apply");
+  return ATEXN_OK;
+}
+
+template <typename T, int V>
+int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, const float* rstd,
+             int64_t N, int64_t C, int64_t D, T* dx, float* dgamma, float* dbeta, void* ws,
+             size_t ws_bytes, hipStream_t st) {
+  const ClPlan p = plan_cl(true, V, N, C, D, cu_count());
+  ATEXN_REQUIRE(ws != nullptr && ws_bytes >= p.ws_bytes,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  float* part = static_cast<float*>(ws);
+  const int Ci = static_cast<int>(C);
+  cl_bwd_sums<T, V><<<p.grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, p.n_work, D, Ci, p.S,
+                                                  p.CT, p.TPP, p.slab_len);
+  ATEXN_CHECK_LAUNCH("cl_bwd_sums");
+  cl_bwd_apply<T, V><<<p.grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx, p.n_work,
+                                                   D, Ci, p.S, p.CT, p.TPP, p.slab_len);
+  ATEXN_CHECK_LAUNCH("cl_bwd_apply");
+  return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N * p.S), C, st);
+}
+
+template <typename T>
+int cl_fwd_t(const void* x_, const float* gamma, const float* beta, int64_t N, int64_t C,
+             int64_t D, float eps, void* y_, float* mean, float* rstd, void* ws, size_t ws_bytes,
+             hipStream_t st) {
+  constexpr int VEC = VecOf<T>::value;
+  const T* x = static_cast<const T*>(x_);
+  T* y = static_cast<T*>(y_);
+  const bool vec = (C % VEC == 0) && aligned16(x) && aligned16(y) && aligned16(gamma) &&
+                   aligned16(beta) && aligned16(mean) && aligned16(rstd);
+  return vec ? cl_fwd_v<T, VEC>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st)
+             : cl_fwd_v<T, 1>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st);
+}
+
+template <typename T>
+int cl_bwd_t(const void* dy_, const void* x_, const float* gamma, const float* mean,
+             const float* rstd, int64_t N, int64_t C, int64_t D, void* dx_, float* dgamma,
+             float* dbeta, void* ws, size_t ws_bytes, hipStream_t st) {
+  constexpr int VEC = VecOf<T>::value;
+  const T* x = static_cast<const T*>(x_);
+  const T* dy = static_cast<const T*>(dy_);
+  T* dx = static_cast<T*>(dx_);
+  const bool vec = (C % VEC == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
+                   aligned16(gamma) && aligned16(mean) && aligned16(rstd);
+  return vec ? cl_bwd_v<T, VEC>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st)
+             : cl_bwd_v<T, 1>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st);
+}
+
+#define ATEXN_INSTANTIATE_CL(T)                                                                  \
+  template int cl_fwd_t<T>(const void*, const float*, const float*, int64_t, int64_t, int64_t,   \
+                           float, void*, float*, float*, void*, size_t, hipStream_t);            \
+  template int cl_bwd_t<T>(const void*, const void*, const float*, const float*, const float*,   \
+                           int64_t, int64_t, int64_t, void*, float*, float*, void*, size_t,      \
+                           hipStream_t);
+
+}  // namespace atexn

@@ -1,0 +1,180 @@
+// Host-side launch planning: which kernel family, which geometry and how much workspace
+// a call needs.  Pure host code with no HIP dependency, shared by the launchers and by
+// the *_workspace_bytes queries so that both always agree.
+//
+// It plays the part of the reference's dispatch ladders
+// (fused_layer_norm_op.cu:824-891, :919-1028; fused_instance_norm_op.cu:1203-1561) but
+// decides from alignment, row length and the CU count instead of from occupancy probes
+// against a 48 KB shared-memory limit.
+#pragma once
+
+#include <stddef.h>
+#include <stdint.h>
+
+#include <algorithm>
+
+namespace atexn {
+
+// Tunables (process-wide; defaults chosen by measurement on MI355X).
+struct Tuning {
+  int fwd_waves_per_cu = 32;      // resident forward: waves kept resident per CU
+  int bwd_ln_threads = 1024;      // resident LayerNorm backward, rows <= one wave: block size
+  int bwd_waves_per_cu = 16;      // resident backward: waves kept resident per CU
+  int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
+  int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
+  int colgrad_items_per_cu = 4;   // LayerNorm column pass of the split path
+  // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
+  // bit 1: the final column reduction).  Anything but 3 gives incomplete results.
+  int bwd_stage_mask = 3;
+};
+Tuning& tuning();
+
+enum class RowsKind { kFwd, kBwdCols /*LayerNorm: per-column dgamma/dbeta*/, kBwdAffine };
+
+inline int64_t div_up(int64_t a, int64_t b) { return (a + b - 1) / b; }
+inline int64_t round_up(int64_t a, int64_t b) { return div_up(a, b) * b; }
+inline size_t align256(size_t b) { return (b + 255) & ~static_cast<size_t>(255); }
+inline int pow2_ceil(int64_t v) {
+  int p = 1;
+  while (p < v) p <<= 1;
+  return p;
+}
+
+struct RowsPlan {
+  int V = 1;  // storage elements per access
+  bool resident = false;
+  // resident
+  int tpr = 0, vpt = 1, threads = 256, rpb = 1;
+  int grid = 1;
+  size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
+  // split
+  int S = 1;
+  int64_t chunk = 0;
+  int split_grid = 1;
+  int col_tiles = 0;  // LayerNorm backward column pass
+  int col_slabs = 0;
+  int64_t rows_per_slab = 0;
+  // workspace sections (bytes from the start of the workspace)
+  size_t off_part = 0, off_pairs = 0, ws_bytes = 0;
+  int part_rows = 0;  // G of the column reduction
+};
+
+// V: vector width in elements (16 / sizeof(T)) when the call is 16-byte aligned, else 1.
+inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
+  const Tuning& t = tuning();
+  RowsPlan p;
+  p.V = V;
+  const int64_t n_vec = D / V;  // D % V == 0 whenever V > 1
+  // Limits follow the register budgets of the resident kernels: forward 1024 threads x 8
+  // vectors; backward 512 threads x 8 (InstanceNorm) or x 4 (LayerNorm, which also keeps
+  // gamma and the dgamma / dbeta accumulators of its columns in registers).
+  const int64_t resident_limit =
+      kind == RowsKind::kFwd ? 8192 : (kind == RowsKind::kBwdAffine ? 4096 : 2048);
+  p.resident = n_vec <= resident_limit;
+  if (p.resident) {
+    if (n_vec <= 64) {
+      p.tpr = std::max(8, pow2_ceil(n_vec));
+      p.vpt = 1;
+    } else if (n_vec <= 128) {
+      p.tpr = 64;
+      p.vpt = 2;
+    } else {
+      p.tpr = 0;
+      p.vpt = n_vec <= 1024 ? 2 : (n_vec <= 2048 ? 4 : 8);
+    }
+    if (p.tpr == 0) {
+      p.threads = static_cast<int>(round_up(div_up(n_vec, p.vpt), 64));
+      p.rpb = 1;
+    } else {
+      p.threads = 256;
+      if (kind == RowsKind::kBwdCols) {
+        // bigger blocks -> fewer partial rows for the column reduction
+        int th = t.bwd_ln_threads;
+        while (th > 256 && div_up(n_rows, th / p.tpr) < cus) th /= 2;
+        p.threads = th;
+      }
+      p.rpb = p.threads / p.tpr;
+    }
+    const int64_t groups = div_up(n_rows, p.rpb);
+    const int waves = p.threads / 64;
+    const int per_cu = std::max(
+        1, (kind == RowsKind::kFwd ? t.fwd_waves_per_cu : t.bwd_waves_per_cu) / waves);
+    p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(groups, int64_t(cus) * per_cu)));
+    if (kind == RowsKind::kBwdCols) {
+      p.part_rows = p.grid;
+      p.off_part = 0;
+      p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
+      if (p.tpr != 0) p.fold_lds = size_t(std::min(waves / 2, 4)) * 2 * size_t(V * p.vpt) * 64 * sizeof(float);
+    } else if (kind == RowsKind::kBwdAffine) {
+      p.part_rows = static_cast<int>(n_rows / C);
+      p.off_part = 0;
+      p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
+    }
+    return p;
+  }
+  // split rows
+  const int64_t gran = int64_t(256) * V;  // one block sweep
+  const int64_t want = div_up(int64_t(cus) * t.split_items_per_cu, std::max<int64_t>(n_rows, 1));
+  const int64_t max_s = std::max<int64_t>(1, D / (gran * 4));
+  int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), 1024));
+  p.chunk = round_up(div_up(D, S), gran);
+  p.S = static_cast<int>(div_up(D, p.chunk));
+  const int64_t n_work = n_rows * p.S;
+  p.split_grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(n_work, int64_t(cus) * 32)));
+  p.off_pairs = 0;
+  size_t bytes = align256(sizeof(float) * 2 * size_t(n_work));
+  if (kind == RowsKind::kBwdCols) {
+    p.col_tiles = static_cast<int>(div_up(D, 256));
+    int64_t slabs = div_up(int64_t(cus) * t.colgrad_items_per_cu, p.col_tiles);
+    slabs = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(slabs, n_rows), 1024));
+    p.rows_per_slab = div_up(n_rows, slabs);
+    p.col_slabs = static_cast<int>(div_up(n_rows, p.rows_per_slab));
+    p.part_rows = p.col_slabs;
+    p.off_part = bytes;
+    bytes += align256(sizeof(float) * 2 * size_t(D) * size_t(p.col_slabs));
+  } else if (kind == RowsKind::kBwdAffine) {
+    p.part_rows = static_cast<int>(n_rows / C);
+    p.off_part = bytes;
+    bytes += align256(sizeof(float) * 2 * size_t(n_rows));
+  }
+  p.ws_bytes = bytes;
+  return p;
+}
+
+// Channels-last InstanceNorm, x as [N, D, C].
+struct ClPlan {
+  int V = 1;
+  int CV = 1;    // channel vectors per pixel
+  int TPP = 1;   // threads per pixel (power of two <= 256)
+  int CT = 1;    // channel tiles
+  int S = 1;     // slabs per instance
+  int64_t slab_len = 0;
+  int64_t n_work = 0;
+  int grid = 1;
+  size_t off_a = 0, off_b = 0, ws_bytes = 0;
+};
+
+inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
+  const Tuning& t = tuning();
+  ClPlan p;
+  p.V = V;
+  p.CV = static_cast<int>(div_up(C, V));
+  p.TPP = std::min(256, pow2_ceil(p.CV));
+  p.CT = static_cast<int>(div_up(p.CV, p.TPP));
+  const int ppb = 256 / p.TPP;
+  const int64_t want = div_up(int64_t(cus) * t.cl_items_per_cu, std::max<int64_t>(N * p.CT, 1));
+  const int64_t max_s = std::max<int64_t>(1, D / (int64_t(ppb) * 4));
+  const int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), 4096));
+  p.slab_len = round_up(div_up(D, S), ppb);
+  p.S = static_cast<int>(div_up(D, p.slab_len));
+  p.n_work = N * p.S * p.CT;
+  p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(p.n_work, int64_t(cus) * 32)));
+  const size_t sect = align256(sizeof(float) * size_t(N) * size_t(p.S) * size_t(C));
+  p.off_a = 0;
+  p.off_b = sect;
+  p.ws_bytes = 2 * sect;  // fwd: pmean + pm2 ; bwd: part[N*S][2][C] (contiguous, 2 sections)
+  (void)bwd;
+  return p;
+}
+
+}  // namespace atexn

@@ -1,0 +1,685 @@
+// Kernels for contiguous rows: LayerNorm over [N, D] and channel-first InstanceNorm
+// over [N*C, D].  They replace the reference's row ladders
+//   forward   fused_layer_norm_op.cu:375-433 (warp/row), :145-193 (block/row, smem),
+//             :573-684 (multi-block), fused_instance_norm_op.cu:959-1004, :1167-1194
+//   backward  fused_layer_norm_op.cu:21-98, :195-255, :523-561, :635-719, :742-803,
+//             fused_instance_norm_op.cu:169-313, :315-366, :594-656
+// with two designs:
+//   * "resident" kernels: the row lives in VGPRs (TPR threads x VPT 128-bit vectors),
+//     is read from HBM exactly once, and its statistics come from an exact local
+//     two-pass followed by a Chan/Welford butterfly across lanes (and LDS across waves);
+//   * "split" kernels for rows that do not fit or are not 16-byte aligned: a row is cut
+//     into S chunks, stage 1 writes per-chunk partials, stage 2 merges them and applies.
+#pragma once
+
+#include "norm_common.cuh"
+
+namespace atexn {
+
+// Geometry of the thread <-> row mapping.  TPR > 0: TPR (power of two <= 64) lanes per
+// row and blockDim.x / TPR rows per block.  TPR == 0: the whole block owns one row.
+template <int TPR>
+struct RowMap {
+  __device__ __forceinline__ static int tpr() { return TPR ? TPR : static_cast<int>(blockDim.x); }
+  __device__ __forceinline__ static int rows_per_block() { return TPR ? static_cast<int>(blockDim.x) / TPR : 1; }
+  __device__ __forceinline__ static int lane_in_row() {
+    return TPR ? static_cast<int>(threadIdx.x) % TPR : static_cast<int>(threadIdx.x);
+  }
+  __device__ __forceinline__ static int slot() { return TPR ? static_cast<int>(threadIdx.x) / TPR : 0; }
+};
+
+// Waves whose accumulators pass through LDS in one step of the backward fold.
+constexpr int kFoldWaves = 4;
+
+// Largest block a resident kernel instantiation is launched with; it fixes the VGPR
+// budget the compiler works against (512 VGPRs per SIMD lane / waves per SIMD).
+template <int TPR, int VPT>
+constexpr int resident_fwd_max_threads() {
+  if (TPR != 0) return 256;
+  return VPT >= 8 ? 1024 : 512;
+}
+template <int TPR, bool BWD_COLS>
+constexpr int resident_bwd_max_threads() {
+  if (TPR != 0) return BWD_COLS ? 1024 : 256;
+  return 512;
+}
+
+// ------------------------------------------------------------------ forward, resident
+// y = (x - mean) * inv_std * gamma + beta ; mean / inv_std saved per row.
+// ROW_AFFINE: gamma / beta are indexed by (row % C) (channel-first InstanceNorm) instead
+// of by column (LayerNorm).  y may alias x: every thread reads all of its vectors of a
+// row before it writes any.  The row is kept as raw 128-bit vectors and converted on
+// use, which halves the register footprint for 16-bit storage.
+template <typename T, int V, int TPR, int VPT, bool ROW_AFFINE>
+__global__ void __launch_bounds__((resident_fwd_max_threads<TPR, VPT>()))
+rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta,
+                  T* y, float* __restrict__ mean_out, float* __restrict__ rstd_out,
+                  int64_t n_rows, int n_vec, int C, float eps) {
+  using M = RowMap<TPR>;
+  constexpr int NE = V * VPT;
+  // gamma / beta live in registers across rows unless that would exhaust the budget
+  constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 4);
+  __shared__ Wf wf_buf[2][16];
+
+  const int tpr = M::tpr();
+  const int rpb = M::rows_per_block();
+  const int lane_r = M::lane_in_row();
+  const int slot = M::slot();
+  const int64_t D = static_cast<int64_t>(n_vec) * V;
+
+  int n_valid_vec = 0;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+
+  float g[GB_REGS ? NE : 1], b[GB_REGS ? NE : 1];
+  if constexpr (GB_REGS) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      float tg[V], tb[V];
+      if (k < n_valid_vec) {
+        const int col = (lane_r + k * tpr) * V;
+        load_f32<V>(gamma + col, tg);
+        load_f32<V>(beta + col, tb);
+      } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) tg[i] = tb[i] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        g[k * V + i] = tg[i];
+        b[k * V + i] = tb[i];
+      }
+    }
+  }
+
+  int it = 0;
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb; row0 < n_rows;
+       row0 += static_cast<int64_t>(gridDim.x) * rpb, ++it) {
+    const int64_t row = row0 + slot;
+    const bool row_ok = row < n_rows;
+    const int nv = row_ok ? n_valid_vec : 0;
+    const T* xr = x + row * D;
+    Pack<T, V> raw[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < nv) raw[k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
+    }
+    // statistics of this thread's elements: exact two-pass over registers
+    Wf w{0.f, 0.f, static_cast<float>(nv * V)};
+    if (nv > 0) {
+      float s = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv) {
+#pragma unroll
+          for (int i = 0; i < V; ++i) s += to_f32(raw[k].v[i]);
+        }
+      }
+      w.mean = s / w.n;
+      float q = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv) {
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const float d = to_f32(raw[k].v[i]) - w.mean;
+            q += d * d;
+          }
+        }
+      }
+      w.m2 = q;
+    }
+    if constexpr (TPR != 0) {
+      w = group_wf<(TPR ? TPR : 1)>(w);
+    } else {
+      w = block_wf(w, wf_buf[it & 1]);
+    }
+    const float mean = w.mean;
+    const float rstd = rsqrtf(w.m2 / static_cast<float>(D) + eps);
+
+    float gs = 1.f, bs = 0.f;
+    if constexpr (ROW_AFFINE) {
+      if (row_ok) {
+        const int c = static_cast<int>(row % C);
+        gs = gamma[c];
+        bs = beta[c];
+      }
+    }
+    T* yr = y + row * D;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < nv) {
+        const int col = (lane_r + k * tpr) * V;
+        float tg[V], tb[V];
+        if constexpr (!ROW_AFFINE && !GB_REGS) {
+          load_f32<V>(gamma + col, tg);
+          load_f32<V>(beta + col, tb);
+        }
+        Pack<T, V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          const float xh = (to_f32(raw[k].v[i]) - mean) * rstd;
+          float r;
+          if constexpr (ROW_AFFINE) {
+            r = xh * gs + bs;
+          } else if constexpr (GB_REGS) {
+            r = xh * g[k * V + i] + b[k * V + i];
+          } else {
+            r = xh * tg[i] + tb[i];
+          }
+          o.v[i] = from_f32<T>(r);
+        }
+        store_pack<T, V>(yr + col, o);
+      }
+    }
+    if (row_ok && lane_r == 0) {
+      mean_out[row] = mean;
+      rstd_out[row] = rstd;
+    }
+  }
+}
+
+// ----------------------------------------------------------------- backward, resident
+// Per row, with xh = (x - mean) * r and g = dy * gamma:
+//   s1 = sum g, s2 = sum g * xh, dx = r * (g - (s1 + xh * s2) / D)
+// which is the reference's (2 (x - mean) dl_dvar + dl_dmu) / D + g r
+// (fused_layer_norm_op.cu:84-88, norm_util.h:369-372,408-410) with
+// dl_dvar = -1/2 r^3 sum g (x - mean), dl_dmu = -r s1.
+//
+// LayerNorm (ROW_AFFINE = false): every thread also accumulates, over all rows it
+// visits, dgamma_j += dy * xh and dbeta_j += dy for the columns it owns; at the end the
+// block folds them (lanes, then waves through LDS, fixed order) and writes ONE partial
+// row part[blockIdx.x][0][0..D) (dgamma) and part[blockIdx.x][1][0..D) (dbeta); a second
+// kernel sums the partial rows.  `part` has gridDim.x * 2 * D floats.
+//
+// InstanceNorm channel-first (ROW_AFFINE = true): gamma is the scalar of channel
+// row % C, the two row sums a = sum dy, b = sum dy * xh give s1 = gamma a, s2 = gamma b and
+// are written to part[n][0][c] = b, part[n][1][c] = a  (n = row / C), i.e. `part` has
+// N * 2 * C floats and the same second kernel folds it over n.
+// dx must not alias dy or x.
+template <typename T, int V, int TPR, int VPT, bool ROW_AFFINE>
+__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE>()))
+rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
+                  const float* __restrict__ gamma, const float* __restrict__ mean_in,
+                  const float* __restrict__ rstd_in, T* __restrict__ dx,
+                  float* __restrict__ part, int64_t n_rows, int n_vec, int C) {
+  using M = RowMap<TPR>;
+  constexpr int NE = V * VPT;
+  __shared__ float2 sum_buf[2][16];
+  // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats
+  extern __shared__ float fold_buf[];
+
+  const int tpr = M::tpr();
+  const int rpb = M::rows_per_block();
+  const int lane_r = M::lane_in_row();
+  const int slot = M::slot();
+  const int64_t D = static_cast<int64_t>(n_vec) * V;
+  const float inv_d = 1.0f / static_cast<float>(D);
+
+  int n_valid_vec = 0;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+
+  float g[ROW_AFFINE ? 1 : NE];
+  float acc_g[ROW_AFFINE ? 1 : NE], acc_b[ROW_AFFINE ? 1 : NE];
+  if constexpr (!ROW_AFFINE) {
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      float tg[V];
+      if (k < n_valid_vec) {
+        load_f32<V>(gamma + (lane_r + k * tpr) * V, tg);
+      } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) tg[i] = 0.f;
+      }
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        g[k * V + i] = tg[i];
+        acc_g[k * V + i] = 0.f;
+        acc_b[k * V + i] = 0.f;
+      }
+    }
+  }
+
+  int it = 0;
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb; row0 < n_rows;
+       row0 += static_cast<int64_t>(gridDim.x) * rpb, ++it) {
+    const int64_t row = row0 + slot;
+    const bool row_ok = row < n_rows;
+    const int nv = row_ok ? n_valid_vec : 0;
+    const T* xr = x + row * D;
+    const T* dyr = dy + row * D;
+    Pack<T, V> px[VPT], pd[VPT];
+    float mean = 0.f, rstd = 0.f, gs = 0.f;
+    if (row_ok) {
+      mean = mean_in[row];
+      rstd = rstd_in[row];
+      if constexpr (ROW_AFFINE) gs = gamma[static_cast<int>(row % C)];
+    }
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < nv) {
+        const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
+        px[k] = load_pack<T, V>(xr + off);
+        pd[k] = load_pack<T, V>(dyr + off);
+      }
+    }
+    float s1 = 0.f, s2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < nv) {
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          const float xh = (to_f32(px[k].v[i]) - mean) * rstd;
+          const float d = to_f32(pd[k].v[i]);
+          if constexpr (ROW_AFFINE) {
+            s1 += d;
+            s2 += d * xh;
+          } else {
+            const float gv = d * g[k * V + i];
+            s1 += gv;
+            s2 += gv * xh;
+            acc_g[k * V + i] += d * xh;
+            acc_b[k * V + i] += d;
+          }
+        }
+      }
+    }
+    if constexpr (TPR != 0) {
+      s1 = group_sum<(TPR ? TPR : 1)>(s1);
+      s2 = group_sum<(TPR ? TPR : 1)>(s2);
+    } else {
+      const float2 r = block_sum2(s1, s2, sum_buf[it & 1]);
+      s1 = r.x;
+      s2 = r.y;
+    }
+    if constexpr (ROW_AFFINE) {
+      if (row_ok && lane_r == 0) {
+        const int64_t n = row / C;
+        const int c = static_cast<int>(row % C);
+        part[(n * 2 + 0) * C + c] = s2;
+        part[(n * 2 + 1) * C + c] = s1;
+      }
+    }
+    T* dxr = dx + row * D;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (k < nv) {
+        Pack<T, V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          const float xh = (to_f32(px[k].v[i]) - mean) * rstd;
+          const float d = to_f32(pd[k].v[i]);
+          float r;
+          if constexpr (ROW_AFFINE) {
+            r = rstd * gs * (d - (s1 + xh * s2) * inv_d);
+          } else {
+            r = rstd * (d * g[k * V + i] - (s1 + xh * s2) * inv_d);
+          }
+          o.v[i] = from_f32<T>(r);
+        }
+        store_pack<T, V>(dxr + static_cast<int64_t>(lane_r + k * tpr) * V, o);
+      }
+    }
+  }
+
+  if constexpr (!ROW_AFFINE) {
+    float* prow = part + static_cast<int64_t>(blockIdx.x) * 2 * D;
+    if constexpr (TPR == 0) {
+      // one row per block: every thread owns its columns outright
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < n_valid_vec) {
+          const int col = (lane_r + k * tpr) * V;
+          float tg[V], tb[V];
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            tg[i] = acc_g[k * V + i];
+            tb[i] = acc_b[k * V + i];
+          }
+          store_f32<V>(prow + col, tg);
+          store_f32<V>(prow + D + col, tb);
+        }
+      }
+    } else {
+      // 1) fold the row slots that share a wave (lanes l, l+TPR, ... own the same columns)
+      if constexpr (TPR < kWave && TPR != 0) {
+#pragma unroll
+        for (int i = 0; i < NE; ++i) {
+#pragma unroll
+          for (int m = (TPR ? TPR : 1); m < kWave; m <<= 1) {
+            acc_g[i] += lane_xor(acc_g[i], m);
+            acc_b[i] += lane_xor(acc_b[i], m);
+          }
+        }
+      }
+      // 2) fold waves pairwise through LDS: upper half writes, lower half adds
+      const int lane = threadIdx.x & (kWave - 1);
+      const int wave = threadIdx.x / kWave;
+      const int nw = blockDim.x / kWave;
+      // (at most kFoldWaves waves' worth of LDS is used per step)
+      for (int half = nw / 2; half >= 1; half >>= 1) {
+        for (int base = 0; base < half; base += kFoldWaves) {
+          const int src_wave = wave - half - base;  // index among the writers of this step
+          if (src_wave >= 0 && src_wave < kFoldWaves && wave < 2 * half) {
+            float* dst = fold_buf + static_cast<size_t>(src_wave) * (2 * NE) * kWave;
+#pragma unroll
+            for (int i = 0; i < NE; ++i) {
+              dst[(2 * i) * kWave + lane] = acc_g[i];
+              dst[(2 * i + 1) * kWave + lane] = acc_b[i];
+            }
+          }
+          __syncthreads();
+          const int dst_wave = wave - base;
+          if (dst_wave >= 0 && dst_wave < kFoldWaves && wave < half) {
+            const float* src = fold_buf + static_cast<size_t>(dst_wave) * (2 * NE) * kWave;
+#pragma unroll
+            for (int i = 0; i < NE; ++i) {
+              acc_g[i] += src[(2 * i) * kWave + lane];
+              acc_b[i] += src[(2 * i + 1) * kWave + lane];
+            }
+          }
+          __syncthreads();
+        }
+      }
+      if (wave == 0 && lane < tpr) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+          if (k < n_valid_vec) {
+            const int col = (lane_r + k * tpr) * V;
+            float tg[V], tb[V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) {
+              tg[i] = acc_g[k * V + i];
+              tb[i] = acc_b[k * V + i];
+            }
+            store_f32<V>(prow + col, tg);
+            store_f32<V>(prow + D + col, tb);
+          }
+        }
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------- column reduction
+// out0[j] = sum_g part[g][0][j], out1[j] = sum_g part[g][1][j] for j < W, g < G, summed
+// in a fixed order (deterministic; the reference likewise uses no atomics,
+// fused_layer_norm_op.cu:763-803, fused_instance_norm_op.cu:442-457).
+// Block = (CX column groups of CW floats) x (CY slices of g).  blockDim.x = CX * CY.
+template <int CW, int CX, int CY>
+__global__ void col_reduce(const float* __restrict__ part, float* __restrict__ out0,
+                           float* __restrict__ out1, int G, int W) {
+  __shared__ float buf[CY][CX][CW];
+  const int cx = threadIdx.x % CX;
+  const int cy = threadIdx.x / CX;
+  const int W2 = 2 * W;
+  const int col = (blockIdx.x * CX + cx) * CW;  // column in the concatenated [2W] row
+  float acc[CW];
+#pragma unroll
+  for (int i = 0; i < CW; ++i) acc[i] = 0.f;
+  if (col < W2) {
+    for (int g = cy; g < G; g += CY) {
+      float t[CW];
+      load_f32<CW>(part + static_cast<int64_t>(g) * W2 + col, t);
+#pragma unroll
+      for (int i = 0; i < CW; ++i) acc[i] += t[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CW; ++i) buf[cy][cx][i] = acc[i];
+  __syncthreads();
+  if (cy == 0 && col < W2) {
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      float s = buf[0][cx][i];
+      for (int k = 1; k < CY; ++k) s += buf[k][cx][i];
+      acc[i] = s;
+    }
+    // CW divides W on the vector path, so a column group never straddles the two halves
+#pragma unroll
+    for (int i = 0; i < CW; ++i) {
+      const int j = col + i;
+      if (j < W) {
+        out0[j] = acc[i];
+      } else {
+        out1[j - W] = acc[i];
+      }
+    }
+  }
+}
+
+// ------------------------------------------------------------------------ split rows
+// A row of D elements is cut into S chunks of `chunk` elements (the last may be short).
+// Work item w = row * S + s; blocks take work items grid-stride.  V = elements per
+// access (16-byte vectors when everything is aligned, 1 otherwise).
+
+template <typename T, int V>
+__device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
+  // Streaming Welford: one vector at a time, exact two-pass inside the vector and a
+  // Chan merge into the running triple.
+  Wf run{0.f, 0.f, 0.f};
+  for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
+       i += static_cast<int64_t>(blockDim.x) * V) {
+    Pack<T, V> pk = load_pack<T, V>(p + i);
+    float f[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) f[k] = to_f32(pk.v[k]);
+    if constexpr (V == 1) {
+      // classic Welford update
+      run.n += 1.f;
+      const float d = f[0] - run.mean;
+      run.mean += d / run.n;
+      run.m2 += d * (f[0] - run.mean);
+    } else {
+      Wf w = local_wf<V>(f, V);
+      run = wf_merge(run, w);
+    }
+  }
+  return run;
+}
+
+// stage 1 forward: stats[w] = (mean, m2) of chunk w; the count follows from geometry.
+template <typename T, int V>
+__global__ void split_fwd_stats(const T* __restrict__ x, float2* __restrict__ stats,
+                                int64_t n_rows, int64_t D, int S, int64_t chunk) {
+  __shared__ Wf wf_buf[2][16];
+  const int64_t n_work = n_rows * S;
+  int it = 0;
+  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x, ++it) {
+    const int64_t row = w / S;
+    const int s = static_cast<int>(w % S);
+    const int64_t beg = static_cast<int64_t>(s) * chunk;
+    const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    Wf r = chunk_wf<T, V>(x + row * D + beg, len);
+    r = block_wf(r, wf_buf[it & 1]);
+    if (threadIdx.x == 0) stats[w] = make_float2(r.mean, r.m2);
+  }
+}
+
+__device__ __forceinline__ Wf merge_chunks(const float2* stats, int S, int64_t D, int64_t chunk) {
+  Wf r{0.f, 0.f, 0.f};
+  for (int s = 0; s < S; ++s) {
+    const int64_t beg = static_cast<int64_t>(s) * chunk;
+    const float2 t = stats[s];
+    Wf o{t.x, t.y, static_cast<float>(beg + chunk <= D ? chunk : D - beg)};
+    r = wf_merge(r, o);
+  }
+  return r;
+}
+
+// stage 2 forward: merge the S chunk statistics of the row, normalise the chunk.
+// y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
+// every thread reads a vector before it writes the same vector.
+template <typename T, int V, bool ROW_AFFINE>
+__global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
+                                const float* __restrict__ gamma, const float* __restrict__ beta,
+                                T* y, float* __restrict__ mean_out,
+                                float* __restrict__ rstd_out, int64_t n_rows, int64_t D, int S,
+                                int64_t chunk, int C, float eps) {
+  const int64_t n_work = n_rows * S;
+  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
+    const int64_t row = w / S;
+    const int s = static_cast<int>(w % S);
+    const Wf r = merge_chunks(stats + row * S, S, D, chunk);
+    const float mean = r.mean;
+    const float rstd = rsqrtf(r.m2 / static_cast<float>(D) + eps);
+    if (s == 0 && threadIdx.x == 0) {
+      mean_out[row] = mean;
+      rstd_out[row] = rstd;
+    }
+    float gs = 1.f, bs = 0.f;
+    if constexpr (ROW_AFFINE) {
+      const int c = static_cast<int>(row % C);
+      gs = gamma[c];
+      bs = beta[c];
+    }
+    const int64_t beg = static_cast<int64_t>(s) * chunk;
+    const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const T* xp = x + row * D + beg;
+    T* yp = y + row * D + beg;
+    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
+         i += static_cast<int64_t>(blockDim.x) * V) {
+      Pack<T, V> pk = load_pack<T, V>(xp + i);
+      Pack<T, V> o;
+      float tg[V], tb[V];
+      if constexpr (!ROW_AFFINE) {
+        load_f32<V>(gamma + beg + i, tg);
+        load_f32<V>(beta + beg + i, tb);
+      }
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float xh = (to_f32(pk.v[k]) - mean) * rstd;
+        if constexpr (ROW_AFFINE) {
+          o.v[k] = from_f32<T>(xh * gs + bs);
+        } else {
+          o.v[k] = from_f32<T>(xh * tg[k] + tb[k]);
+        }
+      }
+      store_pack<T, V>(yp + i, o);
+    }
+  }
+}
+
+// stage 1 backward: sums[w] = (sum g, sum g * xh) over chunk w, g = dy * gamma
+// (ROW_AFFINE: (sum dy, sum dy * xh), gamma applied in stage 2).
+template <typename T, int V, bool ROW_AFFINE>
+__global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
+                               const float* __restrict__ gamma,
+                               const float* __restrict__ mean_in,
+                               const float* __restrict__ rstd_in, float2* __restrict__ sums,
+                               int64_t n_rows, int64_t D, int S, int64_t chunk) {
+  __shared__ float2 sum_buf[2][16];
+  const int64_t n_work = n_rows * S;
+  int it = 0;
+  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x, ++it) {
+    const int64_t row = w / S;
+    const int s = static_cast<int>(w % S);
+    const int64_t beg = static_cast<int64_t>(s) * chunk;
+    const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    const T* xp = x + row * D + beg;
+    const T* dp = dy + row * D + beg;
+    float s1 = 0.f, s2 = 0.f;
+    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
+         i += static_cast<int64_t>(blockDim.x) * V) {
+      Pack<T, V> px = load_pack<T, V>(xp + i);
+      Pack<T, V> pd = load_pack<T, V>(dp + i);
+      float tg[V];
+      if constexpr (!ROW_AFFINE) load_f32<V>(gamma + beg + i, tg);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float xh = (to_f32(px.v[k]) - mean) * rstd;
+        float gv = to_f32(pd.v[k]);
+        if constexpr (!ROW_AFFINE) gv *= tg[k];
+        s1 += gv;
+        s2 += gv * xh;
+      }
+    }
+    const float2 r = block_sum2(s1, s2, sum_buf[it & 1]);
+    if (threadIdx.x == 0) sums[w] = r;
+  }
+}
+
+// stage 2 backward: merge the row's chunk sums, write dx for the chunk.  ROW_AFFINE also
+// writes the per-(n, c) sums into `part` (layout as in rows_bwd_resident).
+template <typename T, int V, bool ROW_AFFINE>
+__global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x,
+                                const float* __restrict__ gamma,
+                                const float* __restrict__ mean_in,
+                                const float* __restrict__ rstd_in,
+                                const float2* __restrict__ sums, T* __restrict__ dx,
+                                float* __restrict__ part, int64_t n_rows, int64_t D, int S,
+                                int64_t chunk, int C) {
+  const int64_t n_work = n_rows * S;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
+    const int64_t row = w / S;
+    const int s = static_cast<int>(w % S);
+    float s1 = 0.f, s2 = 0.f;
+    for (int k = 0; k < S; ++k) {
+      const float2 t = sums[row * S + k];
+      s1 += t.x;
+      s2 += t.y;
+    }
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    float gs = 1.f;
+    if constexpr (ROW_AFFINE) {
+      const int64_t n = row / C;
+      const int c = static_cast<int>(row % C);
+      gs = gamma[c];
+      if (s == 0 && threadIdx.x == 0) {
+        part[(n * 2 + 0) * C + c] = s2;
+        part[(n * 2 + 1) * C + c] = s1;
+      }
+    }
+    const int64_t beg = static_cast<int64_t>(s) * chunk;
+    const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const T* xp = x + row * D + beg;
+    const T* dp = dy + row * D + beg;
+    T* op = dx + row * D + beg;
+    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
+         i += static_cast<int64_t>(blockDim.x) * V) {
+      Pack<T, V> px = load_pack<T, V>(xp + i);
+      Pack<T, V> pd = load_pack<T, V>(dp + i);
+      Pack<T, V> o;
+      float tg[V];
+      if constexpr (!ROW_AFFINE) load_f32<V>(gamma + beg + i, tg);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float xh = (to_f32(px.v[k]) - mean) * rstd;
+        float gv = to_f32(pd.v[k]);
+        if constexpr (!ROW_AFFINE) gv *= tg[k];
+        o.v[k] = from_f32<T>(rstd * gs * (gv - (s1 + xh * s2) * inv_d));
+      }
+      store_pack<T, V>(op + i, o);
+    }
+  }
+}
+
+// LayerNorm dgamma / dbeta when rows are not register-resident: thread <-> column,
+// block (x = column tile of blockDim.x, y = slab of rows); writes
+// part[slab][0][col], part[slab][1][col]; col_reduce finishes.
+// (reference equivalent: fused_layer_norm_op.cu:763-783)
+template <typename T>
+__global__ void ln_colgrad_partial(const T* __restrict__ dy, const T* __restrict__ x,
+                                   const float* __restrict__ mean_in,
+                                   const float* __restrict__ rstd_in, float* __restrict__ part,
+                                   int64_t n_rows, int64_t D, int64_t rows_per_slab) {
+  const int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
+  const int64_t slab = blockIdx.y;
+  const int64_t r0 = slab * rows_per_slab;
+  const int64_t r1 = (r0 + rows_per_slab < n_rows) ? r0 + rows_per_slab : n_rows;
+  if (col >= D) return;
+  float ag = 0.f, ab = 0.f;
+  for (int64_t r = r0; r < r1; ++r) {
+    const float d = to_f32(dy[r * D + col]);
+    const float xh = (to_f32(x[r * D + col]) - mean_in[r]) * rstd_in[r];
+    ag += d * xh;
+    ab += d;
+  }
+  part[(slab * 2 + 0) * D + col] = ag;
+  part[(slab * 2 + 1) * D + col] = ab;
+}
+
+}  // namespace atexn

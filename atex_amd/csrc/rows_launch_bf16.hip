@@ -1,0 +1,6 @@
+// Contiguous-row kernels instantiated for one storage type.
+#include "rows_launch_impl.cuh"
+
+namespace atexn {
+ATEXN_INSTANTIATE_ROWS(bf16_t)
+}  // namespace atexn

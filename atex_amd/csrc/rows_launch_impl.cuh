@@ -1,0 +1,150 @@
+// Launchers for the contiguous-row kernels, templated on the storage type; one
+// translation unit per dtype instantiates them (rows_launch_*.hip).
+#pragma once
+
+#include "plan.h"
+#include "rows_kernels.cuh"
+#include "status.h"
+
+namespace atexn {
+
+template <typename T, int V, bool AFF>
+using FwdResidentFn = void (*)(const T*, const float*, const float*, T*, float*, float*, int64_t,
+                               int, int, float);
+template <typename T, int V, bool AFF>
+using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, const float*, T*,
+                               float*, int64_t, int, int);
+
+template <typename T, int V, bool AFF>
+FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt) {
+  if (tpr == 8) return rows_fwd_resident<T, V, 8, 1, AFF>;
+  if (tpr == 16) return rows_fwd_resident<T, V, 16, 1, AFF>;
+  if (tpr == 32) return rows_fwd_resident<T, V, 32, 1, AFF>;
+  if (tpr == 64 && vpt == 1) return rows_fwd_resident<T, V, 64, 1, AFF>;
+  if (tpr == 64 && vpt == 2) return rows_fwd_resident<T, V, 64, 2, AFF>;
+  if (tpr == 0 && vpt == 2) return rows_fwd_resident<T, V, 0, 2, AFF>;
+  if (tpr == 0 && vpt == 4) return rows_fwd_resident<T, V, 0, 4, AFF>;
+  if (tpr == 0 && vpt == 8) return rows_fwd_resident<T, V, 0, 8, AFF>;
+  return nullptr;
+}
+
+template <typename T, int V, bool AFF>
+BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt) {
+  if (tpr == 8) return rows_bwd_resident<T, V, 8, 1, AFF>;
+  if (tpr == 16) return rows_bwd_resident<T, V, 16, 1, AFF>;
+  if (tpr == 32) return rows_bwd_resident<T, V, 32, 1, AFF>;
+  if (tpr == 64 && vpt == 1) return rows_bwd_resident<T, V, 64, 1, AFF>;
+  if (tpr == 64 && vpt == 2) return rows_bwd_resident<T, V, 64, 2, AFF>;
+  if (tpr == 0 && vpt == 2) return rows_bwd_resident<T, V, 0, 2, AFF>;
+  if (tpr == 0 && vpt == 4) return rows_bwd_resident<T, V, 0, 4, AFF>;
+  if constexpr (AFF) {
+    if (tpr == 0 && vpt == 8) return rows_bwd_resident<T, V, 0, 8, AFF>;
+  }
+  return nullptr;
+}
+
+template <typename T, int V, bool AFF>
+int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
+               int C, float eps, T* y, float* mean, float* rstd, void* ws, size_t ws_bytes,
+               hipStream_t st) {
+  const RowsPlan p = plan_rows(RowsKind::kFwd, V, n_rows, D, C, cu_count());
+  ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && (p.ws_bytes == 0 || ws != nullptr),
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  if (p.resident) {
+    auto fn = pick_fwd_resident<T, V, AFF>(p.tpr, p.vpt);
+    if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident forward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
+    fn<<<p.grid, p.threads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows,
+                                     static_cast<int>(D / V), C, eps);
+    ATEXN_CHECK_LAUNCH("rows_fwd_resident");
+    return ATEXN_OK;
+  }
+  float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
+  split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
+  ATEXN_CHECK_LAUNCH("split_fwd_stats");
+  split_fwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
+                                                          n_rows, D, p.S, p.chunk, C, eps);
+  ATEXN_CHECK_LAUNCH("split_fwd_apply");
+  return ATEXN_OK;
+}
+
+template <typename T, int V, bool AFF>
+int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, const float* rstd,
+               int64_t n_rows, int64_t D, int C, T* dx, float* dgamma, float* dbeta, void* ws,
+               size_t ws_bytes, hipStream_t st) {
+  const RowsPlan p =
+      plan_rows(AFF ? RowsKind::kBwdAffine : RowsKind::kBwdCols, V, n_rows, D, C, cu_count());
+  ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_part);
+  const int64_t W = AFF ? C : D;
+  if (p.resident) {
+    auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt);
+    if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
+    const int stages = tuning().bwd_stage_mask;
+    if (stages & 1) {
+      fn<<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
+                                                static_cast<int>(D / V), C);
+      ATEXN_CHECK_LAUNCH("rows_bwd_resident");
+    }
+    if (!(stages & 2)) return ATEXN_OK;
+    return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+  }
+  float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
+  split_bwd_sums<T, V, AFF><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
+                                                         D, p.S, p.chunk);
+  ATEXN_CHECK_LAUNCH("split_bwd_sums");
+  split_bwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
+                                                          part, n_rows, D, p.S, p.chunk, C);
+  ATEXN_CHECK_LAUNCH("split_bwd_apply");
+  if constexpr (!AFF) {
+    dim3 grid(p.col_tiles, p.col_slabs);
+    ln_colgrad_partial<T><<<grid, 256, 0, st>>>(dy, x, mean, rstd, part, n_rows, D,
+                                                 p.rows_per_slab);
+    ATEXN_CHECK_LAUNCH("ln_colgrad_partial");
+  }
+  return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+}
+
+template <typename T>
+int rows_fwd_t(bool affine, const void* x_, const float* gamma, const float* beta, int64_t n_rows,
+               int64_t D, int C, float eps, void* y_, float* mean, float* rstd, void* ws,
+               size_t ws_bytes, hipStream_t st) {
+  constexpr int VEC = VecOf<T>::value;
+  const T* x = static_cast<const T*>(x_);
+  T* y = static_cast<T*>(y_);
+  const bool vec = (D % VEC == 0) && aligned16(x) && aligned16(y) &&
+                   (affine || (aligned16(gamma) && aligned16(beta)));
+  if (vec) {
+    return affine ? rows_fwd_v<T, VEC, true>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st)
+                  : rows_fwd_v<T, VEC, false>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st);
+  }
+  return affine ? rows_fwd_v<T, 1, true>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st)
+                : rows_fwd_v<T, 1, false>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st);
+}
+
+template <typename T>
+int rows_bwd_t(bool affine, const void* dy_, const void* x_, const float* gamma, const float* mean,
+               const float* rstd, int64_t n_rows, int64_t D, int C, void* dx_, float* dgamma,
+               float* dbeta, void* ws, size_t ws_bytes, hipStream_t st) {
+  constexpr int VEC = VecOf<T>::value;
+  const T* x = static_cast<const T*>(x_);
+  const T* dy = static_cast<const T*>(dy_);
+  T* dx = static_cast<T*>(dx_);
+  const bool vec = (D % VEC == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
+                   aligned16(ws) && (affine || aligned16(gamma));
+  if (vec) {
+    return affine ? rows_bwd_v<T, VEC, true>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st)
+                  : rows_bwd_v<T, VEC, false>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st);
+  }
+  return affine ? rows_bwd_v<T, 1, true>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st)
+                : rows_bwd_v<T, 1, false>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st);
+}
+
+#define ATEXN_INSTANTIATE_ROWS(T)                                                              \
+  template int rows_fwd_t<T>(bool, const void*, const float*, const float*, int64_t, int64_t,  \
+                             int, float, void*, float*, float*, void*, size_t, hipStream_t);   \
+  template int rows_bwd_t<T>(bool, const void*, const void*, const float*, const float*,       \
+                             const float*, int64_t, int64_t, int, void*, float*, float*, void*, \
+                             size_t, hipStream_t);
+
+}  // namespace atexn

@@ -1,0 +1,321 @@
+#!/usr/bin/env python3
+"""Benchmark of the fused LayerNorm / InstanceNorm forward + backward on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case NAME] [--no-cpu]
+
+One "step" is one forward plus one backward call of the hot path (kernel-level C ABI of
+libatex_norms_hip.so) over one batch of synthetic input that is already resident in HBM.
+The default case is the LayerNorm BERT-large token shape, x fp16 [8192, 1024].
+
+Cache honesty: the 16.8 MB tensors of that case would sit in the 256 MB Infinity Cache if
+every step reused them, so the timed loop rotates over enough independent buffer sets
+(x, dy, y, dx, statistics) that a set's lines were last touched more than 512 MB ago.
+
+Output: ONE JSON line on stdout.
+  value        algorithmic bytes of fwd + bwd / wall time per step, in GB/s
+  roofline     the dominant kernel (the backward row kernel), timed alone with events on the
+               launch stream: algorithmic bytes of the backward / its average duration,
+               against the 8 TB/s HBM peak
+  cpu_baseline the C oracle's float flavour (OpenMP over rows) on the same workload, timed
+               on this machine's host cores
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+ROTATE_BYTES = 640 << 20  # footprint the buffer rotation must exceed
+
+# name -> (op, dtype, dims); LayerNorm dims = (N, D); InstanceNorm dims = (N, C, D, channel_first)
+CASES = {
+    "ln_cfg0": ("ln", "f32", (32, 1024)),
+    "ln_bert": ("ln", "f16", (8192, 1024)),
+    "ln_128_f16": ("ln", "f16", (262144, 128)),
+    "ln_128_bf16": ("ln", "bf16", (262144, 128)),
+    "ln_4096_f16": ("ln", "f16", (16384, 4096)),
+    "ln_4096_bf16": ("ln", "bf16", (16384, 4096)),
+    "ln_12288_f16": ("ln", "f16", (2048, 12288)),
+    "ln_12288_bf16": ("ln", "bf16", (2048, 12288)),
+    "in2d_nhwc": ("in", "f16", (8, 64, 128 * 128, False)),
+    "in2d_nchw": ("in", "f16", (8, 64, 128 * 128, True)),
+    "in3d_ndhwc": ("in", "f16", (2, 32, 128 ** 3, False)),
+    "in3d_ncdhw": ("in", "f16", (2, 32, 128 ** 3, True)),
+}
+DEFAULT_CASE = "ln_bert"
+ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
+
+
+def algorithmic_bytes(op, dtype, dims):
+    """(fwd, bwd) bytes every implementation must move: x in, y out, the fp32 parameters and
+    statistics; dy and x in, dx out, statistics in, dgamma / dbeta out."""
+    s = ESIZE[dtype]
+    if op == "ln":
+        N, D = dims
+        return 2 * N * D * s + 8 * D + 8 * N, 3 * N * D * s + 12 * D + 8 * N
+    N, C, D, _ = dims
+    return 2 * N * C * D * s + 8 * C + 8 * N * C, 3 * N * C * D * s + 12 * C + 8 * N * C
+
+
+def _storage(a, dtype):
+    from oracle import oracle as O
+
+    return O.to_storage(a, dtype)
+
+
+def make_host_inputs(op, dtype, dims, seed):
+    rng = np.random.Generator(np.random.PCG64(seed))
+    if op == "ln":
+        N, D = dims
+        x = rng.standard_normal((N, D), dtype=np.float32)
+        x += rng.uniform(-2, 2, size=(N, 1)).astype(np.float32)
+        dy = rng.standard_normal((N, D), dtype=np.float32)
+        P = D
+    else:
+        N, C, D, cf = dims
+        shape = (N, C, D) if cf else (N, D, C)
+        x = rng.standard_normal(shape, dtype=np.float32)
+        dy = rng.standard_normal(shape, dtype=np.float32)
+        P = C
+    gamma = rng.uniform(0.5, 1.5, size=P).astype(np.float32)
+    beta = (rng.standard_normal(P) * 0.1).astype(np.float32)
+    return x, gamma, beta, dy
+
+
+class GpuCase:
+    """Device buffers of one case, R rotating sets, and closures that launch fwd / bwd."""
+
+    def __init__(self, op, dtype, dims, device="cuda:0"):
+        import torch
+
+        from atex_amd.nv_norms import _capi
+
+        self.torch = torch
+        self.capi = _capi
+        self.L = _capi.lib()
+        self.op, self.dtype, self.dims = op, dtype, dims
+        self.code = {"f32": 0, "f16": 1, "bf16": 2}[dtype]
+        tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+        if op == "ln":
+            N, D = dims
+            shape, stat_shape, P = (N, D), (N,), D
+            self.fwd_ws = self.L.atexn_layer_norm_fwd_workspace_bytes(self.code, N, D)
+            self.bwd_ws = self.L.atexn_layer_norm_bwd_workspace_bytes(self.code, N, D)
+        else:
+            N, C, D, cf = dims
+            shape, stat_shape, P = ((N, C, D) if cf else (N, D, C)), (N, C), C
+            self.layout = 0 if cf else 1
+            self.fwd_ws = self.L.atexn_instance_norm_fwd_workspace_bytes(self.code, self.layout, N, C, D)
+            self.bwd_ws = self.L.atexn_instance_norm_bwd_workspace_bytes(self.code, self.layout, N, C, D)
+        n_elem = int(np.prod(shape))
+        set_bytes = 4 * n_elem * ESIZE[dtype]
+        self.n_sets = max(2, min(64, -(-ROTATE_BYTES // set_bytes)))
+        g = torch.Generator(device=device)
+        g.manual_seed(1234)
+        self.sets = []
+        for _ in range(self.n_sets):
+            x = (torch.randn(shape, device=device, dtype=torch.float32, generator=g)).to(tdt)
+            dy = torch.randn(shape, device=device, dtype=torch.float32, generator=g).to(tdt)
+            self.sets.append(dict(
+                x=x, dy=dy, y=torch.empty_like(x), dx=torch.empty_like(x),
+                mean=torch.empty(stat_shape, device=device, dtype=torch.float32),
+                rstd=torch.empty(stat_shape, device=device, dtype=torch.float32)))
+        self.gamma = torch.rand(P, device=device, dtype=torch.float32, generator=g) + 0.5
+        self.beta = torch.randn(P, device=device, dtype=torch.float32, generator=g) * 0.1
+        self.dgamma = torch.empty(P, device=device, dtype=torch.float32)
+        self.dbeta = torch.empty(P, device=device, dtype=torch.float32)
+        wsb = max(self.fwd_ws, self.bwd_ws, 256)
+        self.ws = torch.empty(wsb, device=device, dtype=torch.uint8)
+        self.stream = torch.cuda.current_stream(device).cuda_stream
+
+    def fwd(self, i):
+        s = self.sets[i % self.n_sets]
+        L, c = self.L, self.code
+        if self.op == "ln":
+            N, D = self.dims
+            st = L.atexn_layer_norm_fwd(c, s["x"].data_ptr(), self.gamma.data_ptr(), self.beta.data_ptr(), N, D,
+                                        1e-3, s["y"].data_ptr(), s["mean"].data_ptr(), s["rstd"].data_ptr(),
+                                        self.ws.data_ptr(), self.ws.numel(), self.stream)
+        else:
+            N, C, D, _ = self.dims
+            st = L.atexn_instance_norm_fwd(c, self.layout, s["x"].data_ptr(), self.gamma.data_ptr(),
+                                           self.beta.data_ptr(), N, C, D, 1e-3, s["y"].data_ptr(),
+                                           s["mean"].data_ptr(), s["rstd"].data_ptr(), self.ws.data_ptr(),
+                                           self.ws.numel(), self.stream)
+        if st != 0:
+            self.capi.check(st)
+
+    def bwd(self, i):
+        s = self.sets[i % self.n_sets]
+        L, c = self.L, self.code
+        if self.op == "ln":
+            N, D = self.dims
+            st = L.atexn_layer_norm_bwd(c, s["dy"].data_ptr(), s["x"].data_ptr(), self.gamma.data_ptr(),
+                                        s["mean"].data_ptr(), s["rstd"].data_ptr(), N, D, s["dx"].data_ptr(),
+                                        self.dgamma.data_ptr(), self.dbeta.data_ptr(), self.ws.data_ptr(),
+                                        self.ws.numel(), self.stream)
+        else:
+            N, C, D, _ = self.dims
+            st = L.atexn_instance_norm_bwd(c, self.layout, s["dy"].data_ptr(), s["x"].data_ptr(),
+                                           self.gamma.data_ptr(), s["mean"].data_ptr(), s["rstd"].data_ptr(),
+                                           N, C, D, s["dx"].data_ptr(), self.dgamma.data_ptr(),
+                                           self.dbeta.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream)
+        if st != 0:
+            self.capi.check(st)
+
+    def time_loop(self, fn, steps, warmup):
+        """Average milliseconds per call of fn(i), events on the launch stream."""
+        torch = self.torch
+        for i in range(warmup):
+            fn(i)
+        torch.cuda.synchronize()
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        for i in range(steps):
+            fn(warmup + i)
+        e1.record()
+        torch.cuda.synchronize()
+        return e0.elapsed_time(e1) / steps
+
+
+def cpu_baseline(op, dtype, dims, max_seconds=20.0):
+    """The oracle's float flavour on the same workload (full size when it fits the time
+    bound, else the leading rows / instances), OpenMP threads = host cores in use."""
+    from oracle import oracle as O
+
+    O.build()
+    co = O.COracle()
+    threads = min(16, os.cpu_count() or 1)
+    co.set_num_threads(threads)
+    sample = "full workload"
+    d = list(dims)
+    if op == "in" and d[2] * d[1] * d[0] > 32 * 1024 * 1024:
+        d[0] = 1
+        sample = f"first instance only (N=1 of {dims[0]})"
+    d = tuple(d)
+    x, gamma, beta, dy = make_host_inputs(op, dtype, d, 1001)
+    xs, dys = _storage(x, dtype), _storage(dy, dtype)
+
+    def step():
+        if op == "ln":
+            y, m, r = co.ln_fwd(xs, gamma, beta, 1e-3, dtype, f64=False)
+            co.ln_bwd(dys, xs, gamma, m, r, dtype, f64=False)
+        else:
+            cf = d[3]
+            y, m, r = co.in_fwd(xs, gamma, beta, 1e-3, dtype, cf, f64=False)
+            co.in_bwd(dys, xs, gamma, m, r, dtype, cf, f64=False)
+
+    step()
+    times = []
+    t_end = time.perf_counter() + max_seconds
+    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 2):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    fb, bb = algorithmic_bytes(op, dtype, d)
+    return {
+        "value": (fb + bb) / med / 1e9,
+        "unit": "GB/s",
+        "cores": threads,
+        "kind": "port",
+        "sample": f"{sample}; median of {len(times)} steps, {med * 1e6:.0f} us/step",
+        "us_per_step": med * 1e6,
+    }
+
+
+def run_case(name, steps, warmup, with_cpu=True):
+    op, dtype, dims = CASES[name]
+    fb, bb = algorithmic_bytes(op, dtype, dims)
+    case = GpuCase(op, dtype, dims)
+    L = case.L
+
+    def step(i):
+        case.fwd(i)
+        case.bwd(i)
+
+    ms_step = case.time_loop(step, steps, warmup)
+    ms_fwd = case.time_loop(case.fwd, steps, warmup)
+    ms_bwd = case.time_loop(case.bwd, steps, warmup)
+    # the dominant kernel alone: backward without its final column reduction
+    L.atexn_set_tuning(b"bwd_stage_mask", 1)
+    ms_bwd_main = case.time_loop(case.bwd, steps, warmup)
+    L.atexn_set_tuning(b"bwd_stage_mask", 3)
+    # hot-cache figure (one buffer set reused), labelled as such
+    n_sets = case.n_sets
+    case.n_sets = 1
+    ms_step_hot = case.time_loop(step, steps, warmup)
+    case.n_sets = n_sets
+
+    value = (fb + bb) / (ms_step * 1e-3) / 1e9
+    achieved = bb / (ms_bwd_main * 1e-3) / 1e9
+    if op == "ln":
+        workload = f"LayerNorm fwd+bwd x {dtype} [{dims[0]},{dims[1]}] axis=-1 eps=1e-3, gamma/beta fp32"
+    else:
+        N, C, D, cf = dims
+        workload = (f"InstanceNorm fwd+bwd x {dtype} N={N} C={C} spatial={D} "
+                    f"{'channel-first' if cf else 'channels-last'} eps=1e-3")
+    out = {
+        "metric": "LN/IN fwd+bwd achieved HBM GB/s",
+        "value": value,
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": steps,
+        "warmup": warmup,
+        "ms_per_step": ms_step,
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": dtype,
+        "data": "synthetic",
+        "config": {"workload": workload, "case": name, "rotating_buffer_sets": n_sets,
+                   "algorithmic_bytes_fwd": fb, "algorithmic_bytes_bwd": bb},
+        "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "us_per_call": {"fwd": ms_fwd * 1e3, "bwd": ms_bwd * 1e3, "fwd_bwd": ms_step * 1e3,
+                        "fwd_bwd_hot_cache": ms_step_hot * 1e3},
+        "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9,
+                 "fwd_bwd_hot_cache": (fb + bb) / (ms_step_hot * 1e-3) / 1e9},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
+                     "kernel": "backward row kernel (dx + dgamma/dbeta partials)",
+                     "us": ms_bwd_main * 1e3},
+    }
+    if with_cpu:
+        out["cpu_baseline"] = cpu_baseline(op, dtype, dims)
+    return out
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--case", default=DEFAULT_CASE, choices=sorted(CASES) + ["all"])
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: the path has no cross-GPU exchange; run with --gpus 1")
+    import torch
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
+    if args.case == "all":
+        for name in CASES:
+            steps = args.steps if "3d" not in name else max(10, args.steps // 10)
+            r = run_case(name, steps, args.warmup, with_cpu=False)
+            print(json.dumps(r), flush=True)
+        return
+    print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu)), flush=True)
+
+
+if __name__ == "__main__":
+    main()

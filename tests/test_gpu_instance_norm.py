@@ -1,0 +1,144 @@
+"""GPU parity of the InstanceNorm entry points (through the C ABI) against the CPU oracle.
+
+Shapes: benchmark configurations 3 and 4 (the latter with the spatial extent cut so the
+oracle finishes in seconds) and the shape lists of the reference's own test
+(tests/fused_instance_norm_test.py:145-170): N=2, C=32, rank 4 / 5 with 2^3..2^6 per
+spatial dim, both layouts, plus the non-typical spatial extents.
+"""
+import numpy as np
+import pytest
+
+from tests import util
+from tests.util import TOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+EPS = 1e-3
+
+
+@pytest.fixture(scope="module")
+def capi():
+    return util.Capi()
+
+
+def run_case(capi, coracle, N, C, S, dtype, channel_first, seed_index, stddev=1.0, in_place=False):
+    import torch
+
+    print(f"IN case N={N} C={C} spatial={S} dtype={dtype} channel_first={channel_first} "
+          f"seed={1000 + seed_index} in_place={in_place}", flush=True)
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, channel_first, seed_index, stddev)
+    y_ref, mean_ref, rstd_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, channel_first)
+
+    xd = util.to_device(x, dtype)
+    gd = torch.from_numpy(gamma).cuda()
+    bd = torch.from_numpy(beta).cuda()
+    x_keep = xd.clone() if in_place else xd
+    y, mean, rstd = capi.in_fwd(xd, gd, bd, EPS, dtype, channel_first, y=xd if in_place else None)
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert_close(util.to_host(mean), mean_ref, tol["stat"], "mean")
+    assert_close(util.to_host(rstd), rstd_ref, tol["stat"], "inv_std")
+    assert_close(util.to_host(y), y_ref, tol["y"], "y")
+
+    mean32 = mean_ref.astype(np.float32)
+    rstd32 = rstd_ref.astype(np.float32)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, mean32.astype(np.float64),
+                                            rstd32.astype(np.float64), dtype, channel_first)
+    dx, dg, db = capi.in_bwd(util.to_device(dy, dtype), x_keep, gd, torch.from_numpy(mean32).cuda(),
+                             torch.from_numpy(rstd32).cuda(), dtype, channel_first)
+    torch.cuda.synchronize()
+    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx")
+    assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+    assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("dtype", ["f16", "f32", "bf16"])
+def test_config3_2d(capi, coracle, dtype, channel_first):
+    run_case(capi, coracle, 8, 64, 128 * 128, dtype, channel_first, 3)
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+def test_config4_3d_reduced(capi, coracle, channel_first):
+    # [2,128,128,128,32] with the depth cut to 16: still a multi-workgroup reduction per (n,c)
+    run_case(capi, coracle, 2, 32, 16 * 128 * 128, "f16", channel_first, 4)
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("rank,d_exp", [(4, 3), (4, 4), (4, 5), (4, 6), (5, 3), (5, 4), (5, 5), (5, 6)])
+def test_reference_shapes(capi, coracle, rank, d_exp, dtype, channel_first):
+    # fused_instance_norm_test.py:145-155; x ~ N(0, 10^2) as there
+    spatial = (2 ** d_exp) ** (rank - 2)
+    run_case(capi, coracle, 2, 32, spatial, dtype, channel_first, 20, stddev=10.0)
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("spatial", [1 * 11, 3 * 4, 1 * 31, 1 * 4001, 61 * 82, 113 * 145, 198 * 331, 179 * 2929])
+def test_non_typical_spatial(capi, coracle, spatial, channel_first):
+    # fused_instance_norm_test.py:157-179 (N=1, C=32, fp32)
+    run_case(capi, coracle, 1, 32, spatial, "f32", channel_first, 21, stddev=10.0)
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("C", [1, 3, 5, 24, 48, 100, 256, 520])
+def test_channel_counts(capi, coracle, C, dtype, channel_first):
+    # channel counts that are not a multiple of the vector width or not a power of two
+    run_case(capi, coracle, 3, C, 777, dtype, channel_first, 22)
+
+
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_in_place(capi, coracle, dtype, channel_first):
+    run_case(capi, coracle, 2, 32, 4096, dtype, channel_first, 23, in_place=True)
+    run_case(capi, coracle, 1, 8, 300000, dtype, channel_first, 23, in_place=True)
+
+
+def test_layout_equivalence(capi):
+    """IN over NC... of the transposed tensor equals the transpose of IN over N...C."""
+    import torch
+
+    x, gamma, beta, dy = util.in_inputs(2, 16, 1000, "f32", False, 24)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    x_cl = torch.from_numpy(x).cuda()
+    x_cf = x_cl.permute(0, 2, 1).contiguous()
+    y_cl, m_cl, r_cl = capi.in_fwd(x_cl, gd, bd, EPS, "f32", False)
+    y_cf, m_cf, r_cf = capi.in_fwd(x_cf, gd, bd, EPS, "f32", True)
+    torch.cuda.synchronize()
+    assert_close(util.to_host(y_cf.permute(0, 2, 1).contiguous()), util.to_host(y_cl), 1e-5, "y")
+    assert_close(util.to_host(m_cf), util.to_host(m_cl), 1e-5, "mean")
+    assert_close(util.to_host(r_cf), util.to_host(r_cl), 1e-5, "inv_std")
+
+
+def test_empty(capi):
+    import torch
+
+    L = capi.L
+    dg = torch.full((4,), 7.0, device="cuda")
+    db = torch.full((4,), 7.0, device="cuda")
+    for layout in (0, 1):
+        assert L.atexn_instance_norm_fwd(0, layout, None, None, None, 0, 4, 9, 1e-3, None, None, None, None, 0, None) == 0
+        dg.fill_(7.0)
+        db.fill_(7.0)
+        assert L.atexn_instance_norm_bwd(0, layout, None, None, None, None, None, 0, 4, 9, None,
+                                         dg.data_ptr(), db.data_ptr(), None, 0, None) == 0
+        torch.cuda.synchronize()
+        assert float(dg.abs().sum()) == 0.0 and float(db.abs().sum()) == 0.0
+
+
+def test_deterministic(capi):
+    import torch
+
+    for cf in (False, True):
+        x, gamma, beta, dy = util.in_inputs(4, 64, 4096, "f16", cf, 25)
+        xd, dyd = util.to_device(x, "f16"), util.to_device(dy, "f16")
+        gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+        outs = []
+        for _ in range(2):
+            y, m, r = capi.in_fwd(xd, gd, bd, EPS, "f16", cf)
+            dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, "f16", cf)
+            torch.cuda.synchronize()
+            outs.append([t.clone() for t in (y, m, r, dx, dg, db)])
+        for a, b in zip(*outs):
+            assert torch.equal(a, b)
