@@ -47,7 +47,8 @@ def run_case(capi, coracle, N, C, S, dtype, channel_first, seed_index, stddev=1.
     dx, dg, db = capi.in_bwd(util.to_device(dy, dtype), x_keep, gd, torch.from_numpy(mean32).cuda(),
                              torch.from_numpy(rstd32).cuda(), dtype, channel_first)
     torch.cuda.synchronize()
-    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx")
+    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx",
+                 scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), rstd32, dtype))
     assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
     assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
 

@@ -18,20 +18,29 @@ TOL = {
 }
 
 
-def assert_close(got, ref, rtol, what=""):
+def assert_close(got, ref, rtol, what="", scale=0.0):
+    """`scale`: magnitude of the terms the result is a difference of, when that is larger
+    than the result itself (dx is r*g minus its projections; for a one-element row the
+    exact answer is 0 and only rounding residue is left)."""
     got = np.asarray(got, dtype=np.float64)
     ref = np.asarray(ref, dtype=np.float64)
     assert got.shape == ref.shape, (what, got.shape, ref.shape)
     if ref.size == 0:
         return
     assert np.all(np.isfinite(got)), f"{what}: non-finite values"
-    rms = float(np.sqrt(np.mean(ref * ref)))
+    rms = max(float(np.sqrt(np.mean(ref * ref))), float(scale))
     bound = rtol * np.abs(ref) + rtol * rms
     err = np.abs(got - ref)
     worst = int(np.argmax(err - bound))
     assert np.all(err <= bound), (
         f"{what}: max err {err.max():.3e} (rms(ref) {rms:.3e}); worst at flat index {worst}: "
         f"got {got.flat[worst]!r} ref {ref.flat[worst]!r} bound {bound.flat[worst]:.3e}")
+
+
+def dx_scale(dy, gamma_rms, rstd, dtype):
+    """rms of r * dy * gamma, the leading term of dx."""
+    d = O.from_storage(dy, dtype)
+    return float(np.sqrt(np.mean(d * d))) * float(gamma_rms) * float(np.sqrt(np.mean(np.square(rstd))))
 
 
 # ------------------------------------------------------------------ seeded inputs
