@@ -68,15 +68,14 @@ int fill_zero(float* out, int64_t n, hipStream_t st) {
 
 int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_t W,
                       hipStream_t st) {
-  constexpr int CX = 16, CY = 16;
   ATEXN_REQUIRE(2 * W < (int64_t(1) << 31), "column count %lld too large", (long long)W);
   const int Wi = static_cast<int>(W);
   if (W % 4 == 0 && aligned16(part)) {
-    const int grid = static_cast<int>(div_up(div_up(2 * W, 4), CX));
-    col_reduce<4, CX, CY><<<grid, CX * CY, 0, st>>>(part, out0, out1, G, Wi);
+    const int grid = static_cast<int>(div_up(2 * W, 4 * 4));
+    col_reduce<4, 4><<<grid, kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
   } else {
-    const int grid = static_cast<int>(div_up(2 * W, CX));
-    col_reduce<1, CX, CY><<<grid, CX * CY, 0, st>>>(part, out0, out1, G, Wi);
+    const int grid = static_cast<int>(div_up(2 * W, 16));
+    col_reduce<1, 16><<<grid, kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
   }
   ATEXN_CHECK_LAUNCH("col_reduce");
   return ATEXN_OK;

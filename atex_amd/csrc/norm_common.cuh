@@ -77,17 +77,67 @@ __device__ __forceinline__ void store_f32(float* p, const float (&in)[V]) {
 }
 
 // ------------------------------------------------------------------ cross-lane
-// Exchange with the lane whose id differs in bit `mask` (butterfly step).
+// Exchange with the lane whose id differs in bit `mask` (true butterfly step; goes
+// through the LDS crossbar, so it is kept off the per-row paths).
 __device__ __forceinline__ float lane_xor(float v, int mask) { return __shfl_xor(v, mask, kWave); }
 
-// Butterfly all-reduce (sum) over aligned groups of `width` lanes, width a power of two
-// <= 64.  Every lane of the group ends with the same bits.
+// DPP controls (gfx9 encoding).
+constexpr int kDppQuadXor1 = 0xB1;        // quad_perm:[1,0,3,2]
+constexpr int kDppQuadXor2 = 0x4E;        // quad_perm:[2,3,0,1]
+constexpr int kDppRowHalfMirror = 0x141;  // lane i <-> 7 - i inside each 8 lanes
+constexpr int kDppRowMirror = 0x140;      // lane i <-> 15 - i inside each 16 lanes
+
+template <int CTRL>
+__device__ __forceinline__ float dpp_read(float v) {
+  return __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, true));
+}
+
+// v + (v of the sibling 16-lane row / 32-lane half) through v_permlane{16,32}_swap_b32.
+// The instruction swaps the odd rows (upper half) of its first register with the even rows
+// (lower half) of its second; fed two copies of v, the first register ends up holding the
+// even-row (lower-half) values everywhere and the second the odd-row (upper-half) values,
+// so their sum is the pair total in every lane.  The second copy goes through an empty
+// asm so that the compiler treats the two results as distinct values.
+template <int SPAN>
+__device__ __forceinline__ float swap_add(float v) {
+  const unsigned a = __builtin_bit_cast(unsigned, v);
+  unsigned b = a;
+  asm volatile("" : "+v"(b));
+  unsigned r0, r1;
+  if constexpr (SPAN == 16) {
+    auto r = __builtin_amdgcn_permlane16_swap(a, b, false, false);
+    r0 = r[0];
+    r1 = r[1];
+  } else {
+    auto r = __builtin_amdgcn_permlane32_swap(a, b, false, false);
+    r0 = r[0];
+    r1 = r[1];
+  }
+  return __builtin_bit_cast(float, r0) + __builtin_bit_cast(float, r1);
+}
+
+// All-reduce (sum) over aligned groups of WIDTH lanes, WIDTH a power of two <= 64, with
+// VALU cross-lane operations only: two quad permutes, the two row mirrors, then the
+// gfx950 v_permlane16_swap / v_permlane32_swap for the 32- and 64-lane steps.  The
+// mirrors are not butterflies, but every lane of a sub-group already holds the
+// sub-group's total when they are applied, so pairing with ANY lane of the sibling
+// sub-group is enough.  Additions are commutative, so every lane of the group ends with
+// the same bits.
 template <int WIDTH>
 __device__ __forceinline__ float group_sum(float v) {
-#pragma unroll
-  for (int m = WIDTH / 2; m > 0; m >>= 1) v += lane_xor(v, m);
+  static_assert(WIDTH >= 1 && WIDTH <= 64 && (WIDTH & (WIDTH - 1)) == 0, "bad width");
+  if constexpr (WIDTH >= 2) v += dpp_read<kDppQuadXor1>(v);
+  if constexpr (WIDTH >= 4) v += dpp_read<kDppQuadXor2>(v);
+  if constexpr (WIDTH >= 8) v += dpp_read<kDppRowHalfMirror>(v);
+  if constexpr (WIDTH >= 16) v += dpp_read<kDppRowMirror>(v);
+  if constexpr (WIDTH >= 32) v = swap_add<16>(v);
+  if constexpr (WIDTH >= 64) v = swap_add<32>(v);
   return v;
 }
+
+// Fast reciprocal (v_rcp_f32, 1 ulp): used for counts, which are small integers.
+__device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }
 
 // ------------------------------------------------------------------- Welford
 // (mean, m2 = sum of squared deviations, n) of a set; merge is Chan's pairwise update
@@ -101,7 +151,7 @@ __device__ __forceinline__ Wf wf_merge(const Wf& a, const Wf& b) {
 #pragma clang fp contract(off)
   Wf r;
   r.n = a.n + b.n;
-  const float inv = r.n > 0.f ? 1.0f / r.n : 0.f;
+  const float inv = r.n > 0.f ? fast_rcp(r.n) : 0.f;
   const float d = b.mean - a.mean;
   const float wa = a.mean * a.n;
   const float wb = b.mean * b.n;
@@ -153,6 +203,19 @@ __device__ __forceinline__ float2 block_sum2(float a, float b, float2* buf) {
     r.x += buf[i].x;
     r.y += buf[i].y;
   }
+  return r;
+}
+
+// Block-wide all-reduce of one sum, same contract (`buf` holds 16 floats).
+__device__ __forceinline__ float block_sum1(float a, float* buf) {
+  a = group_sum<kWave>(a);
+  const int nw = blockDim.x / kWave;
+  if (nw == 1) return a;
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = a;
+  __syncthreads();
+  float r = buf[0];
+  for (int i = 1; i < nw; ++i) r += buf[i];
   return r;
 }
 

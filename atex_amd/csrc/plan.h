@@ -23,6 +23,8 @@ struct Tuning {
   int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
   int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
   int colgrad_items_per_cu = 4;   // LayerNorm column pass of the split path
+  int fwd_rows_batch = 2;         // resident kernels, rows <= one wave: rows in flight per
+  int bwd_rows_batch = 2;         //   lane group (1, 2 or 4; vector path only)
   // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
   // bit 1: the final column reduction).  Anything but 3 gives incomplete results.
   int bwd_stage_mask = 3;
@@ -44,7 +46,7 @@ struct RowsPlan {
   int V = 1;  // storage elements per access
   bool resident = false;
   // resident
-  int tpr = 0, vpt = 1, threads = 256, rpb = 1;
+  int tpr = 0, vpt = 1, threads = 256, rpb = 1, rb = 1;
   int grid = 1;
   size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
   // split
@@ -87,15 +89,18 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.rpb = 1;
     } else {
       p.threads = 256;
+      if (V > 1) p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
       if (kind == RowsKind::kBwdCols) {
-        // bigger blocks -> fewer partial rows for the column reduction
-        int th = t.bwd_ln_threads;
-        while (th > 256 && div_up(n_rows, th / p.tpr) < cus) th /= 2;
+        // bigger blocks -> fewer partial rows for the column reduction; batched rows need
+        // the register budget of a 512-thread block
+        int th = std::min(t.bwd_ln_threads, p.rb == 1 ? 1024 : 512);
+        while (th > 256 && div_up(n_rows, int64_t(th / p.tpr) * p.rb) < cus) th /= 2;
         p.threads = th;
       }
       p.rpb = p.threads / p.tpr;
+      while (p.rb > 1 && div_up(n_rows, int64_t(p.rpb) * p.rb) < cus) p.rb /= 2;
     }
-    const int64_t groups = div_up(n_rows, p.rpb);
+    const int64_t groups = div_up(n_rows, int64_t(p.rpb) * p.rb);
     const int waves = p.threads / 64;
     const int per_cu = std::max(
         1, (kind == RowsKind::kFwd ? t.fwd_waves_per_cu : t.bwd_waves_per_cu) / waves);

@@ -38,9 +38,9 @@ constexpr int resident_fwd_max_threads() {
   if (TPR != 0) return 256;
   return VPT >= 8 ? 1024 : 512;
 }
-template <int TPR, bool BWD_COLS>
+template <int TPR, bool BWD_COLS, int RB>
 constexpr int resident_bwd_max_threads() {
-  if (TPR != 0) return BWD_COLS ? 1024 : 256;
+  if (TPR != 0) return BWD_COLS ? (RB == 1 ? 1024 : 512) : 256;
   return 512;
 }
 
@@ -50,7 +50,7 @@ constexpr int resident_bwd_max_threads() {
 // of by column (LayerNorm).  y may alias x: every thread reads all of its vectors of a
 // row before it writes any.  The row is kept as raw 128-bit vectors and converted on
 // use, which halves the register footprint for 16-bit storage.
-template <typename T, int V, int TPR, int VPT, bool ROW_AFFINE>
+template <typename T, int V, int TPR, int VPT, int RB, bool ROW_AFFINE>
 __global__ void __launch_bounds__((resident_fwd_max_threads<TPR, VPT>()))
 rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta,
                   T* y, float* __restrict__ mean_out, float* __restrict__ rstd_out,
@@ -59,13 +59,15 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   constexpr int NE = V * VPT;
   // gamma / beta live in registers across rows unless that would exhaust the budget
   constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 4);
-  __shared__ Wf wf_buf[2][16];
+  static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
+  __shared__ float red_buf[2][2][16];
 
   const int tpr = M::tpr();
   const int rpb = M::rows_per_block();
   const int lane_r = M::lane_in_row();
   const int slot = M::slot();
   const int64_t D = static_cast<int64_t>(n_vec) * V;
+  const float inv_d = 1.0f / static_cast<float>(D);
 
   int n_valid_vec = 0;
 #pragma unroll
@@ -92,89 +94,118 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
     }
   }
 
+  // RB rows per lane group are in flight at once: all their loads are issued before the
+  // first is consumed, and the stages below run over the whole batch so that the
+  // independent reduction chains of its rows interleave.
   int it = 0;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb; row0 < n_rows;
-       row0 += static_cast<int64_t>(gridDim.x) * rpb, ++it) {
-    const int64_t row = row0 + slot;
-    const bool row_ok = row < n_rows;
-    const int nv = row_ok ? n_valid_vec : 0;
-    const T* xr = x + row * D;
-    Pack<T, V> raw[VPT];
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB; row0 < n_rows;
+       row0 += static_cast<int64_t>(gridDim.x) * rpb * RB, ++it) {
+    Pack<T, V> raw[RB][VPT];
+    int nv[RB];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (k < nv) raw[k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
+    for (int r = 0; r < RB; ++r) {
+      const int64_t row = row0 + r * rpb + slot;
+      nv[r] = row < n_rows ? n_valid_vec : 0;
+      const T* xr = x + row * D;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv[r]) raw[r][k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
+      }
     }
-    // statistics of this thread's elements: exact two-pass over registers
-    Wf w{0.f, 0.f, static_cast<float>(nv * V)};
-    if (nv > 0) {
+    // stage 1: convert once, sum; elements outside the row are kept at 0
+    float f[RB][NE];
+    float mean[RB], rstd[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
       float s = 0.f;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < nv) {
 #pragma unroll
-          for (int i = 0; i < V; ++i) s += to_f32(raw[k].v[i]);
+        for (int i = 0; i < V; ++i) {
+          const float v = (k < nv[r]) ? to_f32(raw[r][k].v[i]) : 0.f;
+          f[r][k * V + i] = v;
+          s += v;
         }
       }
-      w.mean = s / w.n;
+      mean[r] = s;
+    }
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      if constexpr (TPR != 0) {
+        mean[r] = group_sum<(TPR ? TPR : 1)>(mean[r]) * inv_d;
+      } else {
+        mean[r] = block_sum1(mean[r], red_buf[it & 1][0]) * inv_d;
+      }
+    }
+    // stage 2: centre (exact second pass over registers), sum of squares
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
       float q = 0.f;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < nv) {
-#pragma unroll
-          for (int i = 0; i < V; ++i) {
-            const float d = to_f32(raw[k].v[i]) - w.mean;
-            q += d * d;
-          }
-        }
-      }
-      w.m2 = q;
-    }
-    if constexpr (TPR != 0) {
-      w = group_wf<(TPR ? TPR : 1)>(w);
-    } else {
-      w = block_wf(w, wf_buf[it & 1]);
-    }
-    const float mean = w.mean;
-    const float rstd = rsqrtf(w.m2 / static_cast<float>(D) + eps);
-
-    float gs = 1.f, bs = 0.f;
-    if constexpr (ROW_AFFINE) {
-      if (row_ok) {
-        const int c = static_cast<int>(row % C);
-        gs = gamma[c];
-        bs = beta[c];
-      }
-    }
-    T* yr = y + row * D;
-#pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (k < nv) {
-        const int col = (lane_r + k * tpr) * V;
-        float tg[V], tb[V];
-        if constexpr (!ROW_AFFINE && !GB_REGS) {
-          load_f32<V>(gamma + col, tg);
-          load_f32<V>(beta + col, tb);
-        }
-        Pack<T, V> o;
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float xh = (to_f32(raw[k].v[i]) - mean) * rstd;
-          float r;
-          if constexpr (ROW_AFFINE) {
-            r = xh * gs + bs;
-          } else if constexpr (GB_REGS) {
-            r = xh * g[k * V + i] + b[k * V + i];
-          } else {
-            r = xh * tg[i] + tb[i];
-          }
-          o.v[i] = from_f32<T>(r);
+          const float d = (k < nv[r]) ? f[r][k * V + i] - mean[r] : 0.f;
+          f[r][k * V + i] = d;
+          q += d * d;
         }
-        store_pack<T, V>(yr + col, o);
       }
+      rstd[r] = q;
     }
-    if (row_ok && lane_r == 0) {
-      mean_out[row] = mean;
-      rstd_out[row] = rstd;
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      float q;
+      if constexpr (TPR != 0) {
+        q = group_sum<(TPR ? TPR : 1)>(rstd[r]);
+      } else {
+        q = block_sum1(rstd[r], red_buf[it & 1][1]);
+      }
+      rstd[r] = rsqrtf(q * inv_d + eps);
+    }
+    // stage 3: scale, shift, store
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const int64_t row = row0 + r * rpb + slot;
+      const bool row_ok = row < n_rows;
+      float gs = 1.f, bs = 0.f;
+      if constexpr (ROW_AFFINE) {
+        if (row_ok) {
+          const int c = static_cast<int>(row % C);
+          gs = gamma[c] * rstd[r];
+          bs = beta[c];
+        }
+      }
+      T* yr = y + row * D;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv[r]) {
+          const int col = (lane_r + k * tpr) * V;
+          float tg[V], tb[V];
+          if constexpr (!ROW_AFFINE && !GB_REGS) {
+            load_f32<V>(gamma + col, tg);
+            load_f32<V>(beta + col, tb);
+          }
+          Pack<T, V> o;
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const float d = f[r][k * V + i];
+            float res;
+            if constexpr (ROW_AFFINE) {
+              res = d * gs + bs;
+            } else if constexpr (GB_REGS) {
+              res = d * (rstd[r] * g[k * V + i]) + b[k * V + i];
+            } else {
+              res = d * (rstd[r] * tg[i]) + tb[i];
+            }
+            o.v[i] = from_f32<T>(res);
+          }
+          store_pack<T, V>(yr + col, o);
+        }
+      }
+      if (row_ok && lane_r == 0) {
+        mean_out[row] = mean[r];
+        rstd_out[row] = rstd[r];
+      }
     }
   }
 }
@@ -197,8 +228,8 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // are written to part[n][0][c] = b, part[n][1][c] = a  (n = row / C), i.e. `part` has
 // N * 2 * C floats and the same second kernel folds it over n.
 // dx must not alias dy or x.
-template <typename T, int V, int TPR, int VPT, bool ROW_AFFINE>
-__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE>()))
+template <typename T, int V, int TPR, int VPT, int RB, bool ROW_AFFINE>
+__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB>()))
 rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* __restrict__ dx,
@@ -241,84 +272,103 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
     }
   }
 
+  static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
   int it = 0;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb; row0 < n_rows;
-       row0 += static_cast<int64_t>(gridDim.x) * rpb, ++it) {
-    const int64_t row = row0 + slot;
-    const bool row_ok = row < n_rows;
-    const int nv = row_ok ? n_valid_vec : 0;
-    const T* xr = x + row * D;
-    const T* dyr = dy + row * D;
-    Pack<T, V> px[VPT], pd[VPT];
-    float mean = 0.f, rstd = 0.f, gs = 0.f;
-    if (row_ok) {
-      mean = mean_in[row];
-      rstd = rstd_in[row];
-      if constexpr (ROW_AFFINE) gs = gamma[static_cast<int>(row % C)];
-    }
+  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB; row0 < n_rows;
+       row0 += static_cast<int64_t>(gridDim.x) * rpb * RB, ++it) {
+    Pack<T, V> px[RB][VPT], pd[RB][VPT];
+    float rstd[RB], mean[RB];
+    int nv[RB];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (k < nv) {
-        const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
-        px[k] = load_pack<T, V>(xr + off);
-        pd[k] = load_pack<T, V>(dyr + off);
-      }
-    }
-    float s1 = 0.f, s2 = 0.f;
+    for (int r = 0; r < RB; ++r) {
+      const int64_t row = row0 + r * rpb + slot;
+      const bool row_ok = row < n_rows;
+      nv[r] = row_ok ? n_valid_vec : 0;
+      const T* xr = x + row * D;
+      const T* dyr = dy + row * D;
+      mean[r] = row_ok ? mean_in[row] : 0.f;
+      rstd[r] = row_ok ? rstd_in[row] : 0.f;
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (k < nv) {
-#pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float xh = (to_f32(px[k].v[i]) - mean) * rstd;
-          const float d = to_f32(pd[k].v[i]);
-          if constexpr (ROW_AFFINE) {
-            s1 += d;
-            s2 += d * xh;
-          } else {
-            const float gv = d * g[k * V + i];
-            s1 += gv;
-            s2 += gv * xh;
-            acc_g[k * V + i] += d * xh;
-            acc_b[k * V + i] += d;
-          }
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv[r]) {
+          const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
+          px[r][k] = load_pack<T, V>(xr + off);
+          pd[r][k] = load_pack<T, V>(dyr + off);
         }
       }
     }
-    if constexpr (TPR != 0) {
-      s1 = group_sum<(TPR ? TPR : 1)>(s1);
-      s2 = group_sum<(TPR ? TPR : 1)>(s2);
-    } else {
-      const float2 r = block_sum2(s1, s2, sum_buf[it & 1]);
-      s1 = r.x;
-      s2 = r.y;
-    }
-    if constexpr (ROW_AFFINE) {
-      if (row_ok && lane_r == 0) {
-        const int64_t n = row / C;
-        const int c = static_cast<int>(row % C);
-        part[(n * 2 + 0) * C + c] = s2;
-        part[(n * 2 + 1) * C + c] = s1;
-      }
-    }
-    T* dxr = dx + row * D;
+    // stage 1: convert once; xh = (x - mean) * r, gv = dy * gamma; row sums and the
+    // column accumulators.  Elements outside the row are 0 and add nothing.
+    float xh[RB][NE], gv[RB][NE];
+    float s1[RB], s2[RB];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) {
-      if (k < nv) {
-        Pack<T, V> o;
+    for (int r = 0; r < RB; ++r) {
+      float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float xh = (to_f32(px[k].v[i]) - mean) * rstd;
-          const float d = to_f32(pd[k].v[i]);
-          float r;
+          const int e = k * V + i;
+          const bool ok = k < nv[r];
+          const float h = ok ? (to_f32(px[r][k].v[i]) - mean[r]) * rstd[r] : 0.f;
+          const float d = ok ? to_f32(pd[r][k].v[i]) : 0.f;
+          xh[r][e] = h;
           if constexpr (ROW_AFFINE) {
-            r = rstd * gs * (d - (s1 + xh * s2) * inv_d);
+            gv[r][e] = d;
+            a1 += d;
+            a2 += d * h;
           } else {
-            r = rstd * (d * g[k * V + i] - (s1 + xh * s2) * inv_d);
+            const float t = d * g[e];
+            gv[r][e] = t;
+            a1 += t;
+            a2 += t * h;
+            acc_g[e] += d * h;
+            acc_b[e] += d;
           }
-          o.v[i] = from_f32<T>(r);
         }
-        store_pack<T, V>(dxr + static_cast<int64_t>(lane_r + k * tpr) * V, o);
+      }
+      s1[r] = a1;
+      s2[r] = a2;
+    }
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      if constexpr (TPR != 0) {
+        s1[r] = group_sum<(TPR ? TPR : 1)>(s1[r]);
+        s2[r] = group_sum<(TPR ? TPR : 1)>(s2[r]);
+      } else {
+        const float2 t = block_sum2(s1[r], s2[r], sum_buf[it & 1]);
+        s1[r] = t.x;
+        s2[r] = t.y;
+      }
+    }
+    // stage 2: dx
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const int64_t row = row0 + r * rpb + slot;
+      const bool row_ok = row < n_rows;
+      float scale = rstd[r];
+      if constexpr (ROW_AFFINE) {
+        if (row_ok) scale *= gamma[static_cast<int>(row % C)];
+        if (row_ok && lane_r == 0) {
+          const int64_t n = row / C;
+          const int c = static_cast<int>(row % C);
+          part[(n * 2 + 0) * C + c] = s2[r];
+          part[(n * 2 + 1) * C + c] = s1[r];
+        }
+      }
+      const float m1 = s1[r] * inv_d, m2 = s2[r] * inv_d;
+      T* dxr = dx + row * D;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (k < nv[r]) {
+          Pack<T, V> o;
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const int e = k * V + i;
+            o.v[i] = from_f32<T>(scale * (gv[r][e] - (m1 + xh[r][e] * m2)));
+          }
+          store_pack<T, V>(dxr + static_cast<int64_t>(lane_r + k * tpr) * V, o);
+        }
       }
     }
   }
@@ -406,11 +456,19 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 // out0[j] = sum_g part[g][0][j], out1[j] = sum_g part[g][1][j] for j < W, g < G, summed
 // in a fixed order (deterministic; the reference likewise uses no atomics,
 // fused_layer_norm_op.cu:763-803, fused_instance_norm_op.cu:442-457).
-// Block = (CX column groups of CW floats) x (CY slices of g).  blockDim.x = CX * CY.
-template <int CW, int CX, int CY>
-__global__ void col_reduce(const float* __restrict__ part, float* __restrict__ out0,
-                           float* __restrict__ out1, int G, int W) {
-  __shared__ float buf[CY][CX][CW];
+// Block of 256 threads = CX column groups of CW floats x (256 / CX) slices of g; a block
+// owns CX * CW adjacent columns of the concatenated [2W] row, so the grid has
+// 2W / (CX * CW) blocks (128 for W = 1024).  Slices are folded by a lane butterfly and a
+// 4-entry LDS step.
+constexpr int kColReduceThreads = 256;
+
+template <int CW, int CX>
+__global__ void __launch_bounds__(kColReduceThreads)
+col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __restrict__ out1,
+           int G, int W) {
+  constexpr int CY = kColReduceThreads / CX;
+  constexpr int NW = kColReduceThreads / kWave;
+  __shared__ float buf[NW][CX][CW];
   const int cx = threadIdx.x % CX;
   const int cy = threadIdx.x / CX;
   const int W2 = 2 * W;
@@ -419,31 +477,49 @@ __global__ void col_reduce(const float* __restrict__ part, float* __restrict__ o
 #pragma unroll
   for (int i = 0; i < CW; ++i) acc[i] = 0.f;
   if (col < W2) {
-    for (int g = cy; g < G; g += CY) {
+    const float* p = part + col;
+    int g = cy;
+    for (; g + 3 * CY < G; g += 4 * CY) {
+      float t0[CW], t1[CW], t2[CW], t3[CW];
+      load_f32<CW>(p + static_cast<int64_t>(g) * W2, t0);
+      load_f32<CW>(p + static_cast<int64_t>(g + CY) * W2, t1);
+      load_f32<CW>(p + static_cast<int64_t>(g + 2 * CY) * W2, t2);
+      load_f32<CW>(p + static_cast<int64_t>(g + 3 * CY) * W2, t3);
+#pragma unroll
+      for (int i = 0; i < CW; ++i) acc[i] += (t0[i] + t1[i]) + (t2[i] + t3[i]);
+    }
+    for (; g < G; g += CY) {
       float t[CW];
-      load_f32<CW>(part + static_cast<int64_t>(g) * W2 + col, t);
+      load_f32<CW>(p + static_cast<int64_t>(g) * W2, t);
 #pragma unroll
       for (int i = 0; i < CW; ++i) acc[i] += t[i];
     }
   }
+  // lanes l, l + CX, ... of a wave hold slices of the same columns
 #pragma unroll
-  for (int i = 0; i < CW; ++i) buf[cy][cx][i] = acc[i];
+  for (int i = 0; i < CW; ++i) {
+#pragma unroll
+    for (int m = CX; m < kWave; m <<= 1) acc[i] += lane_xor(acc[i], m);
+  }
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  if (lane < CX) {
+#pragma unroll
+    for (int i = 0; i < CW; ++i) buf[wave][lane][i] = acc[i];
+  }
   __syncthreads();
-  if (cy == 0 && col < W2) {
+  if (threadIdx.x < CX && col < W2) {
 #pragma unroll
     for (int i = 0; i < CW; ++i) {
       float s = buf[0][cx][i];
-      for (int k = 1; k < CY; ++k) s += buf[k][cx][i];
-      acc[i] = s;
-    }
-    // CW divides W on the vector path, so a column group never straddles the two halves
 #pragma unroll
-    for (int i = 0; i < CW; ++i) {
+      for (int k = 1; k < NW; ++k) s += buf[k][cx][i];
+      // CW divides W on the vector path, so a column group never straddles the two halves
       const int j = col + i;
       if (j < W) {
-        out0[j] = acc[i];
-      } else {
-        out1[j - W] = acc[i];
+        out0[j] = s;
+      } else if (j < W2) {
+        out1[j - W] = s;
       }
     }
   }
