@@ -74,14 +74,15 @@ int atexn_set_tuning(const char* name, int value) {
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_ln_threads")) {
-    ATEXN_REQUIRE(value == 256 || value == 512 || value == 1024, "bwd_ln_threads must be 256, 512 or 1024");
+    ATEXN_REQUIRE(value == 256 || value == 512, "bwd_ln_threads must be 256 or 512");
     t.bwd_ln_threads = value;
   } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
   else if (!strcmp(name, "split_items_per_cu")) t.split_items_per_cu = value;
   else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
   else if (!strcmp(name, "colgrad_items_per_cu")) t.colgrad_items_per_cu = value;
   else if (!strcmp(name, "fwd_rows_batch") || !strcmp(name, "bwd_rows_batch")) {
-    ATEXN_REQUIRE(value == 1 || value == 2 || value == 4, "rows batch must be 1, 2 or 4");
+    ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),
+                  "rows batch must be 1, 2 (or 4, forward only)");
     (name[0] == 'f' ? t.fwd_rows_batch : t.bwd_rows_batch) = value;
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");

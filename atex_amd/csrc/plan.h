@@ -17,14 +17,14 @@ namespace atexn {
 
 // Tunables (process-wide; defaults chosen by measurement on MI355X).
 struct Tuning {
-  int fwd_waves_per_cu = 32;      // resident forward: waves kept resident per CU
-  int bwd_ln_threads = 1024;      // resident LayerNorm backward, rows <= one wave: block size
-  int bwd_waves_per_cu = 16;      // resident backward: waves kept resident per CU
+  int fwd_waves_per_cu = 16;      // resident forward: waves kept resident per CU
+  int bwd_ln_threads = 512;       // resident LayerNorm backward, rows <= one wave: block size
+  int bwd_waves_per_cu = 8;       // resident backward: waves kept resident per CU
   int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
   int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
   int colgrad_items_per_cu = 4;   // LayerNorm column pass of the split path
-  int fwd_rows_batch = 2;         // resident kernels, rows <= one wave: rows in flight per
-  int bwd_rows_batch = 2;         //   lane group (1, 2 or 4; vector path only)
+  int fwd_rows_batch = 4;         // resident kernels, rows <= one wave: rows per batch of a
+  int bwd_rows_batch = 1;         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
   // bit 1: the final column reduction).  Anything but 3 gives incomplete results.
   int bwd_stage_mask = 3;
@@ -47,6 +47,7 @@ struct RowsPlan {
   bool resident = false;
   // resident
   int tpr = 0, vpt = 1, threads = 256, rpb = 1, rb = 1;
+  bool exact = false;  // no lane, vector or row of any batch falls outside the data
   int grid = 1;
   size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
   // split
@@ -67,11 +68,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   RowsPlan p;
   p.V = V;
   const int64_t n_vec = D / V;  // D % V == 0 whenever V > 1
-  // Limits follow the register budgets of the resident kernels: forward 1024 threads x 8
-  // vectors; backward 512 threads x 8 (InstanceNorm) or x 4 (LayerNorm, which also keeps
-  // gamma and the dgamma / dbeta accumulators of its columns in registers).
-  const int64_t resident_limit =
-      kind == RowsKind::kFwd ? 8192 : (kind == RowsKind::kBwdAffine ? 4096 : 2048);
+  // Limits follow the register budgets of the resident kernels at 512 threads: forward 8
+  // vectors per thread, backward 4 (it holds x and dy, and LayerNorm also gamma and the
+  // dgamma / dbeta accumulators of its columns).
+  const int64_t resident_limit = kind == RowsKind::kFwd ? 4096 : 2048;
   p.resident = n_vec <= resident_limit;
   if (p.resident) {
     if (n_vec <= 64) {
@@ -91,9 +91,8 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.threads = 256;
       if (V > 1) p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
       if (kind == RowsKind::kBwdCols) {
-        // bigger blocks -> fewer partial rows for the column reduction; batched rows need
-        // the register budget of a 512-thread block
-        int th = std::min(t.bwd_ln_threads, p.rb == 1 ? 1024 : 512);
+        // bigger blocks -> fewer partial rows for the column reduction
+        int th = std::min(t.bwd_ln_threads, 512);
         while (th > 256 && div_up(n_rows, int64_t(th / p.tpr) * p.rb) < cus) th /= 2;
         p.threads = th;
       }
@@ -101,6 +100,8 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       while (p.rb > 1 && div_up(n_rows, int64_t(p.rpb) * p.rb) < cus) p.rb /= 2;
     }
     const int64_t groups = div_up(n_rows, int64_t(p.rpb) * p.rb);
+    p.exact = V > 1 && n_vec == int64_t(p.tpr == 0 ? p.threads : p.tpr) * p.vpt &&
+              n_rows % (int64_t(p.rpb) * p.rb) == 0;
     const int waves = p.threads / 64;
     const int per_cu = std::max(
         1, (kind == RowsKind::kFwd ? t.fwd_waves_per_cu : t.bwd_waves_per_cu) / waves);

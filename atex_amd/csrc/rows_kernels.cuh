@@ -35,22 +35,30 @@ constexpr int kFoldWaves = 4;
 // budget the compiler works against (512 VGPRs per SIMD lane / waves per SIMD).
 template <int TPR, int VPT>
 constexpr int resident_fwd_max_threads() {
-  if (TPR != 0) return 256;
-  return VPT >= 8 ? 1024 : 512;
+  return TPR != 0 ? 256 : 512;
 }
 template <int TPR, bool BWD_COLS, int RB>
 constexpr int resident_bwd_max_threads() {
-  if (TPR != 0) return BWD_COLS ? (RB == 1 ? 1024 : 512) : 256;
-  return 512;
+  return (TPR != 0 && !BWD_COLS) ? 256 : 512;
 }
 
 // ------------------------------------------------------------------ forward, resident
 // y = (x - mean) * inv_std * gamma + beta ; mean / inv_std saved per row.
 // ROW_AFFINE: gamma / beta are indexed by (row % C) (channel-first InstanceNorm) instead
-// of by column (LayerNorm).  y may alias x: every thread reads all of its vectors of a
-// row before it writes any.  The row is kept as raw 128-bit vectors and converted on
-// use, which halves the register footprint for 16-bit storage.
-template <typename T, int V, int TPR, int VPT, int RB, bool ROW_AFFINE>
+// of by column (LayerNorm).  y may alias x: a thread reads all of its vectors of a row
+// before it writes any, and rows are never shared between lane groups.
+//
+// Statistics: the row is on chip, so the mean comes from one all-reduce of the sums and
+// the variance from a second all-reduce of the squared deviations from that mean (the
+// exact two-pass form, cheaper and more accurate than merging Welford triples across
+// lanes); HBM sees the row once.
+//
+// RB rows per lane group form a batch; the next batch is loaded (software prefetch)
+// before the current one is reduced, so loads overlap the arithmetic.
+// EXACT: every lane owns exactly VPT vectors of every row of every batch (host-checked:
+// n_vec == lanes-per-row * VPT and n_rows % (rows-per-block * RB) == 0); all predicates
+// fold away.
+template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE>
 __global__ void __launch_bounds__((resident_fwd_max_threads<TPR, VPT>()))
 rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta,
                   T* y, float* __restrict__ mean_out, float* __restrict__ rstd_out,
@@ -69,16 +77,19 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   const int64_t D = static_cast<int64_t>(n_vec) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
 
-  int n_valid_vec = 0;
+  int n_valid_vec = VPT;
+  if constexpr (!EXACT) {
+    n_valid_vec = 0;
 #pragma unroll
-  for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+    for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+  }
 
   float g[GB_REGS ? NE : 1], b[GB_REGS ? NE : 1];
   if constexpr (GB_REGS) {
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float tg[V], tb[V];
-      if (k < n_valid_vec) {
+      if (EXACT || k < n_valid_vec) {
         const int col = (lane_r + k * tpr) * V;
         load_f32<V>(gamma + col, tg);
         load_f32<V>(beta + col, tb);
@@ -94,23 +105,39 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
     }
   }
 
-  // RB rows per lane group are in flight at once: all their loads are issued before the
-  // first is consumed, and the stages below run over the whole batch so that the
-  // independent reduction chains of its rows interleave.
-  int it = 0;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB; row0 < n_rows;
-       row0 += static_cast<int64_t>(gridDim.x) * rpb * RB, ++it) {
-    Pack<T, V> raw[RB][VPT];
-    int nv[RB];
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * rpb * RB;
+  int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB;
+
+  auto load_batch = [&](int64_t base, Pack<T, V>(&raw)[RB][VPT]) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int64_t row = row0 + r * rpb + slot;
-      nv[r] = row < n_rows ? n_valid_vec : 0;
+      const int64_t row = base + r * rpb + slot;
+      const int nv = (EXACT || row < n_rows) ? n_valid_vec : 0;
       const T* xr = x + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < nv[r]) raw[r][k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
+        if (EXACT || k < nv) raw[r][k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
       }
+    }
+  };
+
+  // prefetching doubles the raw-vector registers; long rows do without it
+  constexpr bool PREFETCH = VPT * RB <= 4;
+  Pack<T, V> cur[RB][VPT];
+  if (PREFETCH && row0 < n_rows) load_batch(row0, cur);
+  for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+    Pack<T, V> nxt[PREFETCH ? RB : 1][VPT];
+    const bool more = PREFETCH && row0 + stride < n_rows;
+    if constexpr (PREFETCH) {
+      if (more) load_batch(row0 + stride, nxt);
+    } else {
+      load_batch(row0, cur);
+    }
+
+    int nv[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      nv[r] = (EXACT || row0 + r * rpb + slot < n_rows) ? n_valid_vec : 0;
     }
     // stage 1: convert once, sum; elements outside the row are kept at 0
     float f[RB][NE];
@@ -122,7 +149,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float v = (k < nv[r]) ? to_f32(raw[r][k].v[i]) : 0.f;
+          const float v = (EXACT || k < nv[r]) ? to_f32(cur[r][k].v[i]) : 0.f;
           f[r][k * V + i] = v;
           s += v;
         }
@@ -145,7 +172,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float d = (k < nv[r]) ? f[r][k * V + i] - mean[r] : 0.f;
+          const float d = (EXACT || k < nv[r]) ? f[r][k * V + i] - mean[r] : 0.f;
           f[r][k * V + i] = d;
           q += d * d;
         }
@@ -166,7 +193,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int64_t row = row0 + r * rpb + slot;
-      const bool row_ok = row < n_rows;
+      const bool row_ok = EXACT || row < n_rows;
       float gs = 1.f, bs = 0.f;
       if constexpr (ROW_AFFINE) {
         if (row_ok) {
@@ -178,7 +205,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       T* yr = y + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < nv[r]) {
+        if (EXACT || k < nv[r]) {
           const int col = (lane_r + k * tpr) * V;
           float tg[V], tb[V];
           if constexpr (!ROW_AFFINE && !GB_REGS) {
@@ -207,6 +234,15 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
         rstd_out[row] = rstd[r];
       }
     }
+    if constexpr (PREFETCH) {
+      if (more) {
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+#pragma unroll
+          for (int k = 0; k < VPT; ++k) cur[r][k] = nxt[r][k];
+        }
+      }
+    }
   }
 }
 
@@ -227,8 +263,8 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // row % C, the two row sums a = sum dy, b = sum dy * xh give s1 = gamma a, s2 = gamma b and
 // are written to part[n][0][c] = b, part[n][1][c] = a  (n = row / C), i.e. `part` has
 // N * 2 * C floats and the same second kernel folds it over n.
-// dx must not alias dy or x.
-template <typename T, int V, int TPR, int VPT, int RB, bool ROW_AFFINE>
+// dx must not alias dy or x.  RB / EXACT / prefetch as in the forward kernel.
+template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE>
 __global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB>()))
 rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
@@ -236,6 +272,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   float* __restrict__ part, int64_t n_rows, int n_vec, int C) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
+  static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float2 sum_buf[2][16];
   // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats
   extern __shared__ float fold_buf[];
@@ -247,9 +284,12 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
   const int64_t D = static_cast<int64_t>(n_vec) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
 
-  int n_valid_vec = 0;
+  int n_valid_vec = VPT;
+  if constexpr (!EXACT) {
+    n_valid_vec = 0;
 #pragma unroll
-  for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+    for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+  }
 
   float g[ROW_AFFINE ? 1 : NE];
   float acc_g[ROW_AFFINE ? 1 : NE], acc_b[ROW_AFFINE ? 1 : NE];
@@ -257,7 +297,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float tg[V];
-      if (k < n_valid_vec) {
+      if (EXACT || k < n_valid_vec) {
         load_f32<V>(gamma + (lane_r + k * tpr) * V, tg);
       } else {
 #pragma unroll
@@ -272,30 +312,50 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
     }
   }
 
-  static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
-  int it = 0;
-  for (int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB; row0 < n_rows;
-       row0 += static_cast<int64_t>(gridDim.x) * rpb * RB, ++it) {
+  const int64_t stride = static_cast<int64_t>(gridDim.x) * rpb * RB;
+  int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB;
+
+  struct Batch {
     Pack<T, V> px[RB][VPT], pd[RB][VPT];
-    float rstd[RB], mean[RB];
+    float mean[RB], rstd[RB];
+  };
+  auto load_batch = [&](int64_t base, Batch& t) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      const int64_t row = base + r * rpb + slot;
+      const bool row_ok = EXACT || row < n_rows;
+      const int nv = row_ok ? n_valid_vec : 0;
+      const T* xr = x + row * D;
+      const T* dyr = dy + row * D;
+      t.mean[r] = row_ok ? mean_in[row] : 0.f;
+      t.rstd[r] = row_ok ? rstd_in[row] : 0.f;
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) {
+        if (EXACT || k < nv) {
+          const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
+          t.px[r][k] = load_pack<T, V>(xr + off);
+          t.pd[r][k] = load_pack<T, V>(dyr + off);
+        }
+      }
+    }
+  };
+
+  constexpr bool PREFETCH = VPT * RB <= 2;
+  Batch cur;
+  if (PREFETCH && row0 < n_rows) load_batch(row0, cur);
+  for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+    Batch nxt;
+    const bool more = PREFETCH && row0 + stride < n_rows;
+    if constexpr (PREFETCH) {
+      if (more) load_batch(row0 + stride, nxt);
+    } else {
+      load_batch(row0, cur);
+    }
+
     int nv[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int64_t row = row0 + r * rpb + slot;
-      const bool row_ok = row < n_rows;
-      nv[r] = row_ok ? n_valid_vec : 0;
-      const T* xr = x + row * D;
-      const T* dyr = dy + row * D;
-      mean[r] = row_ok ? mean_in[row] : 0.f;
-      rstd[r] = row_ok ? rstd_in[row] : 0.f;
-#pragma unroll
-      for (int k = 0; k < VPT; ++k) {
-        if (k < nv[r]) {
-          const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
-          px[r][k] = load_pack<T, V>(xr + off);
-          pd[r][k] = load_pack<T, V>(dyr + off);
-        }
-      }
+      nv[r] = (EXACT || row0 + r * rpb + slot < n_rows) ? n_valid_vec : 0;
     }
     // stage 1: convert once; xh = (x - mean) * r, gv = dy * gamma; row sums and the
     // column accumulators.  Elements outside the row are 0 and add nothing.
@@ -309,9 +369,9 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const int e = k * V + i;
-          const bool ok = k < nv[r];
-          const float h = ok ? (to_f32(px[r][k].v[i]) - mean[r]) * rstd[r] : 0.f;
-          const float d = ok ? to_f32(pd[r][k].v[i]) : 0.f;
+          const bool ok = EXACT || k < nv[r];
+          const float h = ok ? (to_f32(cur.px[r][k].v[i]) - cur.mean[r]) * cur.rstd[r] : 0.f;
+          const float d = ok ? to_f32(cur.pd[r][k].v[i]) : 0.f;
           xh[r][e] = h;
           if constexpr (ROW_AFFINE) {
             gv[r][e] = d;
@@ -341,12 +401,12 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
         s2[r] = t.y;
       }
     }
-    // stage 2: dx
+    // stage 2: dx = scale * gv + (A * xh + B), A = -scale * s2 / D, B = -scale * s1 / D
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int64_t row = row0 + r * rpb + slot;
-      const bool row_ok = row < n_rows;
-      float scale = rstd[r];
+      const bool row_ok = EXACT || row < n_rows;
+      float scale = cur.rstd[r];
       if constexpr (ROW_AFFINE) {
         if (row_ok) scale *= gamma[static_cast<int>(row % C)];
         if (row_ok && lane_r == 0) {
@@ -356,20 +416,23 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
           part[(n * 2 + 1) * C + c] = s1[r];
         }
       }
-      const float m1 = s1[r] * inv_d, m2 = s2[r] * inv_d;
+      const float ca = -scale * (s2[r] * inv_d), cb = -scale * (s1[r] * inv_d);
       T* dxr = dx + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < nv[r]) {
+        if (EXACT || k < nv[r]) {
           Pack<T, V> o;
 #pragma unroll
           for (int i = 0; i < V; ++i) {
             const int e = k * V + i;
-            o.v[i] = from_f32<T>(scale * (gv[r][e] - (m1 + xh[r][e] * m2)));
+            o.v[i] = from_f32<T>(scale * gv[r][e] + (ca * xh[r][e] + cb));
           }
           store_pack<T, V>(dxr + static_cast<int64_t>(lane_r + k * tpr) * V, o);
         }
       }
+    }
+    if constexpr (PREFETCH) {
+      if (more) cur = nxt;
     }
   }
 

@@ -15,49 +15,52 @@ template <typename T, int V, bool AFF>
 using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, const float*, T*,
                                float*, int64_t, int, int);
 
-// Row batching (RB > 1) exists for the vector path and rows of at most one wave.
+// Row batching (RB > 1) exists for the vector path and rows of at most one wave; the
+// predicate-free EXACT variants exist for the vector path.
 template <typename T, int V, int TPR, int VPT, bool AFF>
-FwdResidentFn<T, V, AFF> fwd_by_batch(int rb) {
-  if constexpr (V > 1 && TPR != 0) {
-    if (rb == 2) return rows_fwd_resident<T, V, TPR, VPT, 2, AFF>;
-    if (rb == 4) return rows_fwd_resident<T, V, TPR, VPT, 4, AFF>;
+FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact) {
+  if constexpr (V > 1) {
+    if constexpr (TPR != 0) {
+      if (rb == 2) return exact ? rows_fwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 2, false, AFF>;
+      if (rb == 4) return exact ? rows_fwd_resident<T, V, TPR, VPT, 4, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 4, false, AFF>;
+    }
+    if (rb == 1 && exact) return rows_fwd_resident<T, V, TPR, VPT, 1, true, AFF>;
   }
-  return rb == 1 ? rows_fwd_resident<T, V, TPR, VPT, 1, AFF> : nullptr;
+  return rb == 1 ? rows_fwd_resident<T, V, TPR, VPT, 1, false, AFF> : nullptr;
 }
 template <typename T, int V, int TPR, int VPT, bool AFF>
-BwdResidentFn<T, V, AFF> bwd_by_batch(int rb) {
-  if constexpr (V > 1 && TPR != 0) {
-    if (rb == 2) return rows_bwd_resident<T, V, TPR, VPT, 2, AFF>;
-    if (rb == 4) return rows_bwd_resident<T, V, TPR, VPT, 4, AFF>;
+BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact) {
+  if constexpr (V > 1) {
+    if constexpr (TPR != 0) {
+      if (rb == 2) return exact ? rows_bwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF>;
+    }
+    if (rb == 1 && exact) return rows_bwd_resident<T, V, TPR, VPT, 1, true, AFF>;
   }
-  return rb == 1 ? rows_bwd_resident<T, V, TPR, VPT, 1, AFF> : nullptr;
+  return rb == 1 ? rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF> : nullptr;
 }
 
 template <typename T, int V, bool AFF>
-FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb) {
-  if (tpr == 8) return fwd_by_batch<T, V, 8, 1, AFF>(rb);
-  if (tpr == 16) return fwd_by_batch<T, V, 16, 1, AFF>(rb);
-  if (tpr == 32) return fwd_by_batch<T, V, 32, 1, AFF>(rb);
-  if (tpr == 64 && vpt == 1) return fwd_by_batch<T, V, 64, 1, AFF>(rb);
-  if (tpr == 64 && vpt == 2) return fwd_by_batch<T, V, 64, 2, AFF>(rb);
-  if (tpr == 0 && vpt == 2) return fwd_by_batch<T, V, 0, 2, AFF>(rb);
-  if (tpr == 0 && vpt == 4) return fwd_by_batch<T, V, 0, 4, AFF>(rb);
-  if (tpr == 0 && vpt == 8) return fwd_by_batch<T, V, 0, 8, AFF>(rb);
+FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb, bool exact) {
+  if (tpr == 8) return fwd_variant<T, V, 8, 1, AFF>(rb, exact);
+  if (tpr == 16) return fwd_variant<T, V, 16, 1, AFF>(rb, exact);
+  if (tpr == 32) return fwd_variant<T, V, 32, 1, AFF>(rb, exact);
+  if (tpr == 64 && vpt == 1) return fwd_variant<T, V, 64, 1, AFF>(rb, exact);
+  if (tpr == 64 && vpt == 2) return fwd_variant<T, V, 64, 2, AFF>(rb, exact);
+  if (tpr == 0 && vpt == 2) return fwd_variant<T, V, 0, 2, AFF>(rb, exact);
+  if (tpr == 0 && vpt == 4) return fwd_variant<T, V, 0, 4, AFF>(rb, exact);
+  if (tpr == 0 && vpt == 8) return fwd_variant<T, V, 0, 8, AFF>(rb, exact);
   return nullptr;
 }
 
 template <typename T, int V, bool AFF>
-BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb) {
-  if (tpr == 8) return bwd_by_batch<T, V, 8, 1, AFF>(rb);
-  if (tpr == 16) return bwd_by_batch<T, V, 16, 1, AFF>(rb);
-  if (tpr == 32) return bwd_by_batch<T, V, 32, 1, AFF>(rb);
-  if (tpr == 64 && vpt == 1) return bwd_by_batch<T, V, 64, 1, AFF>(rb);
-  if (tpr == 64 && vpt == 2) return bwd_by_batch<T, V, 64, 2, AFF>(rb);
-  if (tpr == 0 && vpt == 2) return bwd_by_batch<T, V, 0, 2, AFF>(rb);
-  if (tpr == 0 && vpt == 4) return bwd_by_batch<T, V, 0, 4, AFF>(rb);
-  if constexpr (AFF) {
-    if (tpr == 0 && vpt == 8) return bwd_by_batch<T, V, 0, 8, AFF>(rb);
-  }
+BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact) {
+  if (tpr == 8) return bwd_variant<T, V, 8, 1, AFF>(rb, exact);
+  if (tpr == 16) return bwd_variant<T, V, 16, 1, AFF>(rb, exact);
+  if (tpr == 32) return bwd_variant<T, V, 32, 1, AFF>(rb, exact);
+  if (tpr == 64 && vpt == 1) return bwd_variant<T, V, 64, 1, AFF>(rb, exact);
+  if (tpr == 64 && vpt == 2) return bwd_variant<T, V, 64, 2, AFF>(rb, exact);
+  if (tpr == 0 && vpt == 2) return bwd_variant<T, V, 0, 2, AFF>(rb, exact);
+  if (tpr == 0 && vpt == 4) return bwd_variant<T, V, 0, 4, AFF>(rb, exact);
   return nullptr;
 }
 
@@ -69,7 +72,7 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && (p.ws_bytes == 0 || ws != nullptr),
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   if (p.resident) {
-    auto fn = pick_fwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb);
+    auto fn = pick_fwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident forward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
     fn<<<p.grid, p.threads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows,
                                      static_cast<int>(D / V), C, eps);
@@ -96,7 +99,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_part);
   const int64_t W = AFF ? C : D;
   if (p.resident) {
-    auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb);
+    auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
     const int stages = tuning().bwd_stage_mask;
     if (stages & 1) {
