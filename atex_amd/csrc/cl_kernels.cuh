@@ -7,8 +7,12 @@
 // DivUp(C,32) x ppr x N blocks).  Here a lane owns one 128-bit vector of V adjacent
 // channels, TPP lanes cover a pixel, and a block of 256 threads sweeps 256 / TPP pixels
 // per step, so every wave-load is a contiguous 1 KiB.  The spatial extent of one
-// instance is cut into S slabs, one block per (n, slab, channel tile):
-//   stage 1 writes per-slab per-channel partials, stage 2 merges them and applies.
+// instance is cut into S slabs, one block per (instance, slab, channel tile), two launches:
+//   stage 1  per-slab per-channel partial sums -> workspace
+//   stage 2  every block first folds the S partials of its instance and channel tile
+//            (a few KiB from L2) into LDS, then applies; no separate finalize launch.
+// Small slabs stay in registers between their (single, fully overlapped) batch of loads
+// and their use.
 #pragma once
 
 #include "norm_common.cuh"
@@ -16,310 +20,566 @@
 namespace atexn {
 
 constexpr int kClThreads = 256;
+constexpr int kClMaxTileChannels = 2048;  // 256 lanes x 8 channels
 
-// Thread geometry.  TPP: threads per pixel (power of two, <= 256).
+// Thread geometry.  TPP: threads per pixel (power of two, <= 256; tpp_shift = log2 TPP).
+// The grid is (instances, slabs, channel tiles): the instance is the fastest-varying block
+// coordinate so that, with workgroups dealt round-robin to the XCDs, the slabs of one
+// instance share an XCD and its L2 whenever N is a multiple of the XCD count.
 struct ClGeom {
-  int64_t n;      // instance
-  int s;          // slab
-  int cvi;        // channel-vector index of this thread
-  int slot;       // pixel slot inside the block
-  int ppb;        // pixel slots per block
-  bool ch_ok;     // channel vector inside C
-  int64_t p0, p1; // pixel range of the slab
+  int64_t n;       // instance
+  int s;           // slab
+  int ct;          // channel tile
+  int cvi;         // channel-vector index of this thread
+  int slot;        // pixel slot inside the block
+  int ppb;         // pixel slots per block
+  bool ch_ok;      // channel vector inside C
+  int64_t p0, p1;  // pixel range of the slab
 };
 
-__device__ __forceinline__ ClGeom cl_geom(int64_t work, int S, int CT, int TPP, int CV,
-                                          int64_t D, int64_t slab_len) {
+__device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int64_t D, int64_t slab_len) {
   ClGeom g;
-  const int ct = static_cast<int>(work % CT);
-  const int64_t ns = work / CT;
-  g.s = static_cast<int>(ns % S);
-  g.n = ns / S;
-  g.cvi = ct * TPP + static_cast<int>(threadIdx.x) % TPP;
-  g.slot = static_cast<int>(threadIdx.x) / TPP;
-  g.ppb = kClThreads / TPP;
+  g.n = blockIdx.x;
+  g.s = static_cast<int>(blockIdx.y);
+  g.ct = static_cast<int>(blockIdx.z);
+  const int t = static_cast<int>(threadIdx.x);
+  g.cvi = (g.ct << tpp_shift) | (t & ((1 << tpp_shift) - 1));
+  g.slot = t >> tpp_shift;
+  g.ppb = kClThreads >> tpp_shift;
   g.ch_ok = g.cvi < CV;
   g.p0 = static_cast<int64_t>(g.s) * slab_len;
   g.p1 = g.p0 + slab_len < D ? g.p0 + slab_len : D;
   return g;
 }
 
+// v + v of the lane whose id differs in bit M: VALU cross-lane forms where the ISA has
+// one (quad permutes, row rotate by 8, the 16- and 32-lane swaps), the LDS crossbar
+// otherwise.  Symmetric, so both partners end with the same bits.
+template <int M>
+__device__ __forceinline__ float xor_add(float v) {
+  if constexpr (M == 1) return v + dpp_read<kDppQuadXor1>(v);
+  if constexpr (M == 2) return v + dpp_read<kDppQuadXor2>(v);
+  if constexpr (M == 4) return v + lane_xor(v, 4);
+  if constexpr (M == 8) return v + dpp_read<0x128>(v);  // row_ror:8
+  if constexpr (M == 16) return swap_add<16>(v);
+  if constexpr (M == 32) return swap_add<32>(v);
+}
+
+// Sum over the lanes of a wave that own the same channels (lane ids equal modulo TPP0),
+// for K values at once; TPP0 is a compile-time power of two <= 32.
+template <int K, int TPP0>
+__device__ __forceinline__ void strided_wave_sum(float (&v)[K]) {
+#pragma unroll
+  for (int i = 0; i < K; ++i) {
+    float t = v[i];
+    if constexpr (TPP0 <= 1) t = xor_add<1>(t);
+    if constexpr (TPP0 <= 2) t = xor_add<2>(t);
+    if constexpr (TPP0 <= 4) t = xor_add<4>(t);
+    if constexpr (TPP0 <= 8) t = xor_add<8>(t);
+    if constexpr (TPP0 <= 16) t = xor_add<16>(t);
+    if constexpr (TPP0 <= 32) t = xor_add<32>(t);
+    v[i] = t;
+  }
+}
+
 // Sum K per-thread values over all threads of the block that own the same channels
 // (same threadIdx.x % TPP).  Every such thread ends with the same total, added in a
-// fixed order.  lds: K * 256 floats.  Ends with a barrier-protected state: the caller
-// must __syncthreads() before reusing lds.
+// fixed order.  lds: K * 256 floats; the caller must __syncthreads() before reusing it.
 template <int K>
 __device__ __forceinline__ void cl_block_sum(float (&v)[K], float* lds, int TPP) {
-  for (int m = TPP; m < kWave; m <<= 1) {
-#pragma unroll
-    for (int i = 0; i < K; ++i) v[i] += lane_xor(v[i], m);
+  switch (TPP) {  // one uniform branch; threads per pixel is a power of two
+    case 1: strided_wave_sum<K, 1>(v); break;
+    case 2: strided_wave_sum<K, 2>(v); break;
+    case 4: strided_wave_sum<K, 4>(v); break;
+    case 8: strided_wave_sum<K, 8>(v); break;
+    case 16: strided_wave_sum<K, 16>(v); break;
+    case 32: strided_wave_sum<K, 32>(v); break;
+    default: break;  // 64 and up: a wave holds every channel vector at most once
   }
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
   constexpr int NW = kClThreads / kWave;
-  const int wpc = TPP > kWave ? TPP / kWave : 1;  // waves per channel sweep
-  if (wpc == NW) return;                           // TPP == 256: nothing to fold
+  if (TPP == kClThreads) return;  // every thread owns its channels alone
 #pragma unroll
   for (int i = 0; i < K; ++i) lds[(i * NW + wave) * kWave + lane] = v[i];
   __syncthreads();
+  if (TPP <= kWave) {  // every wave holds the same channel vectors: sum all NW of them
 #pragma unroll
-  for (int i = 0; i < K; ++i) {
-    float s = lds[(i * NW + (wave % wpc)) * kWave + lane];
-    for (int w = (wave % wpc) + wpc; w < NW; w += wpc) s += lds[(i * NW + w) * kWave + lane];
-    v[i] = s;
+    for (int i = 0; i < K; ++i) {
+      float s = lds[(i * NW) * kWave + lane];
+#pragma unroll
+      for (int w = 1; w < NW; ++w) s += lds[(i * NW + w) * kWave + lane];
+      v[i] = s;
+    }
+  } else {  // TPP == 128: waves w and w + 2 share channel vectors
+#pragma unroll
+    for (int i = 0; i < K; ++i) {
+      v[i] = lds[(i * NW + (wave & 1)) * kWave + lane] + lds[(i * NW + (wave & 1) + 2) * kWave + lane];
+    }
   }
 }
 
-// Same for per-channel Welford triples (V channels sharing one count).  lds: (2V+1)*256.
-template <int V>
-__device__ __forceinline__ void cl_block_wf(float (&mean)[V], float (&m2)[V], float& cnt,
-                                            float* lds, int TPP) {
-  for (int m = TPP; m < kWave; m <<= 1) {
-    const float ocnt = lane_xor(cnt, m);
-    float ncnt = cnt;
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      Wf a{mean[i], m2[i], cnt};
-      Wf b{lane_xor(mean[i], m), lane_xor(m2[i], m), ocnt};
-      Wf r = wf_merge(a, b);
-      mean[i] = r.mean;
-      m2[i] = r.m2;
-      ncnt = r.n;
-    }
-    cnt = ncnt;
+// How the threads of a block split the fold over S partial rows for the channels of a
+// tile of `cap` channels (cap = TPP * V, a power of two): P adjacent lanes per channel
+// when the tile has at most 256 channels, else one lane per channel and several sweeps.
+struct FoldMap {
+  int P;       // lanes per channel (power of two, <= 64)
+  int sweeps;  // passes over the tile when it has more channels than threads
+};
+__device__ __forceinline__ FoldMap fold_map(int cap) {
+  FoldMap m;
+  if (cap >= kClThreads) {
+    m.P = 1;
+    m.sweeps = cap / kClThreads;
+  } else {
+    m.P = kClThreads / cap < kWave ? kClThreads / cap : kWave;
+    m.sweeps = 1;
   }
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  constexpr int NW = kClThreads / kWave;
-  const int wpc = TPP > kWave ? TPP / kWave : 1;
-  if (wpc == NW) return;
+  return m;
+}
+
+// Loops over strided indices are written in batches of B whose loads are all issued before
+// the first is consumed: the compiler does not move a load above the bounds check of the
+// iteration before it, so a plain loop would pay one memory latency per iteration.
+template <int B, typename Full, typename Tail>
+__device__ __forceinline__ void batched_for(int64_t first, int64_t end, int64_t step, Full&& full,
+                                            Tail&& tail) {
+  int64_t p = first;
+  for (; p + (B - 1) * step < end; p += B * step) full(p, step);
+  for (; p < end; p += step) tail(p);
+}
+template <int B, typename Full, typename Tail>
+__device__ __forceinline__ void cl_for_pixels(const ClGeom& g, Full&& full, Tail&& tail) {
+  batched_for<B>(g.p0 + g.slot, g.p1, g.ppb, full, tail);
+}
+
+// Resident slabs (U > 0): a thread holds the U pixels of its slot as raw vectors.  Loads
+// are unconditional so that they are all in flight at once: a lane whose pixel or channel
+// vector lies outside the slab reads the slab's first pixel / the last channel vector
+// instead (always valid memory) and is masked out of the arithmetic.
+template <typename T, int V, int U>
+__device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, int CV, int C,
+                                             Pack<T, V> (&raw)[U], bool (&ok)[U]) {
+  const T* b = base_n + static_cast<int64_t>(g.ch_ok ? g.cvi : CV - 1) * V;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    const int64_t p = g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb;
+    ok[u] = g.ch_ok && p < g.p1;
+    raw[u] = load_pack<T, V>(b + (p < g.p1 ? p : g.p0) * C);
+  }
+}
+
+// Pivot of an instance, per channel: the median of the channel's values at the first, the
+// middle and the last pixel.  Forward statistics are accumulated as sum(x - K) and
+// sum((x - K)^2) around this pivot K, which every slab of the instance shares, so slabs
+// (and threads) combine by plain addition, and
+//     mean = K + S1 / D,   var = S2 / D - (S1 / D)^2
+// loses only a factor (1 + (K - mean)^2 / var) of precision; the median of three samples
+// keeps K within the bulk of the data even when one sample is an outlier.
+template <typename T, int V>
+__device__ __forceinline__ void cl_pivot(const T* xn_c, int64_t D, int C, float (&k)[V]) {
+  const Pack<T, V> a = load_pack<T, V>(xn_c);
+  const Pack<T, V> b = load_pack<T, V>(xn_c + (D / 2) * C);
+  const Pack<T, V> c = load_pack<T, V>(xn_c + (D - 1) * C);
 #pragma unroll
   for (int i = 0; i < V; ++i) {
-    lds[((2 * i) * NW + wave) * kWave + lane] = mean[i];
-    lds[((2 * i + 1) * NW + wave) * kWave + lane] = m2[i];
+    k[i] = __builtin_amdgcn_fmed3f(to_f32(a.v[i]), to_f32(b.v[i]), to_f32(c.v[i]));
   }
-  lds[((2 * V) * NW + wave) * kWave + lane] = cnt;
-  __syncthreads();
-  const int w0 = wave % wpc;
-  float c0 = lds[((2 * V) * NW + w0) * kWave + lane];
-  float cend = c0;
-#pragma unroll
-  for (int i = 0; i < V; ++i) {
-    Wf r{lds[((2 * i) * NW + w0) * kWave + lane], lds[((2 * i + 1) * NW + w0) * kWave + lane], c0};
-    for (int w = w0 + wpc; w < NW; w += wpc) {
-      Wf o{lds[((2 * i) * NW + w) * kWave + lane], lds[((2 * i + 1) * NW + w) * kWave + lane],
-           lds[((2 * V) * NW + w) * kWave + lane]};
-      r = wf_merge(r, o);
-    }
-    mean[i] = r.mean;
-    m2[i] = r.m2;
-    cend = r.n;
-  }
-  cnt = cend;
 }
 
 // ---------------------------------------------------------------- forward, stage 1
-// pmean / pm2: [N * S, C] partial mean and sum of squared deviations of each slab.
-template <typename T, int V>
-__global__ void cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pmean,
-                             float* __restrict__ pm2, int64_t n_work, int64_t D, int C, int S,
-                             int CT, int TPP, int64_t slab_len) {
-  __shared__ float lds[(2 * V + 1) * kClThreads];
+// ps1 / ps2: [N * S, C] sums of (x - K) and (x - K)^2 over each slab, K = cl_pivot, which
+// is saved to pivot[N, C].
+// U > 0: the slab is register-resident (slab_len <= U * pixel slots per block) and all its
+// loads are in flight at once; U == 0 streams the slab in batches.
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict__ ps2,
+             float* __restrict__ pivot, int64_t D, int C, int S, int tpp_shift,
+             int64_t slab_len) {
+  __shared__ float lds[2 * V * kClThreads];
   const int CV = (C + V - 1) / V;
-  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
-    const ClGeom g = cl_geom(w, S, CT, TPP, CV, D, slab_len);
-    float mean[V], m2[V], cnt = 0.f;
+  const int TPP = 1 << tpp_shift;
+  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  const T* xn = x + (g.n * D) * C;
+  float k0[V];
+  cl_pivot<T, V>(xn + static_cast<int64_t>(g.ch_ok ? g.cvi : CV - 1) * V, D, C, k0);
+  float acc[2 * V];
 #pragma unroll
-    for (int i = 0; i < V; ++i) mean[i] = m2[i] = 0.f;
-    if (g.ch_ok) {
-      const T* base = x + (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
-      for (int64_t p = g.p0 + g.slot; p < g.p1; p += g.ppb) {
-        Pack<T, V> pk = load_pack<T, V>(base + p * C);
-        cnt += 1.f;
-        const float inv = 1.0f / cnt;
+  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
+  auto add = [&](const Pack<T, V>& pk, bool valid) {
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float f = to_f32(pk.v[i]);
-          const float d = f - mean[i];
-          mean[i] += d * inv;
-          m2[i] += d * (f - mean[i]);
-        }
-      }
+    for (int i = 0; i < V; ++i) {
+      const float d = valid ? to_f32(pk.v[i]) - k0[i] : 0.f;
+      acc[i] += d;
+      acc[V + i] += d * d;
     }
-    cl_block_wf<V>(mean, m2, cnt, lds, TPP);
-    if (g.ch_ok && g.slot == 0) {
-      const int64_t o = (g.n * S + g.s) * C + static_cast<int64_t>(g.cvi) * V;
-      store_f32<V>(pmean + o, mean);
-      store_f32<V>(pm2 + o, m2);
+  };
+  if constexpr (U > 0) {
+    Pack<T, V> raw[U];
+    bool ok[U];
+    cl_load_slab<T, V, U>(xn, g, CV, C, raw, ok);
+#pragma unroll
+    for (int u = 0; u < U; ++u) add(raw[u], ok[u]);
+  } else if (g.ch_ok) {
+    const T* base = xn + static_cast<int64_t>(g.cvi) * V;
+    constexpr int B = 8;
+    cl_for_pixels<B>(
+        g,
+        [&](int64_t p, int64_t step) {
+          Pack<T, V> pk[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(base + (p + u * step) * C);
+#pragma unroll
+          for (int u = 0; u < B; ++u) add(pk[u], true);
+        },
+        [&](int64_t p) { add(load_pack<T, V>(base + p * C), true); });
+  }
+  cl_block_sum<2 * V>(acc, lds, TPP);
+  if (g.ch_ok && g.slot == 0) {
+    float t1[V], t2[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      t1[i] = acc[i];
+      t2[i] = acc[V + i];
     }
-    __syncthreads();  // lds is reused by the next work item
+    const int64_t o = (g.n * S + g.s) * C + static_cast<int64_t>(g.cvi) * V;
+    store_f32<V>(ps1 + o, t1);
+    store_f32<V>(ps2 + o, t2);
+    // stage 2 must not re-read the pivot from x: y may alias x and be half written by then
+    if (g.s == 0) store_f32<V>(pivot + g.n * C + static_cast<int64_t>(g.cvi) * V, k0);
   }
 }
 
 // ---------------------------------------------------------------- forward, stage 2
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
-template <typename T, int V>
-__global__ void cl_fwd_apply(const T* x, const float* __restrict__ pmean,
-                             const float* __restrict__ pm2, const float* __restrict__ gamma,
-                             const float* __restrict__ beta, T* y,
-                             float* __restrict__ mean_out, float* __restrict__ rstd_out,
-                             int64_t n_work, int64_t D, int C, int S, int CT, int TPP,
-                             int64_t slab_len, float eps) {
-  __shared__ float lds[(2 * V + 1) * kClThreads];
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict__ ps2,
+             const float* __restrict__ pivot, const float* __restrict__ gamma,
+             const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
+             float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
+             int64_t slab_len, float eps) {
+  __shared__ float sm_mean[kClMaxTileChannels];
+  __shared__ float sm_rstd[kClMaxTileChannels];
   const int CV = (C + V - 1) / V;
-  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
-    const ClGeom g = cl_geom(w, S, CT, TPP, CV, D, slab_len);
-    float mean[V], m2[V], cnt = 0.f;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const FoldMap fm = fold_map(cap);
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  // resident slab: its loads are issued first and fly while the partials are folded
+  Pack<T, V> raw[U > 0 ? U : 1];
+  bool ok[U > 0 ? U : 1];
+  if constexpr (U > 0) cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  // phase A: add up the S slab partials of every channel of the tile, finish the
+  // statistics around the pivot
+  const int c_base = g.ct * cap;
+  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
+    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
+    const int sub = static_cast<int>(threadIdx.x) % fm.P;
+    const int c = c_base + cl;
+    const bool in = cl < cap && c < C;
+    float s1 = 0.f, s2 = 0.f, kc = 0.f;
+    if (in) {
+      const float* q1 = ps1 + (g.n * S) * C + c;
+      const float* q2 = ps2 + (g.n * S) * C + c;
+      if (sub == 0) kc = pivot[g.n * C + c];
+      constexpr int B = 16;
+      batched_for<B>(
+          sub, S, fm.P,
+          [&](int64_t sl, int64_t step) {
+            float t1[B], t2[B];
 #pragma unroll
-    for (int i = 0; i < V; ++i) mean[i] = m2[i] = 0.f;
-    if (g.ch_ok) {
-      // every pixel slot merges its share of the slab partials
-      for (int s = g.slot; s < S; s += g.ppb) {
-        const int64_t o = (g.n * S + s) * C + static_cast<int64_t>(g.cvi) * V;
-        const int64_t b0 = static_cast<int64_t>(s) * slab_len;
-        const float len = static_cast<float>((b0 + slab_len < D ? b0 + slab_len : D) - b0);
-        float pm[V], pq[V];
-        load_f32<V>(pmean + o, pm);
-        load_f32<V>(pm2 + o, pq);
+            for (int u = 0; u < B; ++u) {
+              t1[u] = q1[(sl + u * step) * C];
+              t2[u] = q2[(sl + u * step) * C];
+            }
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          Wf r = wf_merge(Wf{mean[i], m2[i], cnt}, Wf{pm[i], pq[i], len});
-          mean[i] = r.mean;
-          m2[i] = r.m2;
-        }
-        cnt += len;
+            for (int u = 0; u < B; ++u) {
+              s1 += t1[u];
+              s2 += t2[u];
+            }
+          },
+          [&](int64_t sl) {
+            s1 += q1[sl * C];
+            s2 += q2[sl * C];
+          });
+    }
+    for (int m = 1; m < fm.P; m <<= 1) {
+      s1 += lane_xor(s1, m);
+      s2 += lane_xor(s2, m);
+    }
+    if (sub == 0 && in) {
+      const float dm = s1 * inv_d;
+      const float mean = kc + dm;
+      const float var = fmaxf(s2 * inv_d - dm * dm, 0.f);
+      const float rs = rsqrtf(var + eps);
+      sm_mean[cl] = mean;
+      sm_rstd[cl] = rs;
+      if (g.s == 0) {
+        mean_out[g.n * C + c] = mean;
+        rstd_out[g.n * C + c] = rs;
       }
     }
-    cl_block_wf<V>(mean, m2, cnt, lds, TPP);
-    if (g.ch_ok) {
-      float gm[V], bt[V], rs[V];
-      load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, gm);
-      load_f32<V>(beta + static_cast<int64_t>(g.cvi) * V, bt);
+  }
+  __syncthreads();
+  // phase B: apply
+  if (g.ch_ok) {
+    const int cl0 = (g.cvi - (g.ct << tpp_shift)) * V;
+    float mean[V], sc[V], bt[V];
+    load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, sc);
+    load_f32<V>(beta + static_cast<int64_t>(g.cvi) * V, bt);
 #pragma unroll
-      for (int i = 0; i < V; ++i) rs[i] = rsqrtf(m2[i] / static_cast<float>(D) + eps);
-      if (g.s == 0 && g.slot == 0) {
-        store_f32<V>(mean_out + g.n * C + static_cast<int64_t>(g.cvi) * V, mean);
-        store_f32<V>(rstd_out + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
-      }
-      const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
-      for (int64_t p = g.p0 + g.slot; p < g.p1; p += g.ppb) {
-        Pack<T, V> pk = load_pack<T, V>(x + boff + p * C);
-        Pack<T, V> o;
-#pragma unroll
-        for (int i = 0; i < V; ++i) {
-          // subtract the mean first: x * scale - mean * scale would cancel badly when
-          // |mean| >> std
-          o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * rs[i] * gm[i] + bt[i]);
-        }
-        store_pack<T, V>(y + boff + p * C, o);
-      }
+    for (int i = 0; i < V; ++i) {
+      mean[i] = sm_mean[cl0 + i];
+      sc[i] *= sm_rstd[cl0 + i];
     }
-    __syncthreads();
+    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    auto apply = [&](const Pack<T, V>& pk, int64_t p) {
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        // subtract the mean first: x * scale - mean * scale would cancel badly when
+        // |mean| >> std
+        o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * sc[i] + bt[i]);
+      }
+      store_pack<T, V>(y + boff + p * C, o);
+    };
+    if constexpr (U > 0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (ok[u]) apply(raw[u], g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb);
+      }
+    } else {
+      constexpr int B = 8;
+      cl_for_pixels<B>(
+          g,
+          [&](int64_t p, int64_t step) {
+            Pack<T, V> pk[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
+#pragma unroll
+            for (int u = 0; u < B; ++u) apply(pk[u], p + u * step);
+          },
+          [&](int64_t p) { apply(load_pack<T, V>(x + boff + p * C), p); });
+    }
   }
 }
 
 // --------------------------------------------------------------- backward, stage 1
 // part[(n * S + s)][0][c] = sum dy * xh, part[...][1][c] = sum dy over the slab.
-template <typename T, int V>
-__global__ void cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
-                            const float* __restrict__ mean_in,
-                            const float* __restrict__ rstd_in, float* __restrict__ part,
-                            int64_t n_work, int64_t D, int C, int S, int CT, int TPP,
-                            int64_t slab_len) {
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
+            const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+            float* __restrict__ part, int64_t D, int C, int S, int tpp_shift,
+            int64_t slab_len) {
   __shared__ float lds[2 * V * kClThreads];
   const int CV = (C + V - 1) / V;
-  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
-    const ClGeom g = cl_geom(w, S, CT, TPP, CV, D, slab_len);
-    float acc[2 * V];
+  const int TPP = 1 << tpp_shift;
+  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  float acc[2 * V];
 #pragma unroll
-    for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
-    if (g.ch_ok) {
-      float mu[V], rs[V];
-      load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
-      load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
-      const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
-      for (int64_t p = g.p0 + g.slot; p < g.p1; p += g.ppb) {
-        Pack<T, V> px = load_pack<T, V>(x + boff + p * C);
-        Pack<T, V> pd = load_pack<T, V>(dy + boff + p * C);
+  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
+  Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
+  bool ok[U > 0 ? U : 1];
+  if constexpr (U > 0) {
+    cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
+    cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+  }
+  float mu[V], rs[V];
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float d = to_f32(pd.v[i]);
-          const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
-          acc[i] += d * xh;
-          acc[V + i] += d;
-        }
-      }
+  for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
+  if (g.ch_ok) {
+    load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
+    load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
+  }
+  auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, bool valid) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = valid ? to_f32(pd.v[i]) : 0.f;
+      const float xh = valid ? (to_f32(px.v[i]) - mu[i]) * rs[i] : 0.f;
+      acc[i] += d * xh;
+      acc[V + i] += d;
     }
-    cl_block_sum<2 * V>(acc, lds, TPP);
-    if (g.ch_ok && g.slot == 0) {
-      float* o = part + ((g.n * S + g.s) * 2) * C + static_cast<int64_t>(g.cvi) * V;
-      float t0[V], t1[V];
+  };
+  if constexpr (U > 0) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) {
-        t0[i] = acc[i];
-        t1[i] = acc[V + i];
-      }
-      store_f32<V>(o, t0);
-      store_f32<V>(o + C, t1);
+    for (int u = 0; u < U; ++u) add(rx[u], rd[u], ok[u]);
+  } else if (g.ch_ok) {
+    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    constexpr int B = 4;
+    cl_for_pixels<B>(
+        g,
+        [&](int64_t p, int64_t step) {
+          Pack<T, V> px[B], pd[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
+            pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) add(px[u], pd[u], true);
+        },
+        [&](int64_t p) {
+          add(load_pack<T, V>(x + boff + p * C), load_pack<T, V>(dy + boff + p * C), true);
+        });
+  }
+  cl_block_sum<2 * V>(acc, lds, TPP);
+  if (g.ch_ok && g.slot == 0) {
+    float* o = part + ((g.n * S + g.s) * 2) * C + static_cast<int64_t>(g.cvi) * V;
+    float t0[V], t1[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      t0[i] = acc[i];
+      t1[i] = acc[V + i];
     }
-    __syncthreads();
+    store_f32<V>(o, t0);
+    store_f32<V>(o + C, t1);
   }
 }
 
 // --------------------------------------------------------------- backward, stage 2
 // dx = r * gamma * (dy - (A + xh * B) / D) with A = sum dy, B = sum dy * xh over the
-// whole (n, c) instance (norm_util.h:599-615 in s1 / s2 form).
-template <typename T, int V>
-__global__ void cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x,
-                             const float* __restrict__ gamma,
-                             const float* __restrict__ mean_in,
-                             const float* __restrict__ rstd_in,
-                             const float* __restrict__ part, T* __restrict__ dx,
-                             int64_t n_work, int64_t D, int C, int S, int CT, int TPP,
-                             int64_t slab_len) {
-  __shared__ float lds[2 * V * kClThreads];
+// whole (n, c) instance (norm_util.h:599-615 in s1 / s2 form).  Every block first folds
+// the S slab partials of its instance and channel tile into LDS.  The 2 C outputs of
+// dgamma / dbeta are dealt out over the blocks, each a block-wide sum of one column of
+// all N * S partial rows (fixed order, no atomics), which spares a third launch.
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
+             const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
+             const float* __restrict__ part, T* __restrict__ dx, float* __restrict__ dgamma,
+             float* __restrict__ dbeta, int64_t N, int64_t D, int C, int S, int tpp_shift,
+             int64_t slab_len) {
+  __shared__ float sm_a[kClMaxTileChannels];  // sum dy
+  __shared__ float sm_b[kClMaxTileChannels];  // sum dy * xh
+  __shared__ float red_buf[2][16];
   const int CV = (C + V - 1) / V;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
-  for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
-    const ClGeom g = cl_geom(w, S, CT, TPP, CV, D, slab_len);
-    float acc[2 * V];
+  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  // resident slab: its loads are issued first and fly while the partials are folded
+  Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
+  bool okp[U > 0 ? U : 1];
+  if constexpr (U > 0) {
+    cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, okp);
+    cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, okp);
+  }
+  const int c_base = g.ct * cap;
+  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
+    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;
+    const int sub = static_cast<int>(threadIdx.x) % fm.P;
+    const int c = c_base + cl;
+    const bool in = cl < cap && c < C;
+    float a = 0.f, b = 0.f;
+    if (in) {
+      const float* pr = part + ((g.n * S) * 2) * C + c;
+      constexpr int B = 16;
+      batched_for<B>(
+          sub, S, fm.P,
+          [&](int64_t sl, int64_t step) {
+            float tb[B], ta[B];
 #pragma unroll
-    for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
-    if (g.ch_ok) {
-      for (int s = g.slot; s < S; s += g.ppb) {
-        const float* o = part + ((g.n * S + s) * 2) * C + static_cast<int64_t>(g.cvi) * V;
-        float t0[V], t1[V];
-        load_f32<V>(o, t0);
-        load_f32<V>(o + C, t1);
+            for (int u = 0; u < B; ++u) {
+              tb[u] = pr[((sl + u * step) * 2) * C];
+              ta[u] = pr[((sl + u * step) * 2 + 1) * C];
+            }
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          acc[i] += t0[i];
-          acc[V + i] += t1[i];
-        }
-      }
+            for (int u = 0; u < B; ++u) {
+              b += tb[u];
+              a += ta[u];
+            }
+          },
+          [&](int64_t sl) {
+            b += pr[(sl * 2) * C];
+            a += pr[(sl * 2 + 1) * C];
+          });
     }
-    cl_block_sum<2 * V>(acc, lds, TPP);
-    if (g.ch_ok) {
-      float mu[V], rs[V], gm[V];
-      load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
-      load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
-      load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, gm);
-      const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
-      for (int64_t p = g.p0 + g.slot; p < g.p1; p += g.ppb) {
-        Pack<T, V> px = load_pack<T, V>(x + boff + p * C);
-        Pack<T, V> pd = load_pack<T, V>(dy + boff + p * C);
-        Pack<T, V> o;
-#pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float d = to_f32(pd.v[i]);
-          const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
-          o.v[i] = from_f32<T>(rs[i] * gm[i] * (d - (acc[V + i] + xh * acc[i]) * inv_d));
-        }
-        store_pack<T, V>(dx + boff + p * C, o);
-      }
+    for (int m = 1; m < fm.P; m <<= 1) {
+      a += lane_xor(a, m);
+      b += lane_xor(b, m);
     }
-    __syncthreads();
+    if (sub == 0 && in) {
+      sm_a[cl] = a;
+      sm_b[cl] = b;
+    }
+  }
+  // dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C]) is the sum of one column
+  // of all N * S partial rows; block w of the grid takes outputs w, w + #blocks, ...
+  const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
+  const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  int red_it = 0;
+  for (int64_t o = w; o < 2 * static_cast<int64_t>(C); o += n_blocks) {
+    const int which = o < C ? 0 : 1;
+    const int c = static_cast<int>(o < C ? o : o - C);
+    const int64_t rows = N * S;
+    float t = 0.f;
+    const float* pc = part + static_cast<int64_t>(which) * C + c;
+    batched_for<4>(
+        threadIdx.x, rows, kClThreads,
+        [&](int64_t r, int64_t step) {
+          float v[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[u] = pc[((r + u * step) * 2) * C];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) t += v[u];
+        },
+        [&](int64_t r) { t += pc[(r * 2) * C]; });
+    t = block_sum1(t, red_buf[red_it & 1]);
+    ++red_it;
+    if (threadIdx.x == 0) (which == 0 ? dgamma : dbeta)[c] = t;
+  }
+  __syncthreads();
+  if (g.ch_ok) {
+    const int cl0 = (g.cvi - (g.ct << tpp_shift)) * V;
+    float mu[V], rs[V], sc[V], ca[V], cb[V];
+    load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
+    load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
+    load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, sc);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      sc[i] *= rs[i];
+      ca[i] = -sc[i] * (sm_b[cl0 + i] * inv_d);
+      cb[i] = -sc[i] * (sm_a[cl0 + i] * inv_d);
+    }
+    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    auto apply = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t p) {
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
+        o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * xh + cb[i]));
+      }
+      store_pack<T, V>(dx + boff + p * C, o);
+    };
+    if constexpr (U > 0) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        if (okp[u]) apply(rx[u], rd[u], g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb);
+      }
+    } else {
+      constexpr int B = 4;
+      cl_for_pixels<B>(
+          g,
+          [&](int64_t p, int64_t step) {
+            Pack<T, V> px[B], pd[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+              px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
+              pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
+            }
+#pragma unroll
+            for (int u = 0; u < B; ++u) apply(px[u], pd[u], p + u * step);
+          },
+          [&](int64_t p) {
+            apply(load_pack<T, V>(x + boff + p * C), load_pack<T, V>(dy + boff + p * C), p);
+          });
+    }
   }
 }
 

@@ -16,14 +16,27 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* pmean = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
   float* pm2 = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_b);
+  float* pivot = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_c);
   const int Ci = static_cast<int>(C);
-  cl_fwd_stats<T, V><<<p.grid, kClThreads, 0, st>>>(x, pmean, pm2, p.n_work, D, Ci, p.S, p.CT,
-                                                   p.TPP, p.slab_len);
-  ATEXN_CHECK_LAUNCH("cl_fwd_stats");
-  cl_fwd_apply<T, V><<<p.grid, kClThreads, 0, st>>>(x, pmean, pm2, gamma, beta, y, mean, rstd,
-                                                   p.n_work, D, Ci, p.S, p.CT, p.TPP, p.slab_len,
-                                                   eps);
-  ATEXN_CHECK_LAUNCH("cl_fwd_apply");
+  ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
+  const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
+#define ATEXN_CL_FWD(U_)                                                                       \
+  do {                                                                                        \
+    cl_fwd_stats<T, V, U_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, D, Ci, p.S,        \
+                                                       p.tpp_shift, p.slab_len);              \
+    ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
+    cl_fwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, gamma, beta, y,    \
+                                                       mean, rstd, D, Ci, p.S, p.tpp_shift,   \
+                                                       p.slab_len, eps);                      \
+    ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \
+  } while (0)
+  if constexpr (V > 1) {
+    if (p.U == 4) { ATEXN_CL_FWD(4); return ATEXN_OK; }
+    if (p.U == 8) { ATEXN_CL_FWD(8); return ATEXN_OK; }
+    if (p.U == 16) { ATEXN_CL_FWD(16); return ATEXN_OK; }
+  }
+  ATEXN_CL_FWD(0);
+#undef ATEXN_CL_FWD
   return ATEXN_OK;
 }
 
@@ -36,13 +49,25 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* part = static_cast<float*>(ws);
   const int Ci = static_cast<int>(C);
-  cl_bwd_sums<T, V><<<p.grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, p.n_work, D, Ci, p.S,
-                                                  p.CT, p.TPP, p.slab_len);
-  ATEXN_CHECK_LAUNCH("cl_bwd_sums");
-  cl_bwd_apply<T, V><<<p.grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx, p.n_work,
-                                                   D, Ci, p.S, p.CT, p.TPP, p.slab_len);
-  ATEXN_CHECK_LAUNCH("cl_bwd_apply");
-  return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N * p.S), C, st);
+  ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
+  const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
+#define ATEXN_CL_BWD(U_)                                                                       \
+  do {                                                                                        \
+    cl_bwd_sums<T, V, U_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S,      \
+                                                      p.tpp_shift, p.slab_len);               \
+    ATEXN_CHECK_LAUNCH("cl_bwd_sums");                                                        \
+    cl_bwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx,      \
+                                                       dgamma, dbeta, N, D, Ci, p.S,          \
+                                                       p.tpp_shift, p.slab_len);              \
+    ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \
+  } while (0)
+  if constexpr (V > 1) {
+    if (p.U == 4) { ATEXN_CL_BWD(4); return ATEXN_OK; }
+    if (p.U == 8) { ATEXN_CL_BWD(8); return ATEXN_OK; }
+  }
+  ATEXN_CL_BWD(0);
+#undef ATEXN_CL_BWD
+  return ATEXN_OK;
 }
 
 template <typename T>

@@ -152,12 +152,14 @@ struct ClPlan {
   int V = 1;
   int CV = 1;    // channel vectors per pixel
   int TPP = 1;   // threads per pixel (power of two <= 256)
+  int tpp_shift = 0;
   int CT = 1;    // channel tiles
   int S = 1;     // slabs per instance
+  int U = 0;     // vectors per thread of a register-resident slab (0: streaming)
   int64_t slab_len = 0;
   int64_t n_work = 0;
   int grid = 1;
-  size_t off_a = 0, off_b = 0, ws_bytes = 0;
+  size_t off_a = 0, off_b = 0, off_c = 0, ws_bytes = 0;
 };
 
 inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
@@ -166,6 +168,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.V = V;
   p.CV = static_cast<int>(div_up(C, V));
   p.TPP = std::min(256, pow2_ceil(p.CV));
+  while ((1 << p.tpp_shift) < p.TPP) ++p.tpp_shift;
   p.CT = static_cast<int>(div_up(p.CV, p.TPP));
   const int ppb = 256 / p.TPP;
   const int64_t want = div_up(int64_t(cus) * t.cl_items_per_cu, std::max<int64_t>(N * p.CT, 1));
@@ -175,11 +178,22 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.S = static_cast<int>(div_up(D, p.slab_len));
   p.n_work = N * p.S * p.CT;
   p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(p.n_work, int64_t(cus) * 32)));
+  // a slab of at most 16 (backward: 8, it holds x and dy) vectors per thread stays in
+  // registers between its load and its use
+  const int64_t per_thread = p.slab_len / ppb;
+  const int max_u = bwd ? 8 : 16;
+  for (int u = 4; u <= max_u; u *= 2) {
+    if (per_thread <= u) {
+      p.U = u;
+      break;
+    }
+  }
   const size_t sect = align256(sizeof(float) * size_t(N) * size_t(p.S) * size_t(C));
   p.off_a = 0;
   p.off_b = sect;
-  p.ws_bytes = 2 * sect;  // fwd: pmean + pm2 ; bwd: part[N*S][2][C] (contiguous, 2 sections)
-  (void)bwd;
+  // fwd: slab sums S1, S2 [N*S, C] and the pivots [N, C]; bwd: part[N*S][2][C] (contiguous)
+  p.off_c = 2 * sect;
+  p.ws_bytes = 2 * sect + align256(sizeof(float) * size_t(N) * size_t(C));
   return p;
 }
 
