@@ -102,6 +102,7 @@ def to_host(t, dtype: str | None = None) -> np.ndarray:
     """torch tensor -> float64 numpy values."""
     import torch
 
+    t = t.detach()
     if t.dtype == torch.bfloat16:
         return O.bf16_bits_to_f32(t.view(torch.int16).cpu().numpy().view(np.uint16)).astype(np.float64)
     return t.cpu().numpy().astype(np.float64)
