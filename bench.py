@@ -51,6 +51,18 @@ CASES = {
     "in3d_ncdhw": ("in", "f16", (2, 32, 128 ** 3, True)),
 }
 DEFAULT_CASE = "ln_bert"
+
+# Bytes between L2 and memory per launch of the kernel(s) the roofline object is quoted on,
+# from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, each scaled by
+# what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE x 2.0,
+# WRITE_SIZE x 1.0).  Summaries: profiles/<case>_hbm_traffic.txt.  Cases without a run: None.
+MEASURED_TRAFFIC = {
+    "ln_bert": 52.78e6,                 # rows_bwd_resident
+    "in2d_nchw": 50.49e6,               # rows_bwd_resident (row-affine)
+    "in2d_nhwc": 33.97e6 + 52.59e6,     # cl_bwd_sums + cl_bwd_apply
+    "in3d_ndhwc": 536.94e6 + 806.31e6,  # cl_bwd_sums + cl_bwd_apply
+    "in3d_ncdhw": 536.77e6 + 805.31e6,  # split_bwd_sums + split_bwd_apply
+}
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
 
@@ -233,6 +245,14 @@ def cpu_baseline(op, dtype, dims, max_seconds=20.0):
     }
 
 
+def roofline_kernel(op, dims):
+    if op == "in" and not dims[3]:
+        return "cl_bwd_sums + cl_bwd_apply (channels-last backward, the whole call)"
+    if op == "in" and dims[2] > 16384:
+        return "split_bwd_sums + split_bwd_apply (backward of rows too long for registers)"
+    return "rows_bwd_resident (backward row kernel: dx and the dgamma / dbeta partials)"
+
+
 def run_case(name, steps, warmup, with_cpu=True):
     op, dtype, dims = CASES[name]
     fb, bb = algorithmic_bytes(op, dtype, dims)
@@ -285,8 +305,8 @@ def run_case(name, steps, warmup, with_cpu=True):
         "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9,
                  "fwd_bwd_hot_cache": (fb + bb) / (ms_step_hot * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": None,
-                     "kernel": "backward row kernel (dx + dgamma/dbeta partials)",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
+                     "kernel": roofline_kernel(op, dims),
                      "us": ms_bwd_main * 1e3},
     }
     if with_cpu:
@@ -301,6 +321,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--case", default=DEFAULT_CASE, choices=sorted(CASES) + ["all"])
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="after the case, run 5 device-to-device copies of 64 MiB (torch's "
+                         "elementwise copy kernel): a kernel of known traffic that scales the "
+                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no cross-GPU exchange; run with --gpus 1")
@@ -315,6 +339,12 @@ def main():
             print(json.dumps(r), flush=True)
         return
     print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu)), flush=True)
+    if args.copy_calibration:
+        src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
+        dst = torch.empty_like(src)
+        for _ in range(5):
+            dst.copy_(src)
+        torch.cuda.synchronize()
 
 
 if __name__ == "__main__":
