@@ -68,9 +68,10 @@ int atexn_abi_version(void) { return kAbiVersion; }
 
 /* Benchmark / tuning hook, not part of the drop-in contract: sets a launch-planning
  * parameter by name for the whole process.  Returns ATEXN_INVALID_ARGUMENT for an unknown
- * name or a value < 1. */
+ * name or a value out of range. */
 int atexn_set_tuning(const char* name, int value) {
-  ATEXN_REQUIRE(name != nullptr && value >= 1, "bad tuning request");
+  ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
+  ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass"), "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_ln_threads")) {
@@ -87,6 +88,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
     t.bwd_stage_mask = value;
+  } else if (!strcmp(name, "reverse_second_pass")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "reverse_second_pass must be 0 or 1");
+    t.reverse_second_pass = value;
   }
   else return set_error(ATEXN_INVALID_ARGUMENT, "unknown tuning parameter '%s'", name);
   return ATEXN_OK;

@@ -138,16 +138,6 @@ __device__ __forceinline__ FoldMap fold_map(int cap) {
   return m;
 }
 
-// Loops over strided indices are written in batches of B whose loads are all issued before
-// the first is consumed: the compiler does not move a load above the bounds check of the
-// iteration before it, so a plain loop would pay one memory latency per iteration.
-template <int B, typename Full, typename Tail>
-__device__ __forceinline__ void batched_for(int64_t first, int64_t end, int64_t step, Full&& full,
-                                            Tail&& tail) {
-  int64_t p = first;
-  for (; p + (B - 1) * step < end; p += B * step) full(p, step);
-  for (; p < end; p += step) tail(p);
-}
 template <int B, typename Full, typename Tail>
 __device__ __forceinline__ void cl_for_pixels(const ClGeom& g, Full&& full, Tail&& tail) {
   batched_for<B>(g.p0 + g.slot, g.p1, g.ppb, full, tail);
@@ -260,7 +250,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
              const float* __restrict__ pivot, const float* __restrict__ gamma,
              const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
              float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
-             int64_t slab_len, float eps) {
+             int64_t slab_len, float eps, int rev) {
   __shared__ float sm_mean[kClMaxTileChannels];
   __shared__ float sm_rstd[kClMaxTileChannels];
   const int CV = (C + V - 1) / V;
@@ -354,16 +344,25 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
       }
     } else {
       constexpr int B = 8;
+      // rev: walk the slab from its last pixel (what stage 1 read last is still cached)
+      const int64_t flip = g.p0 + g.p1 - 1;
       cl_for_pixels<B>(
           g,
           [&](int64_t p, int64_t step) {
             Pack<T, V> pk[B];
+            int64_t q[B];
 #pragma unroll
-            for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
+            for (int u = 0; u < B; ++u) {
+              q[u] = rev ? flip - (p + u * step) : p + u * step;
+              pk[u] = load_pack<T, V>(x + boff + q[u] * C);
+            }
 #pragma unroll
-            for (int u = 0; u < B; ++u) apply(pk[u], p + u * step);
+            for (int u = 0; u < B; ++u) apply(pk[u], q[u]);
           },
-          [&](int64_t p) { apply(load_pack<T, V>(x + boff + p * C), p); });
+          [&](int64_t p) {
+            const int64_t q = rev ? flip - p : p;
+            apply(load_pack<T, V>(x + boff + q * C), q);
+          });
     }
   }
 }
@@ -453,7 +452,7 @@ cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __r
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
              const float* __restrict__ part, T* __restrict__ dx, float* __restrict__ dgamma,
              float* __restrict__ dbeta, int64_t N, int64_t D, int C, int S, int tpp_shift,
-             int64_t slab_len) {
+             int64_t slab_len, int rev) {
   __shared__ float sm_a[kClMaxTileChannels];  // sum dy
   __shared__ float sm_b[kClMaxTileChannels];  // sum dy * xh
   __shared__ float red_buf[2][16];
@@ -564,20 +563,24 @@ cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __r
       }
     } else {
       constexpr int B = 4;
+      const int64_t flip = g.p0 + g.p1 - 1;
       cl_for_pixels<B>(
           g,
           [&](int64_t p, int64_t step) {
             Pack<T, V> px[B], pd[B];
+            int64_t q[B];
 #pragma unroll
             for (int u = 0; u < B; ++u) {
-              px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
-              pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
+              q[u] = rev ? flip - (p + u * step) : p + u * step;
+              px[u] = load_pack<T, V>(x + boff + q[u] * C);
+              pd[u] = load_pack<T, V>(dy + boff + q[u] * C);
             }
 #pragma unroll
-            for (int u = 0; u < B; ++u) apply(px[u], pd[u], p + u * step);
+            for (int u = 0; u < B; ++u) apply(px[u], pd[u], q[u]);
           },
           [&](int64_t p) {
-            apply(load_pack<T, V>(x + boff + p * C), load_pack<T, V>(dy + boff + p * C), p);
+            const int64_t q = rev ? flip - p : p;
+            apply(load_pack<T, V>(x + boff + q * C), load_pack<T, V>(dy + boff + q * C), q);
           });
     }
   }

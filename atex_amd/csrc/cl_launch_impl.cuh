@@ -27,7 +27,8 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
     ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
     cl_fwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, gamma, beta, y,    \
                                                        mean, rstd, D, Ci, p.S, p.tpp_shift,   \
-                                                       p.slab_len, eps);                      \
+                                                       p.slab_len, eps,                       \
+                                                       tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
@@ -58,7 +59,8 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
     ATEXN_CHECK_LAUNCH("cl_bwd_sums");                                                        \
     cl_bwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx,      \
                                                        dgamma, dbeta, N, D, Ci, p.S,          \
-                                                       p.tpp_shift, p.slab_len);              \
+                                                       p.tpp_shift, p.slab_len,               \
+                                                       tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {

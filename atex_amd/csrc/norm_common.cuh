@@ -136,6 +136,16 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// Loops over strided indices are written in batches of B whose loads are all issued before
+// the first is consumed: the compiler does not move a load above the bounds check of the
+// iteration before it, so a plain loop would pay one memory latency per iteration.
+template <int B, typename Full, typename Tail>
+__device__ __forceinline__ void batched_for(int64_t first, int64_t end, int64_t step, Full&& full,
+                                            Tail&& tail) {
+  int64_t p = first;
+  for (; p + (B - 1) * step < end; p += B * step) full(p, step);
+  for (; p < end; p += step) tail(p);
+}
 // Fast reciprocal (v_rcp_f32, 1 ulp): used for counts, which are small integers.
 __device__ __forceinline__ float fast_rcp(float v) { return __builtin_amdgcn_rcpf(v); }
 

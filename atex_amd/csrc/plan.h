@@ -28,6 +28,9 @@ struct Tuning {
   // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
   // bit 1: the final column reduction).  Anything but 3 gives incomplete results.
   int bwd_stage_mask = 3;
+  // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
+  // is what the memory-side cache still holds).
+  int reverse_second_pass = 1;
 };
 Tuning& tuning();
 

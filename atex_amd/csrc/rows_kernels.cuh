@@ -592,30 +592,63 @@ col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __re
 // A row of D elements is cut into S chunks of `chunk` elements (the last may be short).
 // Work item w = row * S + s; blocks take work items grid-stride.  V = elements per
 // access (16-byte vectors when everything is aligned, 1 otherwise).
+//
+// Every loop over a chunk runs in batches of kSplitBatch accesses per thread whose loads are
+// all issued before the first is consumed (a plain strided loop keeps one load per thread
+// in flight, far too little to cover the memory latency at this bandwidth).  The second-
+// stage kernels can walk their chunk backwards: stage 1 ends on the chunk's tail, so the
+// tail is what the memory-side cache still holds when stage 2 starts.
 
+constexpr int kSplitBatch = 4;
+
+// Vector index of virtual position p of a chunk of n_vec vectors.
+__device__ __forceinline__ int64_t split_pos(int64_t p, int64_t n_vec, bool rev) {
+  return rev ? n_vec - 1 - p : p;
+}
+
+// Statistics of a chunk as a Welford triple.  Each thread accumulates sum(x - K) and
+// sum((x - K)^2) around its own pivot K = the first element it owns (two FMAs per element,
+// no division), converts to (mean, m2, n) at the end, and the block merges the threads'
+// triples with Chan's formula.  A thread's pivot is one of its own samples, so the shifted
+// sums lose precision only when that sample is an outlier of the thread's data, and then
+// only in that thread's share.
 template <typename T, int V>
 __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
-  // Streaming Welford: one vector at a time, exact two-pass inside the vector and a
-  // Chan merge into the running triple.
-  Wf run{0.f, 0.f, 0.f};
-  for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
-       i += static_cast<int64_t>(blockDim.x) * V) {
-    Pack<T, V> pk = load_pack<T, V>(p + i);
-    float f[V];
+  const int64_t n_vec = len / V;
+  const int64_t tid = threadIdx.x;
+  if (tid >= n_vec) return Wf{0.f, 0.f, 0.f};
+  const float K = to_f32(p[tid * V]);
+  float s1 = 0.f, s2 = 0.f;
+  int64_t cnt = 0;
+  auto acc = [&](const Pack<T, V>& pk) {
 #pragma unroll
-    for (int k = 0; k < V; ++k) f[k] = to_f32(pk.v[k]);
-    if constexpr (V == 1) {
-      // classic Welford update
-      run.n += 1.f;
-      const float d = f[0] - run.mean;
-      run.mean += d / run.n;
-      run.m2 += d * (f[0] - run.mean);
-    } else {
-      Wf w = local_wf<V>(f, V);
-      run = wf_merge(run, w);
+    for (int k = 0; k < V; ++k) {
+      const float d = to_f32(pk.v[k]) - K;
+      s1 += d;
+      s2 += d * d;
     }
-  }
-  return run;
+  };
+  batched_for<kSplitBatch>(
+      tid, n_vec, blockDim.x,
+      [&](int64_t v, int64_t step) {
+        Pack<T, V> pk[kSplitBatch];
+#pragma unroll
+        for (int u = 0; u < kSplitBatch; ++u) pk[u] = load_pack<T, V>(p + (v + u * step) * V);
+#pragma unroll
+        for (int u = 0; u < kSplitBatch; ++u) acc(pk[u]);
+        cnt += kSplitBatch;
+      },
+      [&](int64_t v) {
+        acc(load_pack<T, V>(p + v * V));
+        cnt += 1;
+      });
+  Wf w;
+  w.n = static_cast<float>(cnt * V);
+  const float inv = 1.0f / w.n;
+  const float dm = s1 * inv;
+  w.mean = K + dm;
+  w.m2 = fmaxf(s2 - s1 * dm, 0.f);
+  return w;
 }
 
 // stage 1 forward: stats[w] = (mean, m2) of chunk w; the count follows from geometry.
@@ -649,13 +682,14 @@ __device__ __forceinline__ Wf merge_chunks(const float2* stats, int S, int64_t D
 
 // stage 2 forward: merge the S chunk statistics of the row, normalise the chunk.
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
-// every thread reads a vector before it writes the same vector.
+// every thread reads its vectors of a batch before it writes the same vectors.
 template <typename T, int V, bool ROW_AFFINE>
 __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
                                 const float* __restrict__ gamma, const float* __restrict__ beta,
                                 T* y, float* __restrict__ mean_out,
                                 float* __restrict__ rstd_out, int64_t n_rows, int64_t D, int S,
-                                int64_t chunk, int C, float eps) {
+                                int64_t chunk, int C, float eps, int rev) {
+  constexpr int B = ROW_AFFINE ? kSplitBatch : 2;  // the per-column gamma / beta take registers
   const int64_t n_work = n_rows * S;
   for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
     const int64_t row = w / S;
@@ -675,28 +709,45 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
     }
     const int64_t beg = static_cast<int64_t>(s) * chunk;
     const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const int64_t n_vec = len / V;
     const T* xp = x + row * D + beg;
     T* yp = y + row * D + beg;
-    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
-         i += static_cast<int64_t>(blockDim.x) * V) {
-      Pack<T, V> pk = load_pack<T, V>(xp + i);
+    const float* gp = gamma + beg;
+    const float* bp = beta + beg;
+    const float a = rstd * gs;  // ROW_AFFINE: y = (x - mean) * a + bs
+    auto one = [&](const Pack<T, V>& pk, int64_t i) {
       Pack<T, V> o;
-      float tg[V], tb[V];
-      if constexpr (!ROW_AFFINE) {
-        load_f32<V>(gamma + beg + i, tg);
-        load_f32<V>(beta + beg + i, tb);
-      }
+      if constexpr (ROW_AFFINE) {
 #pragma unroll
-      for (int k = 0; k < V; ++k) {
-        const float xh = (to_f32(pk.v[k]) - mean) * rstd;
-        if constexpr (ROW_AFFINE) {
-          o.v[k] = from_f32<T>(xh * gs + bs);
-        } else {
-          o.v[k] = from_f32<T>(xh * tg[k] + tb[k]);
+        for (int k = 0; k < V; ++k) o.v[k] = from_f32<T>((to_f32(pk.v[k]) - mean) * a + bs);
+      } else {
+        float tg[V], tb[V];
+        load_f32<V>(gp + i, tg);
+        load_f32<V>(bp + i, tb);
+#pragma unroll
+        for (int k = 0; k < V; ++k) {
+          o.v[k] = from_f32<T>((to_f32(pk.v[k]) - mean) * rstd * tg[k] + tb[k]);
         }
       }
       store_pack<T, V>(yp + i, o);
-    }
+    };
+    batched_for<B>(
+        threadIdx.x, n_vec, blockDim.x,
+        [&](int64_t v, int64_t step) {
+          Pack<T, V> pk[B];
+          int64_t i[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            i[u] = split_pos(v + u * step, n_vec, rev) * V;
+            pk[u] = load_pack<T, V>(xp + i[u]);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) one(pk[u], i[u]);
+        },
+        [&](int64_t v) {
+          const int64_t i = split_pos(v, n_vec, rev) * V;
+          one(load_pack<T, V>(xp + i), i);
+        });
   }
 }
 
@@ -708,6 +759,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
                                const float* __restrict__ mean_in,
                                const float* __restrict__ rstd_in, float2* __restrict__ sums,
                                int64_t n_rows, int64_t D, int S, int64_t chunk) {
+  constexpr int B = ROW_AFFINE ? kSplitBatch : 2;
   __shared__ float2 sum_buf[2][16];
   const int64_t n_work = n_rows * S;
   int it = 0;
@@ -716,26 +768,40 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
     const int s = static_cast<int>(w % S);
     const int64_t beg = static_cast<int64_t>(s) * chunk;
     const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const int64_t n_vec = len / V;
     const float mean = mean_in[row], rstd = rstd_in[row];
     const T* xp = x + row * D + beg;
     const T* dp = dy + row * D + beg;
+    const float* gp = gamma + beg;
+    // accumulate sum g and sum g * x; sum g * xh = rstd * (sum g * x - mean * sum g)
+    // would cancel for |mean| >> 1 / rstd, so x is centred first (one subtraction)
     float s1 = 0.f, s2 = 0.f;
-    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
-         i += static_cast<int64_t>(blockDim.x) * V) {
-      Pack<T, V> px = load_pack<T, V>(xp + i);
-      Pack<T, V> pd = load_pack<T, V>(dp + i);
+    auto one = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t i) {
       float tg[V];
-      if constexpr (!ROW_AFFINE) load_f32<V>(gamma + beg + i, tg);
+      if constexpr (!ROW_AFFINE) load_f32<V>(gp + i, tg);
 #pragma unroll
       for (int k = 0; k < V; ++k) {
-        const float xh = (to_f32(px.v[k]) - mean) * rstd;
+        const float xc = to_f32(px.v[k]) - mean;
         float gv = to_f32(pd.v[k]);
         if constexpr (!ROW_AFFINE) gv *= tg[k];
         s1 += gv;
-        s2 += gv * xh;
+        s2 += gv * xc;
       }
-    }
-    const float2 r = block_sum2(s1, s2, sum_buf[it & 1]);
+    };
+    batched_for<B>(
+        threadIdx.x, n_vec, blockDim.x,
+        [&](int64_t v, int64_t step) {
+          Pack<T, V> px[B], pd[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            px[u] = load_pack<T, V>(xp + (v + u * step) * V);
+            pd[u] = load_pack<T, V>(dp + (v + u * step) * V);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) one(px[u], pd[u], (v + u * step) * V);
+        },
+        [&](int64_t v) { one(load_pack<T, V>(xp + v * V), load_pack<T, V>(dp + v * V), v * V); });
+    const float2 r = block_sum2(s1, s2 * rstd, sum_buf[it & 1]);
     if (threadIdx.x == 0) sums[w] = r;
   }
 }
@@ -749,7 +815,8 @@ __global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ 
                                 const float* __restrict__ rstd_in,
                                 const float2* __restrict__ sums, T* __restrict__ dx,
                                 float* __restrict__ part, int64_t n_rows, int64_t D, int S,
-                                int64_t chunk, int C) {
+                                int64_t chunk, int C, int rev) {
+  constexpr int B = ROW_AFFINE ? kSplitBatch : 2;
   const int64_t n_work = n_rows * S;
   const float inv_d = 1.0f / static_cast<float>(D);
   for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
@@ -774,25 +841,45 @@ __global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ 
     }
     const int64_t beg = static_cast<int64_t>(s) * chunk;
     const int64_t len = (beg + chunk <= D ? chunk : D - beg);
+    const int64_t n_vec = len / V;
     const T* xp = x + row * D + beg;
     const T* dp = dy + row * D + beg;
     T* op = dx + row * D + beg;
-    for (int64_t i = static_cast<int64_t>(threadIdx.x) * V; i < len;
-         i += static_cast<int64_t>(blockDim.x) * V) {
-      Pack<T, V> px = load_pack<T, V>(xp + i);
-      Pack<T, V> pd = load_pack<T, V>(dp + i);
+    const float* gp = gamma + beg;
+    // dx = rstd * gs * (g - s1 / D - xh * s2 / D) = ca * g + cb * (x - mean) + cc
+    const float ca = rstd * gs;
+    const float cb = -ca * s2 * inv_d * rstd;
+    const float cc = -ca * s1 * inv_d;
+    auto one = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t i) {
       Pack<T, V> o;
       float tg[V];
-      if constexpr (!ROW_AFFINE) load_f32<V>(gamma + beg + i, tg);
+      if constexpr (!ROW_AFFINE) load_f32<V>(gp + i, tg);
 #pragma unroll
       for (int k = 0; k < V; ++k) {
-        const float xh = (to_f32(px.v[k]) - mean) * rstd;
         float gv = to_f32(pd.v[k]);
         if constexpr (!ROW_AFFINE) gv *= tg[k];
-        o.v[k] = from_f32<T>(rstd * gs * (gv - (s1 + xh * s2) * inv_d));
+        o.v[k] = from_f32<T>(ca * gv + (cb * (to_f32(px.v[k]) - mean) + cc));
       }
       store_pack<T, V>(op + i, o);
-    }
+    };
+    batched_for<B>(
+        threadIdx.x, n_vec, blockDim.x,
+        [&](int64_t v, int64_t step) {
+          Pack<T, V> px[B], pd[B];
+          int64_t i[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            i[u] = split_pos(v + u * step, n_vec, rev) * V;
+            px[u] = load_pack<T, V>(xp + i[u]);
+            pd[u] = load_pack<T, V>(dp + i[u]);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) one(px[u], pd[u], i[u]);
+        },
+        [&](int64_t v) {
+          const int64_t i = split_pos(v, n_vec, rev) * V;
+          one(load_pack<T, V>(xp + i), load_pack<T, V>(dp + i), i);
+        });
   }
 }
 

@@ -83,7 +83,8 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
   ATEXN_CHECK_LAUNCH("split_fwd_stats");
   split_fwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
-                                                          n_rows, D, p.S, p.chunk, C, eps);
+                                                          n_rows, D, p.S, p.chunk, C, eps,
+                                                          tuning().reverse_second_pass);
   ATEXN_CHECK_LAUNCH("split_fwd_apply");
   return ATEXN_OK;
 }
@@ -115,7 +116,8 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
                                                          D, p.S, p.chunk);
   ATEXN_CHECK_LAUNCH("split_bwd_sums");
   split_bwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
-                                                          part, n_rows, D, p.S, p.chunk, C);
+                                                          part, n_rows, D, p.S, p.chunk, C,
+                                                          tuning().reverse_second_pass);
   ATEXN_CHECK_LAUNCH("split_bwd_apply");
   if constexpr (!AFF) {
     dim3 grid(p.col_tiles, p.col_slabs);

@@ -49,6 +49,21 @@ CASES = {
     "in2d_nchw": ("in", "f16", (8, 64, 128 * 128, True)),
     "in3d_ndhwc": ("in", "f16", (2, 32, 128 ** 3, False)),
     "in3d_ncdhw": ("in", "f16", (2, 32, 128 ** 3, True)),
+    # shapes of the reference's own benchmark tables (benchmark_layer_norm.py:53-63,
+    # benchmark_instance_norm.py:58-69), not part of --case all
+    "lnref_10x1e7": ("ln", "f16", (10, 10000000)),
+    "lnref_100x1e6": ("ln", "f16", (100, 1000000)),
+    "lnref_1e3x1e5": ("ln", "f16", (1000, 100000)),
+    "lnref_1e4x1e4": ("ln", "f16", (10000, 10000)),
+    "lnref_1e5x1e3": ("ln", "f16", (100000, 1000)),
+    "lnref_1e6x100": ("ln", "f16", (1000000, 100)),
+    "lnref_1e7x10": ("ln", "f16", (10000000, 10)),
+    "lnref_4x400001": ("ln", "f16", (4, 400001)),
+    "lnref_4x10000001": ("ln", "f16", (4, 10000001)),
+    "inref_8x64x64_cl": ("in", "f16", (8, 64, 64 ** 3, False)),
+    "inref_8x64x64_cf": ("in", "f16", (8, 64, 64 ** 3, True)),
+    "inref_4x256x32_cl": ("in", "f16", (4, 256, 32 ** 3, False)),
+    "inref_4x256x32_cf": ("in", "f16", (4, 256, 32 ** 3, True)),
 }
 DEFAULT_CASE = "ln_bert"
 
@@ -334,6 +349,8 @@ def main():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
     if args.case == "all":
         for name in CASES:
+            if "ref_" in name:
+                continue
             steps = args.steps if "3d" not in name else max(10, args.steps // 10)
             r = run_case(name, steps, args.warmup, with_cpu=False)
             print(json.dumps(r), flush=True)
