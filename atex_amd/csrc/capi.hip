@@ -80,7 +80,7 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
   else if (!strcmp(name, "split_items_per_cu")) t.split_items_per_cu = value;
   else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
-  else if (!strcmp(name, "colgrad_items_per_cu")) t.colgrad_items_per_cu = value;
+  else if (!strcmp(name, "tile_items_per_cu")) t.tile_items_per_cu = value;
   else if (!strcmp(name, "fwd_rows_batch") || !strcmp(name, "bwd_rows_batch")) {
     ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),
                   "rows batch must be 1, 2 (or 4, forward only)");

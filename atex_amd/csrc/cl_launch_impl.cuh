@@ -79,8 +79,7 @@ int cl_fwd_t(const void* x_, const float* gamma, const float* beta, int64_t N, i
   constexpr int VEC = VecOf<T>::value;
   const T* x = static_cast<const T*>(x_);
   T* y = static_cast<T*>(y_);
-  const bool vec = (C % VEC == 0) && aligned16(x) && aligned16(y) && aligned16(gamma) &&
-                   aligned16(beta) && aligned16(mean) && aligned16(rstd);
+  const bool vec = C % VEC == 0;  // 16-byte accesses work at element alignment
   return vec ? cl_fwd_v<T, VEC>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st)
              : cl_fwd_v<T, 1>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st);
 }
@@ -93,8 +92,7 @@ int cl_bwd_t(const void* dy_, const void* x_, const float* gamma, const float* m
   const T* x = static_cast<const T*>(x_);
   const T* dy = static_cast<const T*>(dy_);
   T* dx = static_cast<T*>(dx_);
-  const bool vec = (C % VEC == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
-                   aligned16(gamma) && aligned16(mean) && aligned16(rstd);
+  const bool vec = C % VEC == 0;
   return vec ? cl_bwd_v<T, VEC>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st)
              : cl_bwd_v<T, 1>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st);
 }

@@ -70,12 +70,22 @@ int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_
                       hipStream_t st) {
   ATEXN_REQUIRE(2 * W < (int64_t(1) << 31), "column count %lld too large", (long long)W);
   const int Wi = static_cast<int>(W);
-  if (W % 4 == 0 && aligned16(part)) {
-    const int grid = static_cast<int>(div_up(2 * W, 4 * 4));
-    col_reduce<4, 4><<<grid, kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+  // column groups per block: few when there are many partial rows to share among the
+  // threads of a group, one per thread when there are only a handful of rows
+  if (W % 4 == 0) {
+    if (G >= 128) {
+      col_reduce<4, 4><<<static_cast<int>(div_up(2 * W, 4 * 4)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    } else if (G >= 16) {
+      col_reduce<4, 64><<<static_cast<int>(div_up(2 * W, 4 * 64)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    } else {
+      col_reduce<4, 256><<<static_cast<int>(div_up(2 * W, 4 * 256)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    }
   } else {
-    const int grid = static_cast<int>(div_up(2 * W, 16));
-    col_reduce<1, 16><<<grid, kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    if (G >= 64) {
+      col_reduce<1, 16><<<static_cast<int>(div_up(2 * W, 16)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    } else {
+      col_reduce<1, 256><<<static_cast<int>(div_up(2 * W, 256)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    }
   }
   ATEXN_CHECK_LAUNCH("col_reduce");
   return ATEXN_OK;
@@ -137,30 +147,28 @@ int cl_bwd(int dtype, const void* dy, const void* x, const float* gamma, const f
   ATEXN_DISPATCH(dtype, cl_bwd_t<T>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st));
 }
 
-// Workspace: the larger of the 16-byte-vector plan and the element-wise plan, because
-// pointer alignment is only known at launch.
+// Workspace: the same choice of path as the launchers make (it depends on sizes only).
 static size_t rows_ws(RowsKind kind, int dtype, int64_t n_rows, int64_t D, int C) {
   if (n_rows <= 0 || D <= 0) return 0;
   const int vec = 16 / elem_size(dtype);
   const int cus = cu_count();
-  size_t b = plan_rows(kind, 1, n_rows, D, C, cus).ws_bytes;
-  if (D % vec == 0) b = std::max(b, plan_rows(kind, vec, n_rows, D, C, cus).ws_bytes);
-  return b;
+  const int V = D % vec == 0 ? vec : 1;
+  const bool layer_norm = C == 0;
+  if (layer_norm && D / V > resident_limit(kind)) {
+    return plan_tiles(kind != RowsKind::kFwd, vec, n_rows, D, cus).ws_bytes;
+  }
+  return plan_rows(kind, V, n_rows, D, C, cus).ws_bytes;
 }
 size_t rows_fwd_ws(int dtype, bool affine, int64_t n_rows, int64_t D, int C) {
-  (void)affine;
-  return rows_ws(RowsKind::kFwd, dtype, n_rows, D, C);
+  return rows_ws(RowsKind::kFwd, dtype, n_rows, D, affine ? C : 0);
 }
 size_t rows_bwd_ws(int dtype, bool affine, int64_t n_rows, int64_t D, int C) {
-  return rows_ws(affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols, dtype, n_rows, D, C);
+  return rows_ws(affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols, dtype, n_rows, D, affine ? C : 0);
 }
 static size_t cl_ws(bool bwd, int dtype, int64_t N, int64_t C, int64_t D) {
   if (N <= 0 || C <= 0 || D <= 0) return 0;
   const int vec = 16 / elem_size(dtype);
-  const int cus = cu_count();
-  size_t b = plan_cl(bwd, 1, N, C, D, cus).ws_bytes;
-  if (C % vec == 0) b = std::max(b, plan_cl(bwd, vec, N, C, D, cus).ws_bytes);
-  return b;
+  return plan_cl(bwd, C % vec == 0 ? vec : 1, N, C, D, cu_count()).ws_bytes;
 }
 size_t cl_fwd_ws(int dtype, int64_t N, int64_t C, int64_t D) { return cl_ws(false, dtype, N, C, D); }
 size_t cl_bwd_ws(int dtype, int64_t N, int64_t C, int64_t D) { return cl_ws(true, dtype, N, C, D); }

@@ -22,7 +22,7 @@ struct Tuning {
   int bwd_waves_per_cu = 8;       // resident backward: waves kept resident per CU
   int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
   int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
-  int colgrad_items_per_cu = 4;   // LayerNorm column pass of the split path
+  int tile_items_per_cu = 4;      // LayerNorm long rows: (row slab, column tile) tiles per CU
   int fwd_rows_batch = 4;         // resident kernels, rows <= one wave: rows per batch of a
   int bwd_rows_batch = 1;         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
@@ -57,25 +57,23 @@ struct RowsPlan {
   int S = 1;
   int64_t chunk = 0;
   int split_grid = 1;
-  int col_tiles = 0;  // LayerNorm backward column pass
-  int col_slabs = 0;
-  int64_t rows_per_slab = 0;
   // workspace sections (bytes from the start of the workspace)
   size_t off_part = 0, off_pairs = 0, ws_bytes = 0;
   int part_rows = 0;  // G of the column reduction
 };
 
-// V: vector width in elements (16 / sizeof(T)) when the call is 16-byte aligned, else 1.
+// Longest row, in vectors, that the register-resident kernels take: forward 8 vectors per
+// thread at 512 threads, backward 4 (it holds x and dy, and LayerNorm also gamma and the
+// dgamma / dbeta accumulators of its columns).
+inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kFwd ? 4096 : 2048; }
+
+// V: vector width in elements, 16 / sizeof(T) when D is a multiple of it, else 1.
 inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
   const Tuning& t = tuning();
   RowsPlan p;
   p.V = V;
   const int64_t n_vec = D / V;  // D % V == 0 whenever V > 1
-  // Limits follow the register budgets of the resident kernels at 512 threads: forward 8
-  // vectors per thread, backward 4 (it holds x and dy, and LayerNorm also gamma and the
-  // dgamma / dbeta accumulators of its columns).
-  const int64_t resident_limit = kind == RowsKind::kFwd ? 4096 : 2048;
-  p.resident = n_vec <= resident_limit;
+  p.resident = n_vec <= resident_limit(kind);
   if (p.resident) {
     if (n_vec <= 64) {
       p.tpr = std::max(8, pow2_ceil(n_vec));
@@ -132,19 +130,60 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   p.split_grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(n_work, int64_t(cus) * 32)));
   p.off_pairs = 0;
   size_t bytes = align256(sizeof(float) * 2 * size_t(n_work));
-  if (kind == RowsKind::kBwdCols) {
-    p.col_tiles = static_cast<int>(div_up(D, 256));
-    int64_t slabs = div_up(int64_t(cus) * t.colgrad_items_per_cu, p.col_tiles);
-    slabs = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(slabs, n_rows), 1024));
-    p.rows_per_slab = div_up(n_rows, slabs);
-    p.col_slabs = static_cast<int>(div_up(n_rows, p.rows_per_slab));
-    p.part_rows = p.col_slabs;
-    p.off_part = bytes;
-    bytes += align256(sizeof(float) * 2 * size_t(D) * size_t(p.col_slabs));
-  } else if (kind == RowsKind::kBwdAffine) {
+  if (kind == RowsKind::kBwdAffine) {
     p.part_rows = static_cast<int>(n_rows / C);
     p.off_part = bytes;
     bytes += align256(sizeof(float) * 2 * size_t(n_rows));
+  }
+  p.ws_bytes = bytes;
+  return p;
+}
+
+// LayerNorm rows too long for registers: 2-D tiles of R rows x CW columns (tiles_kernels.cuh).
+// The forward statistics still come from the chunked stage 1 of the split path (S chunks).
+struct TilePlan {
+  int V = 1;
+  int64_t CW = 0;  // columns per tile
+  int CT = 1;      // column tiles
+  int RS = 1;      // row slabs
+  int64_t R = 0;   // rows per slab
+  int S = 1;       // forward: chunks per row of the statistics stage
+  int64_t chunk = 0;
+  int stats_grid = 1;
+  size_t off_pairs = 0, off_rowsum = 0, off_part = 0, ws_bytes = 0;
+};
+
+constexpr int kPlanTileThreads = 256;
+constexpr int kPlanTileVpt = 4;
+
+inline TilePlan plan_tiles(bool bwd, int V, int64_t n_rows, int64_t D, int cus) {
+  const Tuning& t = tuning();
+  TilePlan p;
+  p.V = V;
+  p.CW = int64_t(kPlanTileThreads) * kPlanTileVpt * V;
+  p.CT = static_cast<int>(div_up(D, p.CW));
+  const int64_t want = div_up(int64_t(cus) * t.tile_items_per_cu, p.CT);
+  int64_t rs = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, n_rows), 1024));
+  p.R = div_up(n_rows, rs);
+  p.RS = static_cast<int>(div_up(n_rows, p.R));
+  size_t bytes = 0;
+  if (!bwd) {
+    const int64_t gran = int64_t(256) * V;
+    const int64_t want_s = div_up(int64_t(cus) * t.split_items_per_cu, std::max<int64_t>(n_rows, 1));
+    const int64_t max_s = std::max<int64_t>(1, D / (gran * 4));
+    const int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want_s, max_s), 1024));
+    p.chunk = round_up(div_up(D, S), gran);
+    p.S = static_cast<int>(div_up(D, p.chunk));
+    p.stats_grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(n_rows * p.S, int64_t(cus) * 32)));
+    p.off_pairs = 0;
+    bytes = align256(sizeof(float) * 2 * size_t(n_rows) * size_t(p.S));
+  } else {
+    p.off_pairs = 0;
+    bytes = align256(sizeof(float) * 2 * size_t(n_rows) * size_t(p.CT));
+    p.off_rowsum = bytes;
+    bytes += align256(sizeof(float) * 2 * size_t(n_rows));
+    p.off_part = bytes;
+    if (p.RS > 1) bytes += align256(sizeof(float) * 2 * size_t(D) * size_t(p.RS));
   }
   p.ws_bytes = bytes;
   return p;

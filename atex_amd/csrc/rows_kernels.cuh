@@ -529,9 +529,13 @@ template <int CW, int CX>
 __global__ void __launch_bounds__(kColReduceThreads)
 col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __restrict__ out1,
            int G, int W) {
+  // CX column groups of CW columns per block, CY = threads / CX partial rows in parallel:
+  // CX = 4 for many partial rows, 64 for a few dozen, 256 (one thread per group, no
+  // exchange) for a handful.
   constexpr int CY = kColReduceThreads / CX;
   constexpr int NW = kColReduceThreads / kWave;
-  __shared__ float buf[NW][CX][CW];
+  constexpr int HOLD = CX < kWave ? NW : CY;  // partial sums per column group after the wave fold
+  __shared__ float buf[HOLD > 1 ? HOLD : 1][CX][CW];
   const int cx = threadIdx.x % CX;
   const int cy = threadIdx.x / CX;
   const int W2 = 2 * W;
@@ -558,31 +562,41 @@ col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __re
       for (int i = 0; i < CW; ++i) acc[i] += t[i];
     }
   }
-  // lanes l, l + CX, ... of a wave hold slices of the same columns
+  if constexpr (CX < kWave) {
+    // lanes l, l + CX, ... of a wave hold slices of the same columns
 #pragma unroll
-  for (int i = 0; i < CW; ++i) {
+    for (int i = 0; i < CW; ++i) {
 #pragma unroll
-    for (int m = CX; m < kWave; m <<= 1) acc[i] += lane_xor(acc[i], m);
+      for (int m = CX; m < kWave; m <<= 1) acc[i] += lane_xor(acc[i], m);
+    }
   }
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave = threadIdx.x / kWave;
-  if (lane < CX) {
+  if constexpr (HOLD > 1) {
+    const int lane = threadIdx.x & (kWave - 1);
+    const int slot = CX < kWave ? threadIdx.x / kWave : cy;
+    if (CX >= kWave || lane < CX) {
 #pragma unroll
-    for (int i = 0; i < CW; ++i) buf[wave][lane][i] = acc[i];
+      for (int i = 0; i < CW; ++i) buf[slot][cx][i] = acc[i];
+    }
+    __syncthreads();
+    if (threadIdx.x < CX) {
+#pragma unroll
+      for (int i = 0; i < CW; ++i) {
+        float s = buf[0][cx][i];
+#pragma unroll
+        for (int k = 1; k < HOLD; ++k) s += buf[k][cx][i];
+        acc[i] = s;
+      }
+    }
   }
-  __syncthreads();
   if (threadIdx.x < CX && col < W2) {
 #pragma unroll
     for (int i = 0; i < CW; ++i) {
-      float s = buf[0][cx][i];
-#pragma unroll
-      for (int k = 1; k < NW; ++k) s += buf[k][cx][i];
       // CW divides W on the vector path, so a column group never straddles the two halves
       const int j = col + i;
       if (j < W) {
-        out0[j] = s;
+        out0[j] = acc[i];
       } else if (j < W2) {
-        out1[j - W] = s;
+        out1[j - W] = acc[i];
       }
     }
   }
@@ -615,9 +629,11 @@ __device__ __forceinline__ int64_t split_pos(int64_t p, int64_t n_vec, bool rev)
 template <typename T, int V>
 __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
   const int64_t n_vec = len / V;
+  const int rem = static_cast<int>(len % V);  // only the last chunk of a ragged row
   const int64_t tid = threadIdx.x;
-  if (tid >= n_vec) return Wf{0.f, 0.f, 0.f};
-  const float K = to_f32(p[tid * V]);
+  const bool has_tail = rem != 0 && n_vec % blockDim.x == tid;
+  if (tid >= n_vec && !has_tail) return Wf{0.f, 0.f, 0.f};
+  const float K = to_f32(p[tid < n_vec ? tid * V : n_vec * V]);
   float s1 = 0.f, s2 = 0.f;
   int64_t cnt = 0;
   auto acc = [&](const Pack<T, V>& pk) {
@@ -636,14 +652,22 @@ __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
         for (int u = 0; u < kSplitBatch; ++u) pk[u] = load_pack<T, V>(p + (v + u * step) * V);
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u) acc(pk[u]);
-        cnt += kSplitBatch;
+        cnt += kSplitBatch * V;
       },
       [&](int64_t v) {
         acc(load_pack<T, V>(p + v * V));
-        cnt += 1;
+        cnt += V;
       });
+  if (has_tail) {
+    for (int k = 0; k < rem; ++k) {
+      const float d = to_f32(p[n_vec * V + k]) - K;
+      s1 += d;
+      s2 += d * d;
+    }
+    cnt += rem;
+  }
   Wf w;
-  w.n = static_cast<float>(cnt * V);
+  w.n = static_cast<float>(cnt);
   const float inv = 1.0f / w.n;
   const float dm = s1 * inv;
   w.mean = K + dm;
@@ -881,31 +905,6 @@ __global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ 
           one(load_pack<T, V>(xp + i), load_pack<T, V>(dp + i), i);
         });
   }
-}
-
-// LayerNorm dgamma / dbeta when rows are not register-resident: thread <-> column,
-// block (x = column tile of blockDim.x, y = slab of rows); writes
-// part[slab][0][col], part[slab][1][col]; col_reduce finishes.
-// (reference equivalent: fused_layer_norm_op.cu:763-783)
-template <typename T>
-__global__ void ln_colgrad_partial(const T* __restrict__ dy, const T* __restrict__ x,
-                                   const float* __restrict__ mean_in,
-                                   const float* __restrict__ rstd_in, float* __restrict__ part,
-                                   int64_t n_rows, int64_t D, int64_t rows_per_slab) {
-  const int64_t col = static_cast<int64_t>(blockIdx.x) * blockDim.x + threadIdx.x;
-  const int64_t slab = blockIdx.y;
-  const int64_t r0 = slab * rows_per_slab;
-  const int64_t r1 = (r0 + rows_per_slab < n_rows) ? r0 + rows_per_slab : n_rows;
-  if (col >= D) return;
-  float ag = 0.f, ab = 0.f;
-  for (int64_t r = r0; r < r1; ++r) {
-    const float d = to_f32(dy[r * D + col]);
-    const float xh = (to_f32(x[r * D + col]) - mean_in[r]) * rstd_in[r];
-    ag += d * xh;
-    ab += d;
-  }
-  part[(slab * 2 + 0) * D + col] = ag;
-  part[(slab * 2 + 1) * D + col] = ab;
 }
 
 }  // namespace atexn

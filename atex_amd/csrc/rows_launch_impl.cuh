@@ -4,6 +4,7 @@
 
 #include "plan.h"
 #include "rows_kernels.cuh"
+#include "tiles_kernels.cuh"
 #include "status.h"
 
 namespace atexn {
@@ -79,14 +80,68 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
     ATEXN_CHECK_LAUNCH("rows_fwd_resident");
     return ATEXN_OK;
   }
+  if constexpr (AFF) {
+    float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
+    split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
+    ATEXN_CHECK_LAUNCH("split_fwd_stats");
+    split_fwd_apply<T, V, true><<<p.split_grid, 256, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
+                                                             n_rows, D, p.S, p.chunk, C, eps,
+                                                             tuning().reverse_second_pass);
+    ATEXN_CHECK_LAUNCH("split_fwd_apply");
+    return ATEXN_OK;
+  } else {
+    return set_error(ATEXN_LAUNCH_ERROR, "LayerNorm rows of %lld elements belong to the tile path", (long long)D);
+  }
+}
+
+// LayerNorm rows too long for registers, any D and alignment (tiles_kernels.cuh).
+template <typename T>
+int tiles_fwd(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
+              float eps, T* y, float* mean, float* rstd, void* ws, size_t ws_bytes,
+              hipStream_t st) {
+  constexpr int V = VecOf<T>::value;
+  const TilePlan p = plan_tiles(false, V, n_rows, D, cu_count());
+  ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
-  split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
+  split_fwd_stats<T, V><<<p.stats_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
   ATEXN_CHECK_LAUNCH("split_fwd_stats");
-  split_fwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
-                                                          n_rows, D, p.S, p.chunk, C, eps,
-                                                          tuning().reverse_second_pass);
-  ATEXN_CHECK_LAUNCH("split_fwd_apply");
+  merge_row_stats<4><<<static_cast<unsigned>(div_up(n_rows, 4)), 256, 0, st>>>(stats, mean, rstd, n_rows,
+                                                                        D, p.S, p.chunk, eps);
+  ATEXN_CHECK_LAUNCH("merge_row_stats");
+  const dim3 grid(p.CT, p.RS);
+  tile_fwd_apply<T, V><<<grid, kTileThreads, 0, st>>>(x, gamma, beta, mean, rstd, y, n_rows, D, p.R,
+                                                     tuning().reverse_second_pass);
+  ATEXN_CHECK_LAUNCH("tile_fwd_apply");
   return ATEXN_OK;
+}
+
+template <typename T>
+int tiles_bwd(const T* dy, const T* x, const float* gamma, const float* mean, const float* rstd,
+              int64_t n_rows, int64_t D, T* dx, float* dgamma, float* dbeta, void* ws,
+              size_t ws_bytes, hipStream_t st) {
+  constexpr int V = VecOf<T>::value;
+  const TilePlan p = plan_tiles(true, V, n_rows, D, cu_count());
+  ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  char* base = static_cast<char*>(ws);
+  float2* sums = reinterpret_cast<float2*>(base + p.off_pairs);
+  float2* rowsum = reinterpret_cast<float2*>(base + p.off_rowsum);
+  float* part = reinterpret_cast<float*>(base + p.off_part);
+  const dim3 grid(p.CT, p.RS);
+  const bool direct = p.RS == 1;  // one row slab: the column sums are final
+  tile_bwd_sums<T, V><<<grid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums,
+                                                    direct ? dgamma : part,
+                                                    direct ? dbeta : part + D,
+                                                    direct ? 0 : 2 * D, n_rows, D, p.R);
+  ATEXN_CHECK_LAUNCH("tile_bwd_sums");
+  merge_row_sums<4><<<static_cast<unsigned>(div_up(n_rows, 4)), 256, 0, st>>>(sums, rowsum, n_rows, p.CT);
+  ATEXN_CHECK_LAUNCH("merge_row_sums");
+  tile_bwd_apply<T, V><<<grid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, rowsum, dx, n_rows,
+                                                     D, p.R, tuning().reverse_second_pass);
+  ATEXN_CHECK_LAUNCH("tile_bwd_apply");
+  if (direct) return ATEXN_OK;
+  return launch_col_reduce(part, dgamma, dbeta, p.RS, D, st);
 }
 
 template <typename T, int V, bool AFF>
@@ -111,21 +166,19 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     if (!(stages & 2)) return ATEXN_OK;
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
   }
-  float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
-  split_bwd_sums<T, V, AFF><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
-                                                         D, p.S, p.chunk);
-  ATEXN_CHECK_LAUNCH("split_bwd_sums");
-  split_bwd_apply<T, V, AFF><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
-                                                          part, n_rows, D, p.S, p.chunk, C,
-                                                          tuning().reverse_second_pass);
-  ATEXN_CHECK_LAUNCH("split_bwd_apply");
-  if constexpr (!AFF) {
-    dim3 grid(p.col_tiles, p.col_slabs);
-    ln_colgrad_partial<T><<<grid, 256, 0, st>>>(dy, x, mean, rstd, part, n_rows, D,
-                                                 p.rows_per_slab);
-    ATEXN_CHECK_LAUNCH("ln_colgrad_partial");
+  if constexpr (AFF) {
+    float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
+    split_bwd_sums<T, V, true><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
+                                                            D, p.S, p.chunk);
+    ATEXN_CHECK_LAUNCH("split_bwd_sums");
+    split_bwd_apply<T, V, true><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
+                                                             part, n_rows, D, p.S, p.chunk, C,
+                                                             tuning().reverse_second_pass);
+    ATEXN_CHECK_LAUNCH("split_bwd_apply");
+    return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+  } else {
+    return set_error(ATEXN_LAUNCH_ERROR, "LayerNorm rows of %lld elements belong to the tile path", (long long)D);
   }
-  return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
 }
 
 template <typename T>
@@ -135,8 +188,11 @@ int rows_fwd_t(bool affine, const void* x_, const float* gamma, const float* bet
   constexpr int VEC = VecOf<T>::value;
   const T* x = static_cast<const T*>(x_);
   T* y = static_cast<T*>(y_);
-  const bool vec = (D % VEC == 0) && aligned16(x) && aligned16(y) &&
-                   (affine || (aligned16(gamma) && aligned16(beta)));
+  // 16-byte accesses need no pointer alignment beyond the element's, only whole vectors
+  const bool vec = D % VEC == 0;
+  if (!affine && D / (vec ? VEC : 1) > resident_limit(RowsKind::kFwd)) {
+    return tiles_fwd<T>(x, gamma, beta, n_rows, D, eps, y, mean, rstd, ws, ws_bytes, st);
+  }
   if (vec) {
     return affine ? rows_fwd_v<T, VEC, true>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st)
                   : rows_fwd_v<T, VEC, false>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st);
@@ -153,8 +209,10 @@ int rows_bwd_t(bool affine, const void* dy_, const void* x_, const float* gamma,
   const T* x = static_cast<const T*>(x_);
   const T* dy = static_cast<const T*>(dy_);
   T* dx = static_cast<T*>(dx_);
-  const bool vec = (D % VEC == 0) && aligned16(x) && aligned16(dy) && aligned16(dx) &&
-                   aligned16(ws) && (affine || aligned16(gamma));
+  const bool vec = D % VEC == 0;
+  if (!affine && D / (vec ? VEC : 1) > resident_limit(RowsKind::kBwdCols)) {
+    return tiles_bwd<T>(dy, x, gamma, mean, rstd, n_rows, D, dx, dgamma, dbeta, ws, ws_bytes, st);
+  }
   if (vec) {
     return affine ? rows_bwd_v<T, VEC, true>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st)
                   : rows_bwd_v<T, VEC, false>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st);

@@ -96,6 +96,33 @@ def test_in_place(capi, coracle, dtype, channel_first):
     run_case(capi, coracle, 1, 8, 300000, dtype, channel_first, 23, in_place=True)
 
 
+@pytest.mark.parametrize("channel_first", [False, True])
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("N,C,S", [(2, 32, 4096), (3, 24, 1000), (1, 8, 300000), (2, 64, 100)])
+def test_unaligned_pointers(capi, coracle, N, C, S, dtype, channel_first):
+    """Every array starts one element past an aligned address."""
+    import torch
+
+    print(f"IN unaligned N={N} C={C} spatial={S} dtype={dtype} channel_first={channel_first}", flush=True)
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, channel_first, 26)
+    y_ref, mean_ref, rstd_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, channel_first)
+    xd, dyd = util.misalign(util.to_device(x, dtype)), util.misalign(util.to_device(dy, dtype))
+    gd, bd = util.misalign(torch.from_numpy(gamma).cuda()), util.misalign(torch.from_numpy(beta).cuda())
+    y, mean, rstd = capi.in_fwd(xd, gd, bd, EPS, dtype, channel_first, y=util.misalign(torch.empty_like(xd)))
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert_close(util.to_host(mean), mean_ref, tol["stat"], "mean")
+    assert_close(util.to_host(rstd), rstd_ref, tol["stat"], "inv_std")
+    assert_close(util.to_host(y), y_ref, tol["y"], "y")
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(mean), util.to_host(rstd), dtype, channel_first)
+    dx, dg, db = capi.in_bwd(dyd, xd, gd, util.misalign(mean), util.misalign(rstd), dtype, channel_first)
+    torch.cuda.synchronize()
+    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx",
+                 scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), util.to_host(rstd), dtype))
+    assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+    assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+
+
 def test_layout_equivalence(capi):
     """IN over NC... of the transposed tensor equals the transpose of IN over N...C."""
     import torch

@@ -98,6 +98,43 @@ def test_in_place(capi, coracle, N, D, dtype):
     run_case(capi, coracle, "plain", N, D, dtype, 13, in_place=True)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("N,D", [(64, 1024), (37, 1000), (5, 8192), (3, 40000), (7, 40003), (2, 300001), (1000, 10),
+                                 (500, 100)])
+def test_unaligned_pointers(capi, coracle, N, D, dtype):
+    """Every array starts one element past an aligned address (a slice of a larger tensor):
+    the 16-byte accesses of the kernels must not depend on pointer alignment."""
+    import torch
+
+    print(f"LN unaligned N={N} D={D} dtype={dtype}", flush=True)
+    x, gamma, beta, dy = util.ln_inputs("plain", N, D, dtype, 16)
+    y_ref, mean_ref, rstd_ref = coracle.ln_fwd(x, gamma, beta, EPS, dtype)
+    xd, dyd = util.misalign(util.to_device(x, dtype)), util.misalign(util.to_device(dy, dtype))
+    gd, bd = util.misalign(torch.from_numpy(gamma).cuda()), util.misalign(torch.from_numpy(beta).cuda())
+    y, mean, rstd = capi.ln_fwd(xd, gd, bd, EPS, dtype, y=util.misalign(torch.empty_like(xd)))
+    torch.cuda.synchronize()
+    tol = TOL[dtype]
+    assert_close(util.to_host(mean), mean_ref, tol["stat"], "mean")
+    assert_close(util.to_host(rstd), rstd_ref, tol["stat"], "inv_std")
+    assert_close(util.to_host(y), y_ref, tol["y"], "y")
+    dx_ref, dg_ref, db_ref = coracle.ln_bwd(dy, x, gamma, util.to_host(mean), util.to_host(rstd), dtype)
+    dx, dg, db = capi.ln_bwd(dyd, xd, gd, util.misalign(mean), util.misalign(rstd), dtype)
+    torch.cuda.synchronize()
+    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx",
+                 scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), util.to_host(rstd), dtype))
+    assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+    assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("N,D", [(10, 1000000), (100, 100000), (4, 400001), (3, 1000003), (1000, 40000),
+                                 (300, 33000), (2, 2 ** 20 + 7)])
+def test_long_rows(capi, coracle, N, D, dtype):
+    """Rows beyond the register-resident limit, as in the reference's benchmark table
+    (benchmarks/benchmark_layer_norm.py:53-63): few long rows, odd lengths included."""
+    run_case(capi, coracle, "plain", N, D, dtype, 17)
+
+
 def test_many_rows_narrow(capi, coracle):
     run_case(capi, coracle, "plain", 100000, 10, "f32", 14)
     run_case(capi, coracle, "plain", 50000, 100, "f16", 14)

@@ -98,6 +98,18 @@ def to_device(a: np.ndarray, dtype: str, device="cuda:0"):
     return torch.from_numpy(a).to(device)
 
 
+def misalign(t, elements: int = 1):
+    """A copy of t whose storage starts `elements` elements past an allocation boundary, so
+    that no row, vector or parameter array is 16-byte aligned."""
+    import torch
+
+    buf = torch.empty(t.numel() + elements, dtype=t.dtype, device=t.device)
+    v = buf[elements:].view(t.shape)
+    v.copy_(t)
+    assert v.data_ptr() % 16 != 0 or t.numel() == 0
+    return v
+
+
 def to_host(t, dtype: str | None = None) -> np.ndarray:
     """torch tensor -> float64 numpy values."""
     import torch
