@@ -77,11 +77,16 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   const int64_t D = static_cast<int64_t>(n_vec) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
 
-  int n_valid_vec = VPT;
-  if constexpr (!EXACT) {
-    n_valid_vec = 0;
+  // Non-EXACT: loads are never predicated (a predicated load costs a full memory latency
+  // of its own).  A vector slot beyond the row reads the row's last vector, a row beyond
+  // the batch reads the last row, and the values are masked out of the arithmetic.
+  bool vec_ok[VPT];
+  int col[VPT];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+  for (int k = 0; k < VPT; ++k) {
+    const int idx = lane_r + k * tpr;
+    vec_ok[k] = EXACT || idx < n_vec;
+    col[k] = (vec_ok[k] ? idx : n_vec - 1) * V;
   }
 
   float g[GB_REGS ? NE : 1], b[GB_REGS ? NE : 1];
@@ -89,14 +94,8 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float tg[V], tb[V];
-      if (EXACT || k < n_valid_vec) {
-        const int col = (lane_r + k * tpr) * V;
-        load_f32<V>(gamma + col, tg);
-        load_f32<V>(beta + col, tb);
-      } else {
-#pragma unroll
-        for (int i = 0; i < V; ++i) tg[i] = tb[i] = 0.f;
-      }
+      load_f32<V>(gamma + col[k], tg);
+      load_f32<V>(beta + col[k], tb);
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         g[k * V + i] = tg[i];
@@ -112,12 +111,9 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int64_t row = base + r * rpb + slot;
-      const int nv = (EXACT || row < n_rows) ? n_valid_vec : 0;
-      const T* xr = x + row * D;
+      const T* xr = x + ((EXACT || row < n_rows) ? row : n_rows - 1) * D;
 #pragma unroll
-      for (int k = 0; k < VPT; ++k) {
-        if (EXACT || k < nv) raw[r][k] = load_pack<T, V>(xr + static_cast<int64_t>(lane_r + k * tpr) * V);
-      }
+      for (int k = 0; k < VPT; ++k) raw[r][k] = load_pack<T, V>(xr + col[k]);
     }
   };
 
@@ -134,11 +130,9 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       load_batch(row0, cur);
     }
 
-    int nv[RB];
+    bool row_ok[RB];
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      nv[r] = (EXACT || row0 + r * rpb + slot < n_rows) ? n_valid_vec : 0;
-    }
+    for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
     // stage 1: convert once, sum; elements outside the row are kept at 0
     float f[RB][NE];
     float mean[RB], rstd[RB];
@@ -149,7 +143,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float v = (EXACT || k < nv[r]) ? to_f32(cur[r][k].v[i]) : 0.f;
+          const float v = (EXACT || (vec_ok[k] && row_ok[r])) ? to_f32(cur[r][k].v[i]) : 0.f;
           f[r][k * V + i] = v;
           s += v;
         }
@@ -172,7 +166,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float d = (EXACT || k < nv[r]) ? f[r][k * V + i] - mean[r] : 0.f;
+          const float d = (EXACT || (vec_ok[k] && row_ok[r])) ? f[r][k * V + i] - mean[r] : 0.f;
           f[r][k * V + i] = d;
           q += d * d;
         }
@@ -193,10 +187,9 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int64_t row = row0 + r * rpb + slot;
-      const bool row_ok = EXACT || row < n_rows;
       float gs = 1.f, bs = 0.f;
       if constexpr (ROW_AFFINE) {
-        if (row_ok) {
+        if (row_ok[r]) {
           const int c = static_cast<int>(row % C);
           gs = gamma[c] * rstd[r];
           bs = beta[c];
@@ -205,13 +198,12 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       T* yr = y + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (EXACT || k < nv[r]) {
-          const int col = (lane_r + k * tpr) * V;
-          float tg[V], tb[V];
-          if constexpr (!ROW_AFFINE && !GB_REGS) {
-            load_f32<V>(gamma + col, tg);
-            load_f32<V>(beta + col, tb);
-          }
+        float tg[V], tb[V];
+        if constexpr (!ROW_AFFINE && !GB_REGS) {
+          load_f32<V>(gamma + col[k], tg);
+          load_f32<V>(beta + col[k], tb);
+        }
+        if (EXACT || (vec_ok[k] && row_ok[r])) {
           Pack<T, V> o;
 #pragma unroll
           for (int i = 0; i < V; ++i) {
@@ -226,10 +218,10 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
             }
             o.v[i] = from_f32<T>(res);
           }
-          store_pack<T, V>(yr + col, o);
+          store_pack<T, V>(yr + col[k], o);
         }
       }
-      if (row_ok && lane_r == 0) {
+      if (row_ok[r] && lane_r == 0) {
         mean_out[row] = mean[r];
         rstd_out[row] = rstd[r];
       }
@@ -284,11 +276,15 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
   const int64_t D = static_cast<int64_t>(n_vec) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
 
-  int n_valid_vec = VPT;
-  if constexpr (!EXACT) {
-    n_valid_vec = 0;
+  // Non-EXACT: unpredicated loads from clamped positions, masked arithmetic (see the
+  // forward kernel).
+  bool vec_ok[VPT];
+  int col[VPT];
 #pragma unroll
-    for (int k = 0; k < VPT; ++k) n_valid_vec += (lane_r + k * tpr < n_vec) ? 1 : 0;
+  for (int k = 0; k < VPT; ++k) {
+    const int idx = lane_r + k * tpr;
+    vec_ok[k] = EXACT || idx < n_vec;
+    col[k] = (vec_ok[k] ? idx : n_vec - 1) * V;
   }
 
   float g[ROW_AFFINE ? 1 : NE];
@@ -297,12 +293,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       float tg[V];
-      if (EXACT || k < n_valid_vec) {
-        load_f32<V>(gamma + (lane_r + k * tpr) * V, tg);
-      } else {
-#pragma unroll
-        for (int i = 0; i < V; ++i) tg[i] = 0.f;
-      }
+      load_f32<V>(gamma + col[k], tg);
 #pragma unroll
       for (int i = 0; i < V; ++i) {
         g[k * V + i] = tg[i];
@@ -322,20 +313,16 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
   auto load_batch = [&](int64_t base, Batch& t) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int64_t row = base + r * rpb + slot;
-      const bool row_ok = EXACT || row < n_rows;
-      const int nv = row_ok ? n_valid_vec : 0;
+      const int64_t row_q = base + r * rpb + slot;
+      const int64_t row = (EXACT || row_q < n_rows) ? row_q : n_rows - 1;
       const T* xr = x + row * D;
       const T* dyr = dy + row * D;
-      t.mean[r] = row_ok ? mean_in[row] : 0.f;
-      t.rstd[r] = row_ok ? rstd_in[row] : 0.f;
+      t.mean[r] = mean_in[row];
+      t.rstd[r] = rstd_in[row];
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (EXACT || k < nv) {
-          const int64_t off = static_cast<int64_t>(lane_r + k * tpr) * V;
-          t.px[r][k] = load_pack<T, V>(xr + off);
-          t.pd[r][k] = load_pack<T, V>(dyr + off);
-        }
+        t.px[r][k] = load_pack<T, V>(xr + col[k]);
+        t.pd[r][k] = load_pack<T, V>(dyr + col[k]);
       }
     }
   };
@@ -352,11 +339,9 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
       load_batch(row0, cur);
     }
 
-    int nv[RB];
+    bool row_ok[RB];
 #pragma unroll
-    for (int r = 0; r < RB; ++r) {
-      nv[r] = (EXACT || row0 + r * rpb + slot < n_rows) ? n_valid_vec : 0;
-    }
+    for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
     // stage 1: convert once; xh = (x - mean) * r, gv = dy * gamma; row sums and the
     // column accumulators.  Elements outside the row are 0 and add nothing.
     float xh[RB][NE], gv[RB][NE];
@@ -369,7 +354,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const int e = k * V + i;
-          const bool ok = EXACT || k < nv[r];
+          const bool ok = EXACT || (vec_ok[k] && row_ok[r]);
           const float h = ok ? (to_f32(cur.px[r][k].v[i]) - cur.mean[r]) * cur.rstd[r] : 0.f;
           const float d = ok ? to_f32(cur.pd[r][k].v[i]) : 0.f;
           xh[r][e] = h;
@@ -405,11 +390,10 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       const int64_t row = row0 + r * rpb + slot;
-      const bool row_ok = EXACT || row < n_rows;
       float scale = cur.rstd[r];
       if constexpr (ROW_AFFINE) {
-        if (row_ok) scale *= gamma[static_cast<int>(row % C)];
-        if (row_ok && lane_r == 0) {
+        if (row_ok[r]) scale *= gamma[static_cast<int>(row % C)];
+        if (row_ok[r] && lane_r == 0) {
           const int64_t n = row / C;
           const int c = static_cast<int>(row % C);
           part[(n * 2 + 0) * C + c] = s2[r];
@@ -420,14 +404,14 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
       T* dxr = dx + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (EXACT || k < nv[r]) {
+        if (EXACT || (vec_ok[k] && row_ok[r])) {
           Pack<T, V> o;
 #pragma unroll
           for (int i = 0; i < V; ++i) {
             const int e = k * V + i;
             o.v[i] = from_f32<T>(scale * gv[r][e] + (ca * xh[r][e] + cb));
           }
-          store_pack<T, V>(dxr + static_cast<int64_t>(lane_r + k * tpr) * V, o);
+          store_pack<T, V>(dxr + col[k], o);
         }
       }
     }
@@ -442,16 +426,15 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
       // one row per block: every thread owns its columns outright
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (k < n_valid_vec) {
-          const int col = (lane_r + k * tpr) * V;
+        if (vec_ok[k]) {
           float tg[V], tb[V];
 #pragma unroll
           for (int i = 0; i < V; ++i) {
             tg[i] = acc_g[k * V + i];
             tb[i] = acc_b[k * V + i];
           }
-          store_f32<V>(prow + col, tg);
-          store_f32<V>(prow + D + col, tb);
+          store_f32<V>(prow + col[k], tg);
+          store_f32<V>(prow + D + col[k], tb);
         }
       }
     } else {
@@ -498,16 +481,15 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
       if (wave == 0 && lane < tpr) {
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
-          if (k < n_valid_vec) {
-            const int col = (lane_r + k * tpr) * V;
+          if (vec_ok[k]) {
             float tg[V], tb[V];
 #pragma unroll
             for (int i = 0; i < V; ++i) {
               tg[i] = acc_g[k * V + i];
               tb[i] = acc_b[k * V + i];
             }
-            store_f32<V>(prow + col, tg);
-            store_f32<V>(prow + D + col, tb);
+            store_f32<V>(prow + col[k], tg);
+            store_f32<V>(prow + D + col[k], tb);
           }
         }
       }
