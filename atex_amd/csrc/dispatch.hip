@@ -152,12 +152,10 @@ static size_t rows_ws(RowsKind kind, int dtype, int64_t n_rows, int64_t D, int C
   if (n_rows <= 0 || D <= 0) return 0;
   const int vec = 16 / elem_size(dtype);
   const int cus = cu_count();
-  const int V = D % vec == 0 ? vec : 1;
   const bool layer_norm = C == 0;
-  if (layer_norm && D / V > resident_limit(kind)) {
-    return plan_tiles(kind != RowsKind::kFwd, vec, n_rows, D, cus).ws_bytes;
-  }
-  return plan_rows(kind, V, n_rows, D, C, cus).ws_bytes;
+  const RowsRoute r = route_rows(kind, layer_norm, vec, D);
+  if (r.tiles) return plan_tiles(kind != RowsKind::kFwd, vec, n_rows, D, cus).ws_bytes;
+  return plan_rows(kind, r.V, n_rows, D, C, cus).ws_bytes;
 }
 size_t rows_fwd_ws(int dtype, bool affine, int64_t n_rows, int64_t D, int C) {
   return rows_ws(RowsKind::kFwd, dtype, n_rows, D, affine ? C : 0);

@@ -64,6 +64,19 @@ __device__ __forceinline__ void store_pack_n(T* p, const Pack<T, V>& v, int cnt)
   }
 }
 
+// Elements lo .. V-1 of a vector (lo == 0: the single wide access).
+template <typename T, int V>
+__device__ __forceinline__ void store_pack_from(T* p, const Pack<T, V>& v, int lo) {
+  if (lo == 0) {
+    store_pack<T, V>(p, v);
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (i >= lo) p[i] = v.v[i];
+  }
+}
+
 template <typename T>
 __device__ __forceinline__ float to_f32(T v) {
   return static_cast<float>(v);
@@ -121,6 +134,18 @@ __device__ __forceinline__ void store_f32_n(float* p, const float (&in)[V], int 
 #pragma unroll
   for (int i = 0; i < V; ++i) {
     if (i < cnt) p[i] = in[i];
+  }
+}
+
+template <int V>
+__device__ __forceinline__ void store_f32_from(float* p, const float (&in)[V], int lo) {
+  if (lo == 0) {
+    store_f32<V>(p, in);
+    return;
+  }
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    if (i >= lo) p[i] = in[i];
   }
 }
 

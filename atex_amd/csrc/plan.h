@@ -51,6 +51,7 @@ struct RowsPlan {
   // resident
   int tpr = 0, vpt = 1, threads = 256, rpb = 1, rb = 1;
   bool exact = false;  // no lane, vector or row of any batch falls outside the data
+  bool ragged = false;  // D % V != 0: the last vector of a row is partial
   int grid = 1;
   size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
   // split
@@ -67,12 +68,32 @@ struct RowsPlan {
 // dgamma / dbeta accumulators of its columns).
 inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kFwd ? 4096 : 2048; }
 
-// V: vector width in elements, 16 / sizeof(T) when D is a multiple of it, else 1.
+// Which kernels take a contiguous-row problem.  vec = 16 / sizeof(T).
+//   V = vec: rows of whole vectors, or ragged rows (D % vec != 0, D >= vec) short enough
+//            for the register-resident kernels; V = 1: everything else on the row kernels;
+//   tiles:   LayerNorm rows beyond the resident limit (any D).
+struct RowsRoute {
+  int V = 1;
+  bool tiles = false;
+};
+inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t D) {
+  RowsRoute r;
+  if (D % vec == 0) {
+    r.V = vec;
+  } else if (D >= vec && div_up(D, vec) <= resident_limit(kind)) {
+    r.V = vec;
+  }
+  r.tiles = layer_norm && div_up(D, r.V) > resident_limit(kind);
+  return r;
+}
+
+// V: vector width in elements (see route_rows).
 inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
   const Tuning& t = tuning();
   RowsPlan p;
   p.V = V;
-  const int64_t n_vec = D / V;  // D % V == 0 whenever V > 1
+  const int64_t n_vec = div_up(D, V);
+  p.ragged = D % V != 0;  // resident kernels only
   p.resident = n_vec <= resident_limit(kind);
   if (p.resident) {
     if (n_vec <= 64) {
@@ -90,7 +111,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.rpb = 1;
     } else {
       p.threads = 256;
-      if (V > 1) p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
+      if (V > 1 && !p.ragged) p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
       if (kind == RowsKind::kBwdCols) {
         // bigger blocks -> fewer partial rows for the column reduction
         int th = std::min(t.bwd_ln_threads, 512);
@@ -101,7 +122,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       while (p.rb > 1 && div_up(n_rows, int64_t(p.rpb) * p.rb) < cus) p.rb /= 2;
     }
     const int64_t groups = div_up(n_rows, int64_t(p.rpb) * p.rb);
-    p.exact = V > 1 && n_vec == int64_t(p.tpr == 0 ? p.threads : p.tpr) * p.vpt &&
+    p.exact = V > 1 && !p.ragged && n_vec == int64_t(p.tpr == 0 ? p.threads : p.tpr) * p.vpt &&
               n_rows % (int64_t(p.rpb) * p.rb) == 0;
     const int waves = p.threads / 64;
     const int per_cu = std::max(

@@ -56,15 +56,20 @@ constexpr int resident_bwd_max_threads() {
 // RB rows per lane group form a batch; the next batch is loaded (software prefetch)
 // before the current one is reduced, so loads overlap the arithmetic.
 // EXACT: every lane owns exactly VPT vectors of every row of every batch (host-checked:
-// n_vec == lanes-per-row * VPT and n_rows % (rows-per-block * RB) == 0); all predicates
+// D == lanes-per-row * VPT * V and n_rows % (rows-per-block * RB) == 0); all predicates
 // fold away.
-template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE>
+// RAGGED: D is not a multiple of V.  The lane after the last full vector takes the LAST V
+// elements of the row (an access that overlaps its neighbour's, at element alignment) and
+// uses only the D % V of them that no other lane owns; its stores are element-wise.
+template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
+          bool RAGGED = false>
 __global__ void __launch_bounds__((resident_fwd_max_threads<TPR, VPT>()))
 rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta,
                   T* y, float* __restrict__ mean_out, float* __restrict__ rstd_out,
-                  int64_t n_rows, int n_vec, int C, float eps) {
+                  int64_t n_rows, int d_elems, int C, float eps) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
+  static_assert(!(RAGGED && (EXACT || RB != 1 || V == 1)), "ragged rows use the plain variant");
   // gamma / beta live in registers across rows unless that would exhaust the budget
   constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 4);
   static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
@@ -74,20 +79,31 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   const int rpb = M::rows_per_block();
   const int lane_r = M::lane_in_row();
   const int slot = M::slot();
-  const int64_t D = static_cast<int64_t>(n_vec) * V;
+  const int64_t D = d_elems;
   const float inv_d = 1.0f / static_cast<float>(D);
 
   // Non-EXACT: loads are never predicated (a predicated load costs a full memory latency
-  // of its own).  A vector slot beyond the row reads the row's last vector, a row beyond
-  // the batch reads the last row, and the values are masked out of the arithmetic.
+  // of its own).  A vector slot beyond the row reads the row's last V elements, a row
+  // beyond the batch reads the last row, and the values are masked out of the arithmetic.
+  const int n_full = d_elems / V;
+  const int rem = RAGGED ? d_elems % V : 0;
   bool vec_ok[VPT];
   int col[VPT];
+  int lo[VPT];  // RAGGED: first element of the vector that this lane owns
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = lane_r + k * tpr;
-    vec_ok[k] = EXACT || idx < n_vec;
-    col[k] = (vec_ok[k] ? idx : n_vec - 1) * V;
+    const bool full = EXACT || idx < n_full;
+    const bool tail = RAGGED && idx == n_full;
+    vec_ok[k] = full || tail;
+    col[k] = full ? idx * V : d_elems - V;
+    lo[k] = tail ? V - rem : 0;
   }
+  auto elem_ok = [&](int r_ok, int k, int i) -> bool {
+    if constexpr (EXACT) return true;
+    if constexpr (RAGGED) return vec_ok[k] && r_ok && i >= lo[k];
+    return vec_ok[k] && r_ok;
+  };
 
   float g[GB_REGS ? NE : 1], b[GB_REGS ? NE : 1];
   if constexpr (GB_REGS) {
@@ -143,7 +159,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float v = (EXACT || (vec_ok[k] && row_ok[r])) ? to_f32(cur[r][k].v[i]) : 0.f;
+          const float v = elem_ok(row_ok[r], k, i) ? to_f32(cur[r][k].v[i]) : 0.f;
           f[r][k * V + i] = v;
           s += v;
         }
@@ -166,7 +182,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float d = (EXACT || (vec_ok[k] && row_ok[r])) ? f[r][k * V + i] - mean[r] : 0.f;
+          const float d = elem_ok(row_ok[r], k, i) ? f[r][k * V + i] - mean[r] : 0.f;
           f[r][k * V + i] = d;
           q += d * d;
         }
@@ -218,7 +234,11 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
             }
             o.v[i] = from_f32<T>(res);
           }
-          store_pack<T, V>(yr + col[k], o);
+          if constexpr (RAGGED) {
+            store_pack_from<T, V>(yr + col[k], o, lo[k]);
+          } else {
+            store_pack<T, V>(yr + col[k], o);
+          }
         }
       }
       if (row_ok[r] && lane_r == 0) {
@@ -256,14 +276,16 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // are written to part[n][0][c] = b, part[n][1][c] = a  (n = row / C), i.e. `part` has
 // N * 2 * C floats and the same second kernel folds it over n.
 // dx must not alias dy or x.  RB / EXACT / prefetch as in the forward kernel.
-template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE>
+template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
+          bool RAGGED = false>
 __global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB>()))
 rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* __restrict__ dx,
-                  float* __restrict__ part, int64_t n_rows, int n_vec, int C) {
+                  float* __restrict__ part, int64_t n_rows, int d_elems, int C) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
+  static_assert(!(RAGGED && (EXACT || RB != 1 || V == 1)), "ragged rows use the plain variant");
   static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float2 sum_buf[2][16];
   // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats
@@ -273,18 +295,24 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
   const int rpb = M::rows_per_block();
   const int lane_r = M::lane_in_row();
   const int slot = M::slot();
-  const int64_t D = static_cast<int64_t>(n_vec) * V;
+  const int64_t D = d_elems;
   const float inv_d = 1.0f / static_cast<float>(D);
 
-  // Non-EXACT: unpredicated loads from clamped positions, masked arithmetic (see the
-  // forward kernel).
+  // Non-EXACT / RAGGED: unpredicated loads from clamped positions, masked arithmetic (see
+  // the forward kernel).
+  const int n_full = d_elems / V;
+  const int rem = RAGGED ? d_elems % V : 0;
   bool vec_ok[VPT];
   int col[VPT];
+  int lo[VPT];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = lane_r + k * tpr;
-    vec_ok[k] = EXACT || idx < n_vec;
-    col[k] = (vec_ok[k] ? idx : n_vec - 1) * V;
+    const bool full = EXACT || idx < n_full;
+    const bool tail = RAGGED && idx == n_full;
+    vec_ok[k] = full || tail;
+    col[k] = full ? idx * V : d_elems - V;
+    lo[k] = tail ? V - rem : 0;
   }
 
   float g[ROW_AFFINE ? 1 : NE];
@@ -354,7 +382,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const int e = k * V + i;
-          const bool ok = EXACT || (vec_ok[k] && row_ok[r]);
+          const bool ok = EXACT || (vec_ok[k] && row_ok[r] && (!RAGGED || i >= lo[k]));
           const float h = ok ? (to_f32(cur.px[r][k].v[i]) - cur.mean[r]) * cur.rstd[r] : 0.f;
           const float d = ok ? to_f32(cur.pd[r][k].v[i]) : 0.f;
           xh[r][e] = h;
@@ -411,7 +439,11 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
             const int e = k * V + i;
             o.v[i] = from_f32<T>(scale * gv[r][e] + (ca * xh[r][e] + cb));
           }
-          store_pack<T, V>(dxr + col[k], o);
+          if constexpr (RAGGED) {
+            store_pack_from<T, V>(dxr + col[k], o, lo[k]);
+          } else {
+            store_pack<T, V>(dxr + col[k], o);
+          }
         }
       }
     }
@@ -433,8 +465,13 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
             tg[i] = acc_g[k * V + i];
             tb[i] = acc_b[k * V + i];
           }
-          store_f32<V>(prow + col[k], tg);
-          store_f32<V>(prow + D + col[k], tb);
+          if constexpr (RAGGED) {
+            store_f32_from<V>(prow + col[k], tg, lo[k]);
+            store_f32_from<V>(prow + D + col[k], tb, lo[k]);
+          } else {
+            store_f32<V>(prow + col[k], tg);
+            store_f32<V>(prow + D + col[k], tb);
+          }
         }
       }
     } else {
@@ -488,8 +525,13 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
               tg[i] = acc_g[k * V + i];
               tb[i] = acc_b[k * V + i];
             }
-            store_f32<V>(prow + col[k], tg);
-            store_f32<V>(prow + D + col[k], tb);
+            if constexpr (RAGGED) {
+              store_f32_from<V>(prow + col[k], tg, lo[k]);
+              store_f32_from<V>(prow + D + col[k], tb, lo[k]);
+            } else {
+              store_f32<V>(prow + col[k], tg);
+              store_f32<V>(prow + D + col[k], tb);
+            }
           }
         }
       }

@@ -19,8 +19,9 @@ using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, c
 // Row batching (RB > 1) exists for the vector path and rows of at most one wave; the
 // predicate-free EXACT variants exist for the vector path.
 template <typename T, int V, int TPR, int VPT, bool AFF>
-FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact) {
+FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
+    if (ragged) return rows_fwd_resident<T, V, TPR, VPT, 1, false, AFF, true>;
     if constexpr (TPR != 0) {
       if (rb == 2) return exact ? rows_fwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 2, false, AFF>;
       if (rb == 4) return exact ? rows_fwd_resident<T, V, TPR, VPT, 4, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 4, false, AFF>;
@@ -30,8 +31,9 @@ FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact) {
   return rb == 1 ? rows_fwd_resident<T, V, TPR, VPT, 1, false, AFF> : nullptr;
 }
 template <typename T, int V, int TPR, int VPT, bool AFF>
-BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact) {
+BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
+    if (ragged) return rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF, true>;
     if constexpr (TPR != 0) {
       if (rb == 2) return exact ? rows_bwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF>;
     }
@@ -41,27 +43,30 @@ BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact) {
 }
 
 template <typename T, int V, bool AFF>
-FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb, bool exact) {
-  if (tpr == 8) return fwd_variant<T, V, 8, 1, AFF>(rb, exact);
-  if (tpr == 16) return fwd_variant<T, V, 16, 1, AFF>(rb, exact);
-  if (tpr == 32) return fwd_variant<T, V, 32, 1, AFF>(rb, exact);
-  if (tpr == 64 && vpt == 1) return fwd_variant<T, V, 64, 1, AFF>(rb, exact);
-  if (tpr == 64 && vpt == 2) return fwd_variant<T, V, 64, 2, AFF>(rb, exact);
-  if (tpr == 0 && vpt == 2) return fwd_variant<T, V, 0, 2, AFF>(rb, exact);
-  if (tpr == 0 && vpt == 4) return fwd_variant<T, V, 0, 4, AFF>(rb, exact);
-  if (tpr == 0 && vpt == 8) return fwd_variant<T, V, 0, 8, AFF>(rb, exact);
+FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb, bool exact, bool ragged) {
+  // element-wise rows are only the ones shorter than a vector
+  if constexpr (V == 1) return tpr == 8 && vpt == 1 ? fwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  if (tpr == 8) return fwd_variant<T, V, 8, 1, AFF>(rb, exact, ragged);
+  if (tpr == 16) return fwd_variant<T, V, 16, 1, AFF>(rb, exact, ragged);
+  if (tpr == 32) return fwd_variant<T, V, 32, 1, AFF>(rb, exact, ragged);
+  if (tpr == 64 && vpt == 1) return fwd_variant<T, V, 64, 1, AFF>(rb, exact, ragged);
+  if (tpr == 64 && vpt == 2) return fwd_variant<T, V, 64, 2, AFF>(rb, exact, ragged);
+  if (tpr == 0 && vpt == 2) return fwd_variant<T, V, 0, 2, AFF>(rb, exact, ragged);
+  if (tpr == 0 && vpt == 4) return fwd_variant<T, V, 0, 4, AFF>(rb, exact, ragged);
+  if (tpr == 0 && vpt == 8) return fwd_variant<T, V, 0, 8, AFF>(rb, exact, ragged);
   return nullptr;
 }
 
 template <typename T, int V, bool AFF>
-BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact) {
-  if (tpr == 8) return bwd_variant<T, V, 8, 1, AFF>(rb, exact);
-  if (tpr == 16) return bwd_variant<T, V, 16, 1, AFF>(rb, exact);
-  if (tpr == 32) return bwd_variant<T, V, 32, 1, AFF>(rb, exact);
-  if (tpr == 64 && vpt == 1) return bwd_variant<T, V, 64, 1, AFF>(rb, exact);
-  if (tpr == 64 && vpt == 2) return bwd_variant<T, V, 64, 2, AFF>(rb, exact);
-  if (tpr == 0 && vpt == 2) return bwd_variant<T, V, 0, 2, AFF>(rb, exact);
-  if (tpr == 0 && vpt == 4) return bwd_variant<T, V, 0, 4, AFF>(rb, exact);
+BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact, bool ragged) {
+  if constexpr (V == 1) return tpr == 8 && vpt == 1 ? bwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  if (tpr == 8) return bwd_variant<T, V, 8, 1, AFF>(rb, exact, ragged);
+  if (tpr == 16) return bwd_variant<T, V, 16, 1, AFF>(rb, exact, ragged);
+  if (tpr == 32) return bwd_variant<T, V, 32, 1, AFF>(rb, exact, ragged);
+  if (tpr == 64 && vpt == 1) return bwd_variant<T, V, 64, 1, AFF>(rb, exact, ragged);
+  if (tpr == 64 && vpt == 2) return bwd_variant<T, V, 64, 2, AFF>(rb, exact, ragged);
+  if (tpr == 0 && vpt == 2) return bwd_variant<T, V, 0, 2, AFF>(rb, exact, ragged);
+  if (tpr == 0 && vpt == 4) return bwd_variant<T, V, 0, 4, AFF>(rb, exact, ragged);
   return nullptr;
 }
 
@@ -73,10 +78,10 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && (p.ws_bytes == 0 || ws != nullptr),
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   if (p.resident) {
-    auto fn = pick_fwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact);
+    auto fn = pick_fwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact, p.ragged);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident forward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
-    fn<<<p.grid, p.threads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows,
-                                     static_cast<int>(D / V), C, eps);
+    fn<<<p.grid, p.threads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows, static_cast<int>(D), C,
+                                     eps);
     ATEXN_CHECK_LAUNCH("rows_fwd_resident");
     return ATEXN_OK;
   }
@@ -155,12 +160,12 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_part);
   const int64_t W = AFF ? C : D;
   if (p.resident) {
-    auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact);
+    auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact, p.ragged);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
     const int stages = tuning().bwd_stage_mask;
     if (stages & 1) {
       fn<<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
-                                                static_cast<int>(D / V), C);
+                                                static_cast<int>(D), C);
       ATEXN_CHECK_LAUNCH("rows_bwd_resident");
     }
     if (!(stages & 2)) return ATEXN_OK;
@@ -188,12 +193,12 @@ int rows_fwd_t(bool affine, const void* x_, const float* gamma, const float* bet
   constexpr int VEC = VecOf<T>::value;
   const T* x = static_cast<const T*>(x_);
   T* y = static_cast<T*>(y_);
-  // 16-byte accesses need no pointer alignment beyond the element's, only whole vectors
-  const bool vec = D % VEC == 0;
-  if (!affine && D / (vec ? VEC : 1) > resident_limit(RowsKind::kFwd)) {
+  // 16-byte accesses need no pointer alignment beyond the element's
+  const RowsRoute route = route_rows(RowsKind::kFwd, !affine, VEC, D);
+  if (route.tiles) {
     return tiles_fwd<T>(x, gamma, beta, n_rows, D, eps, y, mean, rstd, ws, ws_bytes, st);
   }
-  if (vec) {
+  if (route.V > 1) {
     return affine ? rows_fwd_v<T, VEC, true>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st)
                   : rows_fwd_v<T, VEC, false>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, ws, ws_bytes, st);
   }
@@ -209,11 +214,12 @@ int rows_bwd_t(bool affine, const void* dy_, const void* x_, const float* gamma,
   const T* x = static_cast<const T*>(x_);
   const T* dy = static_cast<const T*>(dy_);
   T* dx = static_cast<T*>(dx_);
-  const bool vec = D % VEC == 0;
-  if (!affine && D / (vec ? VEC : 1) > resident_limit(RowsKind::kBwdCols)) {
+  const RowsRoute route =
+      route_rows(affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols, !affine, VEC, D);
+  if (route.tiles) {
     return tiles_bwd<T>(dy, x, gamma, mean, rstd, n_rows, D, dx, dgamma, dbeta, ws, ws_bytes, st);
   }
-  if (vec) {
+  if (route.V > 1) {
     return affine ? rows_bwd_v<T, VEC, true>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st)
                   : rows_bwd_v<T, VEC, false>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st);
   }
