@@ -153,7 +153,8 @@ static size_t rows_ws(RowsKind kind, int dtype, int64_t n_rows, int64_t D, int C
   const int vec = 16 / elem_size(dtype);
   const int cus = cu_count();
   const bool layer_norm = C == 0;
-  const RowsRoute r = route_rows(kind, layer_norm, vec, D);
+  const RowsRoute r = route_rows(kind, layer_norm, vec, n_rows, D);
+  if (r.small) return plan_small(kind, r.V, n_rows, D, C, cus).ws_bytes;
   if (r.tiles) return plan_tiles(kind != RowsKind::kFwd, vec, n_rows, D, cus).ws_bytes;
   return plan_rows(kind, r.V, n_rows, D, C, cus).ws_bytes;
 }

@@ -72,12 +72,21 @@ inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kFwd ? 4
 //   V = vec: rows of whole vectors, or ragged rows (D % vec != 0, D >= vec) short enough
 //            for the register-resident kernels; V = 1: everything else on the row kernels;
 //   tiles:   LayerNorm rows beyond the resident limit (any D).
+//   small:   rows of at most 4 vectors when there are many of them: one thread per row.
 struct RowsRoute {
   int V = 1;
   bool tiles = false;
+  bool small = false;
 };
-inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t D) {
+constexpr int kPlanSmallMaxVec = 4;
+constexpr int64_t kPlanSmallMinRows = 4096;
+inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, int64_t D) {
   RowsRoute r;
+  if (D >= vec && div_up(D, vec) <= kPlanSmallMaxVec && n_rows >= kPlanSmallMinRows) {
+    r.V = vec;
+    r.small = true;
+    return r;
+  }
   if (D % vec == 0) {
     r.V = vec;
   } else if (D >= vec && div_up(D, vec) <= resident_limit(kind)) {
@@ -85,6 +94,26 @@ inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t D) 
   }
   r.tiles = layer_norm && div_up(D, r.V) > resident_limit(kind);
   return r;
+}
+
+struct SmallPlan {
+  int NV = 1;
+  int grid = 1;
+  int part_rows = 0;
+  size_t ws_bytes = 0;
+};
+inline SmallPlan plan_small(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
+  SmallPlan p;
+  p.NV = static_cast<int>(div_up(D, V));
+  p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(div_up(n_rows, 256), int64_t(cus) * 8)));
+  if (kind == RowsKind::kBwdCols) {
+    p.part_rows = p.grid;
+    p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
+  } else if (kind == RowsKind::kBwdAffine) {
+    p.part_rows = static_cast<int>(n_rows / C);
+    p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
+  }
+  return p;
 }
 
 // V: vector width in elements (see route_rows).

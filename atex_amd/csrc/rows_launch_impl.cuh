@@ -4,6 +4,7 @@
 
 #include "plan.h"
 #include "rows_kernels.cuh"
+#include "small_kernels.cuh"
 #include "tiles_kernels.cuh"
 #include "status.h"
 
@@ -97,6 +98,46 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   } else {
     return set_error(ATEXN_LAUNCH_ERROR, "LayerNorm rows of %lld elements belong to the tile path", (long long)D);
   }
+}
+
+// Many rows of at most four vectors: one thread per row (small_kernels.cuh).
+template <typename T, bool AFF>
+int small_fwd_launch(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
+                     int C, float eps, T* y, float* mean, float* rstd, hipStream_t st) {
+  constexpr int V = VecOf<T>::value;
+  const SmallPlan p = plan_small(RowsKind::kFwd, V, n_rows, D, C, cu_count());
+  const int Di = static_cast<int>(D);
+  switch (p.NV) {
+    case 1: small_fwd<T, V, 1, AFF><<<p.grid, kSmallThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows, Di, C, eps); break;
+    case 2: small_fwd<T, V, 2, AFF><<<p.grid, kSmallThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows, Di, C, eps); break;
+    case 3: small_fwd<T, V, 3, AFF><<<p.grid, kSmallThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows, Di, C, eps); break;
+    default: small_fwd<T, V, 4, AFF><<<p.grid, kSmallThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, n_rows, Di, C, eps); break;
+  }
+  ATEXN_CHECK_LAUNCH("small_fwd");
+  return ATEXN_OK;
+}
+
+template <typename T, bool AFF>
+int small_bwd_launch(const T* dy, const T* x, const float* gamma, const float* mean,
+                     const float* rstd, int64_t n_rows, int64_t D, int C, T* dx, float* dgamma,
+                     float* dbeta, void* ws, size_t ws_bytes, hipStream_t st) {
+  constexpr int V = VecOf<T>::value;
+  const SmallPlan p = plan_small(AFF ? RowsKind::kBwdAffine : RowsKind::kBwdCols, V, n_rows, D, C, cu_count());
+  ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
+                "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
+  float* part = static_cast<float*>(ws);
+  const int Di = static_cast<int>(D);
+  if (tuning().bwd_stage_mask & 1) {
+    switch (p.NV) {
+      case 1: small_bwd<T, V, 1, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
+      case 2: small_bwd<T, V, 2, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
+      case 3: small_bwd<T, V, 3, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
+      default: small_bwd<T, V, 4, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
+    }
+    ATEXN_CHECK_LAUNCH("small_bwd");
+  }
+  if (!(tuning().bwd_stage_mask & 2)) return ATEXN_OK;
+  return launch_col_reduce(part, dgamma, dbeta, p.part_rows, AFF ? C : D, st);
 }
 
 // LayerNorm rows too long for registers, any D and alignment (tiles_kernels.cuh).
@@ -194,7 +235,11 @@ int rows_fwd_t(bool affine, const void* x_, const float* gamma, const float* bet
   const T* x = static_cast<const T*>(x_);
   T* y = static_cast<T*>(y_);
   // 16-byte accesses need no pointer alignment beyond the element's
-  const RowsRoute route = route_rows(RowsKind::kFwd, !affine, VEC, D);
+  const RowsRoute route = route_rows(RowsKind::kFwd, !affine, VEC, n_rows, D);
+  if (route.small) {
+    return affine ? small_fwd_launch<T, true>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, st)
+                  : small_fwd_launch<T, false>(x, gamma, beta, n_rows, D, C, eps, y, mean, rstd, st);
+  }
   if (route.tiles) {
     return tiles_fwd<T>(x, gamma, beta, n_rows, D, eps, y, mean, rstd, ws, ws_bytes, st);
   }
@@ -215,7 +260,11 @@ int rows_bwd_t(bool affine, const void* dy_, const void* x_, const float* gamma,
   const T* dy = static_cast<const T*>(dy_);
   T* dx = static_cast<T*>(dx_);
   const RowsRoute route =
-      route_rows(affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols, !affine, VEC, D);
+      route_rows(affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols, !affine, VEC, n_rows, D);
+  if (route.small) {
+    return affine ? small_bwd_launch<T, true>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st)
+                  : small_bwd_launch<T, false>(dy, x, gamma, mean, rstd, n_rows, D, C, dx, dgamma, dbeta, ws, ws_bytes, st);
+  }
   if (route.tiles) {
     return tiles_bwd<T>(dy, x, gamma, mean, rstd, n_rows, D, dx, dgamma, dbeta, ws, ws_bytes, st);
   }

@@ -123,6 +123,13 @@ def test_unaligned_pointers(capi, coracle, N, C, S, dtype, channel_first):
     assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16"])
+@pytest.mark.parametrize("N,C,S", [(64, 64, 27), (128, 40, 8), (16, 300, 30), (70, 64, 12)])
+def test_tiny_spatial_channel_first(capi, coracle, N, C, S, dtype):
+    """N * C >= 4096 planes of a few elements each: one thread per (n, c) plane."""
+    run_case(capi, coracle, N, C, S, dtype, True, 27)
+
+
 def test_layout_equivalence(capi):
     """IN over NC... of the transposed tensor equals the transpose of IN over N...C."""
     import torch

@@ -135,6 +135,16 @@ def test_long_rows(capi, coracle, N, D, dtype):
     run_case(capi, coracle, "plain", N, D, dtype, 17)
 
 
+@pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("N,D", [(5000, 4), (4096, 7), (5000, 8), (100000, 10), (4500, 13), (10000, 16), (4100, 31),
+                                 (6000, 32), (7777, 25)])
+def test_many_tiny_rows(capi, coracle, N, D, dtype):
+    """Many rows of a few elements (one thread per row), as in the 10000000 x 10 line of the
+    reference's benchmark table and the D = 11, 12, 16, 31 cases of its tests."""
+    run_case(capi, coracle, "plain", N, D, dtype, 18)
+    run_case(capi, coracle, "plain", N, D, dtype, 18, in_place=True)
+
+
 def test_many_rows_narrow(capi, coracle):
     run_case(capi, coracle, "plain", 100000, 10, "f32", 14)
     run_case(capi, coracle, "plain", 50000, 100, "f16", 14)
