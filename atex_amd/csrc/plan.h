@@ -69,8 +69,8 @@ struct RowsPlan {
 inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kFwd ? 4096 : 2048; }
 
 // Which kernels take a contiguous-row problem.  vec = 16 / sizeof(T).
-//   V = vec: rows of whole vectors, or ragged rows (D % vec != 0, D >= vec) short enough
-//            for the register-resident kernels; V = 1: everything else on the row kernels;
+//   V = vec: rows of at least one vector (a ragged end, D % vec != 0, is handled inside the
+//            kernels); V = 1: rows shorter than a vector;
 //   tiles:   LayerNorm rows beyond the resident limit (any D).
 //   small:   rows of at most 4 vectors when there are many of them: one thread per row.
 struct RowsRoute {
@@ -87,11 +87,7 @@ inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_r
     r.small = true;
     return r;
   }
-  if (D % vec == 0) {
-    r.V = vec;
-  } else if (D >= vec && div_up(D, vec) <= resident_limit(kind)) {
-    r.V = vec;
-  }
+  if (D >= vec) r.V = vec;  // ragged row ends are handled by every vector kernel
   r.tiles = layer_norm && div_up(D, r.V) > resident_limit(kind);
   return r;
 }
@@ -122,7 +118,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   RowsPlan p;
   p.V = V;
   const int64_t n_vec = div_up(D, V);
-  p.ragged = D % V != 0;  // resident kernels only
+  p.ragged = D % V != 0;
   p.resident = n_vec <= resident_limit(kind);
   if (p.resident) {
     if (n_vec <= 64) {

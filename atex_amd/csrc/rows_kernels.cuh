@@ -796,6 +796,24 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
           const int64_t i = split_pos(v, n_vec, rev) * V;
           one(load_pack<T, V>(xp + i), i);
         });
+    // ragged row end (last chunk only): the elements after the last full vector
+    const int rem = static_cast<int>(len % V);
+    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+      const int64_t i = n_vec * V;
+      Pack<T, V> o;
+      const Pack<T, V> pk = load_pack_n<T, V>(xp + i, rem);
+      if constexpr (ROW_AFFINE) {
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = from_f32<T>((to_f32(pk.v[k]) - mean) * a + bs);
+      } else {
+        float tg[V], tb[V];
+        load_f32_n<V>(gp + i, tg, rem);
+        load_f32_n<V>(bp + i, tb, rem);
+#pragma unroll
+        for (int k = 0; k < V; ++k) o.v[k] = from_f32<T>((to_f32(pk.v[k]) - mean) * rstd * tg[k] + tb[k]);
+      }
+      store_pack_n<T, V>(yp + i, o, rem);
+    }
   }
 }
 
@@ -849,6 +867,23 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
           for (int u = 0; u < B; ++u) one(px[u], pd[u], (v + u * step) * V);
         },
         [&](int64_t v) { one(load_pack<T, V>(xp + v * V), load_pack<T, V>(dp + v * V), v * V); });
+    const int rem = static_cast<int>(len % V);
+    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+      // zero-filled dy beyond the row end adds nothing
+      const int64_t i = n_vec * V;
+      const Pack<T, V> px = load_pack_n<T, V>(xp + i, rem);
+      const Pack<T, V> pd = load_pack_n<T, V>(dp + i, rem);
+      float tg[V];
+      if constexpr (!ROW_AFFINE) load_f32_n<V>(gp + i, tg, rem);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        const float xc = to_f32(px.v[k]) - mean;
+        float gv = to_f32(pd.v[k]);
+        if constexpr (!ROW_AFFINE) gv *= tg[k];
+        s1 += gv;
+        s2 += gv * xc;
+      }
+    }
     const float2 r = block_sum2(s1, s2 * rstd, sum_buf[it & 1]);
     if (threadIdx.x == 0) sums[w] = r;
   }
@@ -928,6 +963,22 @@ __global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ 
           const int64_t i = split_pos(v, n_vec, rev) * V;
           one(load_pack<T, V>(xp + i), load_pack<T, V>(dp + i), i);
         });
+    const int rem = static_cast<int>(len % V);
+    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+      const int64_t i = n_vec * V;
+      const Pack<T, V> px = load_pack_n<T, V>(xp + i, rem);
+      const Pack<T, V> pd = load_pack_n<T, V>(dp + i, rem);
+      Pack<T, V> o;
+      float tg[V];
+      if constexpr (!ROW_AFFINE) load_f32_n<V>(gp + i, tg, rem);
+#pragma unroll
+      for (int k = 0; k < V; ++k) {
+        float gv = to_f32(pd.v[k]);
+        if constexpr (!ROW_AFFINE) gv *= tg[k];
+        o.v[k] = from_f32<T>(ca * gv + (cb * (to_f32(px.v[k]) - mean) + cc));
+      }
+      store_pack_n<T, V>(op + i, o, rem);
+    }
   }
 }
 

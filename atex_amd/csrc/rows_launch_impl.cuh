@@ -86,7 +86,7 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
     ATEXN_CHECK_LAUNCH("rows_fwd_resident");
     return ATEXN_OK;
   }
-  if constexpr (AFF) {
+  if constexpr (AFF && V > 1) {
     float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
     split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
     ATEXN_CHECK_LAUNCH("split_fwd_stats");
@@ -96,7 +96,7 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
     ATEXN_CHECK_LAUNCH("split_fwd_apply");
     return ATEXN_OK;
   } else {
-    return set_error(ATEXN_LAUNCH_ERROR, "LayerNorm rows of %lld elements belong to the tile path", (long long)D);
+    return set_error(ATEXN_LAUNCH_ERROR, "rows of %lld elements have no split kernel on this path", (long long)D);
   }
 }
 
@@ -212,7 +212,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     if (!(stages & 2)) return ATEXN_OK;
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
   }
-  if constexpr (AFF) {
+  if constexpr (AFF && V > 1) {
     float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
     split_bwd_sums<T, V, true><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
                                                             D, p.S, p.chunk);
@@ -223,7 +223,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     ATEXN_CHECK_LAUNCH("split_bwd_apply");
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
   } else {
-    return set_error(ATEXN_LAUNCH_ERROR, "LayerNorm rows of %lld elements belong to the tile path", (long long)D);
+    return set_error(ATEXN_LAUNCH_ERROR, "rows of %lld elements have no split kernel on this path", (long long)D);
   }
 }
 
