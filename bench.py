@@ -69,14 +69,14 @@ DEFAULT_CASE = "ln_bert"
 
 # Bytes between L2 and memory per launch of the kernel(s) the roofline object is quoted on,
 # from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, each scaled by
-# what the same counter reads for the 64 MiB copy of --copy-calibration (FETCH_SIZE x 2.0,
+# what the same counter reads for the 64 MiB negation of --copy-calibration (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0).  Summaries: profiles/<case>_hbm_traffic.txt.  Cases without a run: None.
 MEASURED_TRAFFIC = {
     "ln_bert": 52.78e6,                 # rows_bwd_resident
-    "in2d_nchw": 50.49e6,               # rows_bwd_resident (row-affine)
-    "in2d_nhwc": 33.97e6 + 52.59e6,     # cl_bwd_sums + cl_bwd_apply
-    "in3d_ndhwc": 536.94e6 + 806.31e6,  # cl_bwd_sums + cl_bwd_apply
-    "in3d_ncdhw": 536.77e6 + 805.31e6,  # split_bwd_sums + split_bwd_apply
+    "in2d_nchw": 50.50e6,               # rows_bwd_resident (row-affine)
+    "in2d_nhwc": 33.99e6 + 52.59e6,     # cl_bwd_sums + cl_bwd_apply
+    "in3d_ndhwc": 537.00e6 + 806.36e6,  # cl_bwd_sums + cl_bwd_apply
+    "in3d_ncdhw": 536.85e6 + 805.40e6,  # split_bwd_sums + split_bwd_apply
 }
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
@@ -291,6 +291,16 @@ def run_case(name, steps, warmup, with_cpu=True):
     ms_step_hot = case.time_loop(step, steps, warmup)
     case.n_sets = n_sets
 
+    # what plain streaming kernels reach on the same tensors and rotation (torch's elementwise
+    # kernels): a copy (1 read + 1 write, the forward's traffic) and an add (2 reads + 1 write,
+    # the backward's)
+    tensor_bytes = case.sets[0]["x"].numel() * ESIZE[dtype]
+    ms_copy = case.time_loop(lambda i: case.sets[i % case.n_sets]["y"].copy_(case.sets[i % case.n_sets]["x"]),
+                             steps, warmup)
+    torch = case.torch
+    ms_add = case.time_loop(lambda i: torch.add(case.sets[i % case.n_sets]["x"], case.sets[i % case.n_sets]["dy"],
+                                                out=case.sets[i % case.n_sets]["dx"]), steps, warmup)
+
     value = (fb + bb) / (ms_step * 1e-3) / 1e9
     achieved = bb / (ms_bwd_main * 1e-3) / 1e9
     if op == "ln":
@@ -319,6 +329,9 @@ def run_case(name, steps, warmup, with_cpu=True):
                         "fwd_bwd_hot_cache": ms_step_hot * 1e3},
         "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9,
                  "fwd_bwd_hot_cache": (fb + bb) / (ms_step_hot * 1e-3) / 1e9},
+        "streaming_reference": {"copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
+                                "add_us": ms_add * 1e3, "add_gbps": 3 * tensor_bytes / (ms_add * 1e-3) / 1e9,
+                                "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
                      "kernel": roofline_kernel(op, dims),
@@ -337,9 +350,10 @@ def main():
     ap.add_argument("--case", default=DEFAULT_CASE, choices=sorted(CASES) + ["all"])
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--copy-calibration", action="store_true",
-                    help="after the case, run 5 device-to-device copies of 64 MiB (torch's "
-                         "elementwise copy kernel): a kernel of known traffic that scales the "
-                         "FETCH_SIZE / WRITE_SIZE counters of a rocprofv3 --pmc run")
+                    help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
+                         "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
+                         "known traffic that scales the FETCH_SIZE / WRITE_SIZE counters of a "
+                         "rocprofv3 --pmc run")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: the path has no cross-GPU exchange; run with --gpus 1")
@@ -360,7 +374,7 @@ def main():
         src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
         dst = torch.empty_like(src)
         for _ in range(5):
-            dst.copy_(src)
+            torch.neg(src, out=dst)
         torch.cuda.synchronize()
 
 
