@@ -4,7 +4,7 @@
 //
 // It plays the part of the reference's dispatch ladders
 // (fused_layer_norm_op.cu:824-891, :919-1028; fused_instance_norm_op.cu:1203-1561) but
-// decides from alignment, row length and the CU count instead of from occupancy probes
+// decides from row length, row count and the CU count instead of from occupancy probes
 // against a 48 KB shared-memory limit.
 #pragma once
 

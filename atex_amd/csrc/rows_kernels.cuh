@@ -6,10 +6,13 @@
 //             fused_instance_norm_op.cu:169-313, :315-366, :594-656
 // with two designs:
 //   * "resident" kernels: the row lives in VGPRs (TPR threads x VPT 128-bit vectors),
-//     is read from HBM exactly once, and its statistics come from an exact local
-//     two-pass followed by a Chan/Welford butterfly across lanes (and LDS across waves);
-//   * "split" kernels for rows that do not fit or are not 16-byte aligned: a row is cut
-//     into S chunks, stage 1 writes per-chunk partials, stage 2 merges them and applies.
+//     is read from HBM exactly once, and its statistics come from an exact two-pass over
+//     the registers, each pass one all-reduce across the row's lanes (DPP, LDS across waves);
+//   * "split" kernels for channel-first planes that do not fit: a row is cut into S
+//     chunks, stage 1 writes per-chunk partials, stage 2 merges them and applies
+//     (LayerNorm rows that do not fit go to tiles_kernels.cuh, many tiny rows to
+//     small_kernels.cuh).
+// All of them use 16-byte accesses at element alignment; rows may have any length.
 #pragma once
 
 #include "norm_common.cuh"
@@ -629,7 +632,7 @@ col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __re
 // ------------------------------------------------------------------------ split rows
 // A row of D elements is cut into S chunks of `chunk` elements (the last may be short).
 // Work item w = row * S + s; blocks take work items grid-stride.  V = elements per
-// access (16-byte vectors when everything is aligned, 1 otherwise).
+// access (a 16-byte vector; a ragged row end is finished element-wise by one thread).
 //
 // Every loop over a chunk runs in batches of kSplitBatch accesses per thread whose loads are
 // all issued before the first is consumed (a plain strided loop keeps one load per thread

@@ -20,6 +20,9 @@
  *     rsqrt(biased_variance + epsilon) (reference: cc/kernels/norm_util.h:253-258);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); every call is
  *     asynchronous on it, re-entrant, allocates nothing and keeps no device state;
+ *   - data pointers need only the alignment of their element type (2 or 4 bytes): the
+ *     kernels' 16-byte accesses work at any element offset, so slices of larger tensors
+ *     can be passed as they are;
  *   - `workspace` is device scratch of at least *_workspace_bytes(...) bytes, 256-byte
  *     aligned; it may be NULL when that size is 0;
  *   - return value: ATEXN_OK, ATEXN_INVALID_ARGUMENT (nothing launched) or
