@@ -88,6 +88,12 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
     t.bwd_stage_mask = value;
+  } else if (!strcmp(name, "fwd_vpt2_max_vec")) {
+    ATEXN_REQUIRE(value >= 1024 && value <= 2048, "fwd_vpt2_max_vec must be in [1024, 2048]");
+    t.fwd_vpt2_max_vec = value;
+  } else if (!strcmp(name, "bwd_vpt2_max_vec")) {
+    ATEXN_REQUIRE(value >= 1024 && value <= 1536, "bwd_vpt2_max_vec must be in [1024, 1536]");
+    t.bwd_vpt2_max_vec = value;
   } else if (!strcmp(name, "reverse_second_pass")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "reverse_second_pass must be 0 or 1");
     t.reverse_second_pass = value;

@@ -70,23 +70,34 @@ int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_
                       hipStream_t st) {
   ATEXN_REQUIRE(2 * W < (int64_t(1) << 31), "column count %lld too large", (long long)W);
   const int Wi = static_cast<int>(W);
-  // column groups per block: few when there are many partial rows to share among the
-  // threads of a group, one per thread when there are only a handful of rows
+  // Column groups per block (CX): the more, the longer the contiguous run a wave reads per
+  // partial row, but the fewer blocks and the fewer rows in parallel (256 / CX).  Take the
+  // largest CX that still gives every CU a block and every row-lane at least two rows.
+  const int cus = cu_count();
+  auto fits = [&](int cw, int cx) {
+    return div_up(2 * W, int64_t(cw) * cx) >= cus && (256 / cx) * 2 <= std::max(G, 2);
+  };
+#define ATEXN_COL_REDUCE(CW_, CX_)                                                              \
+  col_reduce<CW_, CX_><<<static_cast<int>(div_up(2 * W, int64_t(CW_) * CX_)), kColReduceThreads, \
+                         0, st>>>(part, out0, out1, G, Wi)
   if (W % 4 == 0) {
-    if (G >= 128) {
-      col_reduce<4, 4><<<static_cast<int>(div_up(2 * W, 4 * 4)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
-    } else if (G >= 16) {
-      col_reduce<4, 64><<<static_cast<int>(div_up(2 * W, 4 * 64)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    if (fits(4, 256) || G < 8) {
+      ATEXN_COL_REDUCE(4, 256);
+    } else if (fits(4, 64)) {
+      ATEXN_COL_REDUCE(4, 64);
+    } else if (fits(4, 16)) {
+      ATEXN_COL_REDUCE(4, 16);
     } else {
-      col_reduce<4, 256><<<static_cast<int>(div_up(2 * W, 4 * 256)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+      ATEXN_COL_REDUCE(4, 4);
     }
   } else {
-    if (G >= 64) {
-      col_reduce<1, 16><<<static_cast<int>(div_up(2 * W, 16)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+    if (fits(1, 256) || G < 8) {
+      ATEXN_COL_REDUCE(1, 256);
     } else {
-      col_reduce<1, 256><<<static_cast<int>(div_up(2 * W, 256)), kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi);
+      ATEXN_COL_REDUCE(1, 16);
     }
   }
+#undef ATEXN_COL_REDUCE
   ATEXN_CHECK_LAUNCH("col_reduce");
   return ATEXN_OK;
 }

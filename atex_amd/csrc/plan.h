@@ -31,6 +31,10 @@ struct Tuning {
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
   int reverse_second_pass = 1;
+  // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
+  // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
+  int fwd_vpt2_max_vec = 1024;
+  int bwd_vpt2_max_vec = 1536;
 };
 Tuning& tuning();
 
@@ -129,7 +133,8 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.vpt = 2;
     } else {
       p.tpr = 0;
-      p.vpt = n_vec <= 1024 ? 2 : (n_vec <= 2048 ? 4 : 8);
+      const int vpt2_max = kind == RowsKind::kFwd ? t.fwd_vpt2_max_vec : t.bwd_vpt2_max_vec;
+      p.vpt = n_vec <= vpt2_max ? 2 : (n_vec <= 2048 ? 4 : 8);
     }
     if (p.tpr == 0) {
       p.threads = static_cast<int>(round_up(div_up(n_vec, p.vpt), 64));

@@ -38,10 +38,11 @@ constexpr int kFoldWaves = 4;
 // budget the compiler works against (512 VGPRs per SIMD lane / waves per SIMD).
 template <int TPR, int VPT>
 constexpr int resident_fwd_max_threads() {
-  return TPR != 0 ? 256 : 512;
+  return TPR != 0 ? 256 : (VPT == 2 ? 1024 : 512);
 }
-template <int TPR, bool BWD_COLS, int RB>
+template <int TPR, bool BWD_COLS, int RB, int VPT>
 constexpr int resident_bwd_max_threads() {
+  if (TPR == 0 && VPT == 2) return 768;
   return (TPR != 0 && !BWD_COLS) ? 256 : 512;
 }
 
@@ -281,7 +282,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // dx must not alias dy or x.  RB / EXACT / prefetch as in the forward kernel.
 template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
           bool RAGGED = false>
-__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB>()))
+__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT>()))
 rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* __restrict__ dx,

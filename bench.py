@@ -51,6 +51,8 @@ CASES = {
     "in3d_ncdhw": ("in", "f16", (2, 32, 128 ** 3, True)),
     # shapes of the reference's own benchmark tables (benchmark_layer_norm.py:53-63,
     # benchmark_instance_norm.py:58-69), not part of --case all
+    "ln_8192x10240": ("ln", "f16", (8192, 10240)),
+    "ln_4096x16384": ("ln", "f16", (4096, 16384)),
     "lnref_10x1e7": ("ln", "f16", (10, 10000000)),
     "lnref_100x1e6": ("ln", "f16", (100, 1000000)),
     "lnref_1e3x1e5": ("ln", "f16", (1000, 100000)),
@@ -363,7 +365,7 @@ def main():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
     if args.case == "all":
         for name in CASES:
-            if "ref_" in name:
+            if "ref_" in name or "x1" in name:
                 continue
             steps = args.steps if "3d" not in name else max(10, args.steps // 10)
             r = run_case(name, steps, args.warmup, with_cpu=False)
