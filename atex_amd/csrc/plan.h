@@ -19,7 +19,9 @@ namespace atexn {
 struct Tuning {
   int fwd_waves_per_cu = 16;      // resident forward: waves kept resident per CU
   int bwd_ln_threads = 512;       // resident LayerNorm backward, rows <= one wave: block size
-  int bwd_waves_per_cu = 8;       // resident backward: waves kept resident per CU
+  int bwd_waves_per_cu = 8;       // resident LayerNorm backward: waves kept resident per CU
+                                  //   (each block adds a partial row to the column reduction)
+  int bwd_affine_waves_per_cu = 32;  // resident channel-first backward (no partial rows)
   int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
   int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
   int tile_items_per_cu = 4;      // LayerNorm long rows: (row slab, column tile) tiles per CU
@@ -156,7 +158,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
               n_rows % (int64_t(p.rpb) * p.rb) == 0;
     const int waves = p.threads / 64;
     const int per_cu = std::max(
-        1, (kind == RowsKind::kFwd ? t.fwd_waves_per_cu : t.bwd_waves_per_cu) / waves);
+        1, (kind == RowsKind::kFwd        ? t.fwd_waves_per_cu
+            : kind == RowsKind::kBwdCols ? t.bwd_waves_per_cu
+                                         : t.bwd_affine_waves_per_cu) /
+               waves);
     p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(groups, int64_t(cus) * per_cu)));
     if (kind == RowsKind::kBwdCols) {
       p.part_rows = p.grid;
