@@ -270,6 +270,12 @@ def roofline_kernel(op, dims):
     return "rows_bwd_resident (backward row kernel: dx and the dgamma / dbeta partials)"
 
 
+def torch_mod():
+    import torch
+
+    return torch
+
+
 def run_case(name, steps, warmup, with_cpu=True):
     op, dtype, dims = CASES[name]
     fb, bb = algorithmic_bytes(op, dtype, dims)
@@ -292,6 +298,28 @@ def run_case(name, steps, warmup, with_cpu=True):
     case.n_sets = 1
     ms_step_hot = case.time_loop(step, steps, warmup)
     case.n_sets = n_sets
+
+    # the same fwd + bwd steps captured once into a HIP graph (one pass over all buffer sets)
+    # and replayed: what a caller that captures its step gets
+    ms_step_graph = None
+    try:
+        side = torch_mod().cuda.Stream()
+        side.wait_stream(torch_mod().cuda.current_stream())
+        graph = torch_mod().cuda.CUDAGraph()
+        with torch_mod().cuda.stream(side):
+            old = case.stream
+            case.stream = side.cuda_stream
+            step(0)
+            side.synchronize()
+            with torch_mod().cuda.graph(graph, stream=side):
+                for i in range(case.n_sets):
+                    step(i)
+            case.stream = old
+        torch_mod().cuda.synchronize()
+        reps = max(1, steps // case.n_sets)
+        ms_step_graph = case.time_loop(lambda i: graph.replay(), reps, 2) / case.n_sets
+    except Exception as e:  # graph capture is an extra, never fatal
+        print(f"hip graph timing skipped: {e}", file=sys.stderr)
 
     # what plain streaming kernels reach on the same tensors and rotation (torch's elementwise
     # kernels): a copy (1 read + 1 write, the forward's traffic) and an add (2 reads + 1 write,
@@ -328,7 +356,8 @@ def run_case(name, steps, warmup, with_cpu=True):
                    "algorithmic_bytes_fwd": fb, "algorithmic_bytes_bwd": bb},
         "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
         "us_per_call": {"fwd": ms_fwd * 1e3, "bwd": ms_bwd * 1e3, "fwd_bwd": ms_step * 1e3,
-                        "fwd_bwd_hot_cache": ms_step_hot * 1e3},
+                        "fwd_bwd_hot_cache": ms_step_hot * 1e3,
+                        "fwd_bwd_hip_graph": None if ms_step_graph is None else ms_step_graph * 1e3},
         "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9,
                  "fwd_bwd_hot_cache": (fb + bb) / (ms_step_hot * 1e-3) / 1e9},
         "streaming_reference": {"copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
