@@ -31,13 +31,19 @@ struct ClGeom {
   int s;           // slab
   int ct;          // channel tile
   int cvi;         // channel-vector index of this thread
+  int coff;        // first channel of the thread's vector: cvi * V, except that the last
+                   //   vector of a C that is not a multiple of V starts at C - V (it overlaps
+                   //   its neighbour) and owns only its elements lo .. V-1
+  int lo;
   int slot;        // pixel slot inside the block
   int ppb;         // pixel slots per block
   bool ch_ok;      // channel vector inside C
   int64_t p0, p1;  // pixel range of the slab
 };
 
-__device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int64_t D, int64_t slab_len) {
+template <bool RG>
+__device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, int64_t D,
+                                          int64_t slab_len) {
   ClGeom g;
   g.n = blockIdx.x;
   g.s = static_cast<int>(blockIdx.y);
@@ -47,6 +53,14 @@ __device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int64_t D, int6
   g.slot = t >> tpp_shift;
   g.ppb = kClThreads >> tpp_shift;
   g.ch_ok = g.cvi < CV;
+  const int nominal = (g.ch_ok ? g.cvi : CV - 1) * V;
+  if constexpr (RG) {  // C is not a multiple of V (and C >= V)
+    g.coff = nominal + V <= C ? nominal : C - V;
+    g.lo = g.ch_ok ? nominal - g.coff : 0;
+  } else {
+    g.coff = nominal;
+    g.lo = 0;
+  }
   g.p0 = static_cast<int64_t>(g.s) * slab_len;
   g.p1 = g.p0 + slab_len < D ? g.p0 + slab_len : D;
   return g;
@@ -150,7 +164,7 @@ __device__ __forceinline__ void cl_for_pixels(const ClGeom& g, Full&& full, Tail
 template <typename T, int V, int U>
 __device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, int CV, int C,
                                              Pack<T, V> (&raw)[U], bool (&ok)[U]) {
-  const T* b = base_n + static_cast<int64_t>(g.ch_ok ? g.cvi : CV - 1) * V;
+  const T* b = base_n + g.coff;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     const int64_t p = g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb;
@@ -182,7 +196,7 @@ __device__ __forceinline__ void cl_pivot(const T* xn_c, int64_t D, int C, float 
 // is saved to pivot[N, C].
 // U > 0: the slab is register-resident (slab_len <= U * pixel slots per block) and all its
 // loads are in flight at once; U == 0 streams the slab in batches.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict__ ps2,
              float* __restrict__ pivot, int64_t D, int C, int S, int tpp_shift,
@@ -190,10 +204,10 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict
   __shared__ float lds[2 * V * kClThreads];
   const int CV = (C + V - 1) / V;
   const int TPP = 1 << tpp_shift;
-  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   const T* xn = x + (g.n * D) * C;
   float k0[V];
-  cl_pivot<T, V>(xn + static_cast<int64_t>(g.ch_ok ? g.cvi : CV - 1) * V, D, C, k0);
+  cl_pivot<T, V>(xn + g.coff, D, C, k0);
   float acc[2 * V];
 #pragma unroll
   for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
@@ -212,7 +226,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict
 #pragma unroll
     for (int u = 0; u < U; ++u) add(raw[u], ok[u]);
   } else if (g.ch_ok) {
-    const T* base = xn + static_cast<int64_t>(g.cvi) * V;
+    const T* base = xn + g.coff;
     constexpr int B = 8;
     cl_for_pixels<B>(
         g,
@@ -233,18 +247,18 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict
       t1[i] = acc[i];
       t2[i] = acc[V + i];
     }
-    const int64_t o = (g.n * S + g.s) * C + static_cast<int64_t>(g.cvi) * V;
-    store_f32<V>(ps1 + o, t1);
-    store_f32<V>(ps2 + o, t2);
+    const int64_t o = (g.n * S + g.s) * C + g.coff;
+    store_f32_from<V>(ps1 + o, t1, RG ? g.lo : 0);
+    store_f32_from<V>(ps2 + o, t2, RG ? g.lo : 0);
     // stage 2 must not re-read the pivot from x: y may alias x and be half written by then
-    if (g.s == 0) store_f32<V>(pivot + g.n * C + static_cast<int64_t>(g.cvi) * V, k0);
+    if (g.s == 0) store_f32_from<V>(pivot + g.n * C + g.coff, k0, RG ? g.lo : 0);
   }
 }
 
 // ---------------------------------------------------------------- forward, stage 2
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict__ ps2,
              const float* __restrict__ pivot, const float* __restrict__ gamma,
@@ -258,7 +272,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
   const int cap = TPP * V;
   const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
-  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   // resident slab: its loads are issued first and fly while the partials are folded
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
@@ -317,16 +331,18 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
   __syncthreads();
   // phase B: apply
   if (g.ch_ok) {
-    const int cl0 = (g.cvi - (g.ct << tpp_shift)) * V;
+    // channel of element i inside the tile; elements the thread does not own may fall before
+    // the tile (their results are never stored)
+    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
     float mean[V], sc[V], bt[V];
-    load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, sc);
-    load_f32<V>(beta + static_cast<int64_t>(g.cvi) * V, bt);
+    load_f32<V>(gamma + g.coff, sc);
+    load_f32<V>(beta + g.coff, bt);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      mean[i] = sm_mean[cl0 + i];
-      sc[i] *= sm_rstd[cl0 + i];
+      mean[i] = sm_mean[RG && cl0 + i < 0 ? 0 : cl0 + i];
+      sc[i] *= sm_rstd[RG && cl0 + i < 0 ? 0 : cl0 + i];
     }
-    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& pk, int64_t p) {
       Pack<T, V> o;
 #pragma unroll
@@ -335,7 +351,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
         // |mean| >> std
         o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * sc[i] + bt[i]);
       }
-      store_pack<T, V>(y + boff + p * C, o);
+      store_pack_from<T, V>(y + boff + p * C, o, RG ? g.lo : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll
@@ -369,7 +385,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
 
 // --------------------------------------------------------------- backward, stage 1
 // part[(n * S + s)][0][c] = sum dy * xh, part[...][1][c] = sum dy over the slab.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
             const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
@@ -378,7 +394,7 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
   __shared__ float lds[2 * V * kClThreads];
   const int CV = (C + V - 1) / V;
   const int TPP = 1 << tpp_shift;
-  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   float acc[2 * V];
 #pragma unroll
   for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
@@ -392,8 +408,8 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
   for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
   if (g.ch_ok) {
-    load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
-    load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
+    load_f32<V>(mean_in + g.n * C + g.coff, mu);
+    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
   }
   auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, bool valid) {
 #pragma unroll
@@ -408,7 +424,7 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 #pragma unroll
     for (int u = 0; u < U; ++u) add(rx[u], rd[u], ok[u]);
   } else if (g.ch_ok) {
-    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    const int64_t boff = (g.n * D) * C + g.coff;
     constexpr int B = 4;
     cl_for_pixels<B>(
         g,
@@ -428,15 +444,15 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
   }
   cl_block_sum<2 * V>(acc, lds, TPP);
   if (g.ch_ok && g.slot == 0) {
-    float* o = part + ((g.n * S + g.s) * 2) * C + static_cast<int64_t>(g.cvi) * V;
+    float* o = part + ((g.n * S + g.s) * 2) * C + g.coff;
     float t0[V], t1[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       t0[i] = acc[i];
       t1[i] = acc[V + i];
     }
-    store_f32<V>(o, t0);
-    store_f32<V>(o + C, t1);
+    store_f32_from<V>(o, t0, RG ? g.lo : 0);
+    store_f32_from<V>(o + C, t1, RG ? g.lo : 0);
   }
 }
 
@@ -446,7 +462,7 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 // the S slab partials of its instance and channel tile into LDS.  The 2 C outputs of
 // dgamma / dbeta are dealt out over the blocks, each a block-wide sum of one column of
 // all N * S partial rows (fixed order, no atomics), which spares a third launch.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
@@ -461,7 +477,7 @@ cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __r
   const int cap = TPP * V;
   const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
-  const ClGeom g = cl_geom(tpp_shift, CV, D, slab_len);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   // resident slab: its loads are issued first and fly while the partials are folded
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool okp[U > 0 ? U : 1];
@@ -535,18 +551,20 @@ cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __r
   }
   __syncthreads();
   if (g.ch_ok) {
-    const int cl0 = (g.cvi - (g.ct << tpp_shift)) * V;
+    // channel of element i inside the tile; elements the thread does not own may fall before
+    // the tile (their results are never stored)
+    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
     float mu[V], rs[V], sc[V], ca[V], cb[V];
-    load_f32<V>(mean_in + g.n * C + static_cast<int64_t>(g.cvi) * V, mu);
-    load_f32<V>(rstd_in + g.n * C + static_cast<int64_t>(g.cvi) * V, rs);
-    load_f32<V>(gamma + static_cast<int64_t>(g.cvi) * V, sc);
+    load_f32<V>(mean_in + g.n * C + g.coff, mu);
+    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
+    load_f32<V>(gamma + g.coff, sc);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       sc[i] *= rs[i];
-      ca[i] = -sc[i] * (sm_b[cl0 + i] * inv_d);
-      cb[i] = -sc[i] * (sm_a[cl0 + i] * inv_d);
+      ca[i] = -sc[i] * (sm_b[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
+      cb[i] = -sc[i] * (sm_a[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
     }
-    const int64_t boff = (g.n * D) * C + static_cast<int64_t>(g.cvi) * V;
+    const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t p) {
       Pack<T, V> o;
 #pragma unroll
@@ -554,7 +572,7 @@ cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __r
         const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
         o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * xh + cb[i]));
       }
-      store_pack<T, V>(dx + boff + p * C, o);
+      store_pack_from<T, V>(dx + boff + p * C, o, RG ? g.lo : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll

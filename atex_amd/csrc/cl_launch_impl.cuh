@@ -20,23 +20,26 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   const int Ci = static_cast<int>(C);
   ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
-#define ATEXN_CL_FWD(U_)                                                                       \
+#define ATEXN_CL_FWD(U_, RG_)                                                                  \
   do {                                                                                        \
-    cl_fwd_stats<T, V, U_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, D, Ci, p.S,        \
+    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, D, Ci, p.S,   \
                                                        p.tpp_shift, p.slab_len);              \
     ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
-    cl_fwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, gamma, beta, y,    \
+    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, gamma, beta, y, \
                                                        mean, rstd, D, Ci, p.S, p.tpp_shift,   \
                                                        p.slab_len, eps,                       \
                                                        tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
-    if (p.U == 4) { ATEXN_CL_FWD(4); return ATEXN_OK; }
-    if (p.U == 8) { ATEXN_CL_FWD(8); return ATEXN_OK; }
-    if (p.U == 16) { ATEXN_CL_FWD(16); return ATEXN_OK; }
+    // a channel count that is not a multiple of V: streaming kernels with an overlapping
+    // last channel vector
+    if (C % V != 0) { ATEXN_CL_FWD(0, true); return ATEXN_OK; }
+    if (p.U == 4) { ATEXN_CL_FWD(4, false); return ATEXN_OK; }
+    if (p.U == 8) { ATEXN_CL_FWD(8, false); return ATEXN_OK; }
+    if (p.U == 16) { ATEXN_CL_FWD(16, false); return ATEXN_OK; }
   }
-  ATEXN_CL_FWD(0);
+  ATEXN_CL_FWD(0, false);
 #undef ATEXN_CL_FWD
   return ATEXN_OK;
 }
@@ -52,22 +55,23 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   const int Ci = static_cast<int>(C);
   ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
-#define ATEXN_CL_BWD(U_)                                                                       \
+#define ATEXN_CL_BWD(U_, RG_)                                                                  \
   do {                                                                                        \
-    cl_bwd_sums<T, V, U_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S,      \
+    cl_bwd_sums<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S, \
                                                       p.tpp_shift, p.slab_len);               \
     ATEXN_CHECK_LAUNCH("cl_bwd_sums");                                                        \
-    cl_bwd_apply<T, V, U_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx,      \
+    cl_bwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx, \
                                                        dgamma, dbeta, N, D, Ci, p.S,          \
                                                        p.tpp_shift, p.slab_len,               \
                                                        tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
-    if (p.U == 4) { ATEXN_CL_BWD(4); return ATEXN_OK; }
-    if (p.U == 8) { ATEXN_CL_BWD(8); return ATEXN_OK; }
+    if (C % V != 0) { ATEXN_CL_BWD(0, true); return ATEXN_OK; }
+    if (p.U == 4) { ATEXN_CL_BWD(4, false); return ATEXN_OK; }
+    if (p.U == 8) { ATEXN_CL_BWD(8, false); return ATEXN_OK; }
   }
-  ATEXN_CL_BWD(0);
+  ATEXN_CL_BWD(0, false);
 #undef ATEXN_CL_BWD
   return ATEXN_OK;
 }
@@ -79,7 +83,9 @@ int cl_fwd_t(const void* x_, const float* gamma, const float* beta, int64_t N, i
   constexpr int VEC = VecOf<T>::value;
   const T* x = static_cast<const T*>(x_);
   T* y = static_cast<T*>(y_);
-  const bool vec = C % VEC == 0;  // 16-byte accesses work at element alignment
+  // 16-byte accesses work at element alignment; a C that is not a multiple of the vector
+  // width is covered by an overlapping last vector
+  const bool vec = C >= VEC;
   return vec ? cl_fwd_v<T, VEC>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st)
              : cl_fwd_v<T, 1>(x, gamma, beta, N, C, D, eps, y, mean, rstd, ws, ws_bytes, st);
 }
@@ -92,7 +98,7 @@ int cl_bwd_t(const void* dy_, const void* x_, const float* gamma, const float* m
   const T* x = static_cast<const T*>(x_);
   const T* dy = static_cast<const T*>(dy_);
   T* dx = static_cast<T*>(dx_);
-  const bool vec = C % VEC == 0;
+  const bool vec = C >= VEC;
   return vec ? cl_bwd_v<T, VEC>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st)
              : cl_bwd_v<T, 1>(dy, x, gamma, mean, rstd, N, C, D, dx, dgamma, dbeta, ws, ws_bytes, st);
 }

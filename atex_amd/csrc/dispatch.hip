@@ -178,7 +178,7 @@ size_t rows_bwd_ws(int dtype, bool affine, int64_t n_rows, int64_t D, int C) {
 static size_t cl_ws(bool bwd, int dtype, int64_t N, int64_t C, int64_t D) {
   if (N <= 0 || C <= 0 || D <= 0) return 0;
   const int vec = 16 / elem_size(dtype);
-  return plan_cl(bwd, C % vec == 0 ? vec : 1, N, C, D, cu_count()).ws_bytes;
+  return plan_cl(bwd, C >= vec ? vec : 1, N, C, D, cu_count()).ws_bytes;
 }
 size_t cl_fwd_ws(int dtype, int64_t N, int64_t C, int64_t D) { return cl_ws(false, dtype, N, C, D); }
 size_t cl_bwd_ws(int dtype, int64_t N, int64_t C, int64_t D) { return cl_ws(true, dtype, N, C, D); }

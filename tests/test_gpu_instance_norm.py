@@ -83,7 +83,7 @@ def test_non_typical_spatial(capi, coracle, spatial, channel_first):
 
 @pytest.mark.parametrize("channel_first", [False, True])
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
-@pytest.mark.parametrize("C", [1, 3, 5, 24, 48, 100, 256, 520])
+@pytest.mark.parametrize("C", [1, 3, 5, 9, 12, 17, 24, 48, 100, 255, 256, 520, 2049])
 def test_channel_counts(capi, coracle, C, dtype, channel_first):
     # channel counts that are not a multiple of the vector width or not a power of two
     run_case(capi, coracle, 3, C, 777, dtype, channel_first, 22)
