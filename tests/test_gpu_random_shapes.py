@@ -1,0 +1,101 @@
+"""Seeded sweep over random shapes, dtypes, layouts, alignments and in-place use: every kernel
+family and every boundary between them (resident / tiles / small / split / channels-last,
+exact / non-exact / ragged) is crossed many times, each case checked against the oracle."""
+import numpy as np
+import pytest
+
+from tests import util
+from tests.util import TOL, assert_close
+
+pytestmark = pytest.mark.gpu
+
+EPS = 1e-3
+
+
+def _pick_d(rng):
+    kind = rng.integers(0, 6)
+    if kind == 0:
+        return int(rng.integers(1, 40))                       # tiny rows
+    if kind == 1:
+        return int(rng.integers(40, 1100))                    # sub-wave / one-wave rows
+    if kind == 2:
+        return int(8 * rng.integers(16, 2100))                # whole vectors, block-wide rows
+    if kind == 3:
+        return int(rng.integers(1100, 17000))                 # ragged block-wide rows
+    if kind == 4:
+        return int(rng.integers(16000, 40000))                # around the resident limits
+    return int(rng.integers(40000, 300000))                   # long rows
+
+
+def _check(got, ref, dy, gamma, rstd, dtype):
+    y, m, r, dx, dg, db = got
+    y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref = ref
+    tol = TOL[dtype]
+    assert_close(util.to_host(m), m_ref, tol["stat"], "mean")
+    assert_close(util.to_host(r), r_ref, tol["stat"], "inv_std")
+    assert_close(util.to_host(y), y_ref, tol["y"], "y")
+    scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), rstd, dtype)
+    assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx", scale=scale)
+    assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+    assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_layer_norm_random(coracle, seed):
+    import torch
+
+    capi = util.Capi()
+    rng = np.random.Generator(np.random.PCG64(5000 + seed))
+    D = _pick_d(rng)
+    budget = 3_000_000
+    N = int(rng.integers(1, max(2, min(20000, budget // D))))
+    if D <= 32 and rng.random() < 0.5:
+        N = int(rng.integers(4096, 30000))                    # the thread-per-row kernels
+    dtype = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+    mis = bool(rng.integers(0, 2))
+    in_place = bool(rng.integers(0, 2))
+    print(f"LN random seed={seed} N={N} D={D} dtype={dtype} misaligned={mis} in_place={in_place}", flush=True)
+    x, gamma, beta, dy = util.ln_inputs("row_mean", N, D, dtype, 100 + seed)
+    y_ref, m_ref, r_ref = coracle.ln_fwd(x, gamma, beta, EPS, dtype)
+    wrap = util.misalign if mis else (lambda t: t)
+    xd, dyd = wrap(util.to_device(x, dtype)), wrap(util.to_device(dy, dtype))
+    gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
+    x_keep = xd.clone() if in_place else xd
+    y, m, r = capi.ln_fwd(xd, gd, bd, EPS, dtype, y=xd if in_place else None)
+    torch.cuda.synchronize()
+    dx_ref, dg_ref, db_ref = coracle.ln_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype)
+    dx, dg, db = capi.ln_bwd(dyd, x_keep, gd, m, r, dtype)
+    torch.cuda.synchronize()
+    _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
+
+
+@pytest.mark.parametrize("seed", range(48))
+def test_instance_norm_random(coracle, seed):
+    import torch
+
+    capi = util.Capi()
+    rng = np.random.Generator(np.random.PCG64(7000 + seed))
+    cf = bool(rng.integers(0, 2))
+    C = int([rng.integers(1, 9), rng.integers(8, 70), 8 * rng.integers(1, 40), rng.integers(60, 600)][int(rng.integers(0, 4))])
+    S = _pick_d(rng) if cf else int([rng.integers(1, 50), rng.integers(50, 5000), rng.integers(5000, 60000)][int(rng.integers(0, 3))])
+    budget = 3_000_000
+    N = int(rng.integers(1, max(2, min(64, budget // (C * S) + 1))))
+    if C * S * N > 2 * budget:
+        S = max(1, 2 * budget // (C * N))
+    dtype = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+    mis = bool(rng.integers(0, 2))
+    in_place = bool(rng.integers(0, 2))
+    print(f"IN random seed={seed} N={N} C={C} spatial={S} dtype={dtype} channel_first={cf} misaligned={mis} "
+          f"in_place={in_place}", flush=True)
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, cf, 200 + seed)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, cf)
+    wrap = util.misalign if mis else (lambda t: t)
+    xd, dyd = wrap(util.to_device(x, dtype)), wrap(util.to_device(dy, dtype))
+    gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
+    x_keep = xd.clone() if in_place else xd
+    y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, cf, y=xd if in_place else None)
+    torch.cuda.synchronize()
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, cf)
+    dx, dg, db = capi.in_bwd(dyd, x_keep, gd, m, r, dtype, cf)
+    torch.cuda.synchronize()
+    _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
