@@ -89,6 +89,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
     t.bwd_stage_mask = value;
+  } else if (!strcmp(name, "bwd_wave_groups")) {
+    ATEXN_REQUIRE(value == 1 || value == 2, "bwd_wave_groups must be 1 (on) or 2 (off)");
+    t.bwd_wave_groups = value == 1;
   } else if (!strcmp(name, "fwd_vpt2_max_vec")) {
     ATEXN_REQUIRE(value >= 1024 && value <= 2048, "fwd_vpt2_max_vec must be in [1024, 2048]");
     t.fwd_vpt2_max_vec = value;

@@ -289,6 +289,26 @@ __device__ __forceinline__ float2 block_sum2(float a, float b, float2* buf) {
   return r;
 }
 
+// All-reduce of two sums over each group of WPG consecutive waves of the block (a row held
+// by WPG * 64 threads); same buffer contract as block_sum2.  Every wave of the block must
+// call it (it contains a block-wide barrier).
+template <int WPG>
+__device__ __forceinline__ float2 wavegroup_sum2(float a, float b, float2* buf) {
+  a = group_sum<kWave>(a);
+  b = group_sum<kWave>(b);
+  const int wave = threadIdx.x / kWave;
+  if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = make_float2(a, b);
+  __syncthreads();
+  const int first = wave / WPG * WPG;
+  float2 r = buf[first];
+#pragma unroll
+  for (int i = 1; i < WPG; ++i) {
+    r.x += buf[first + i].x;
+    r.y += buf[first + i].y;
+  }
+  return r;
+}
+
 // Block-wide all-reduce of one sum, same contract (`buf` holds 16 floats).
 __device__ __forceinline__ float block_sum1(float a, float* buf) {
   a = group_sum<kWave>(a);

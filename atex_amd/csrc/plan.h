@@ -35,6 +35,7 @@ struct Tuning {
   int reverse_second_pass = 1;
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
+  int bwd_wave_groups = 1;  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   int fwd_vpt2_max_vec = 1024;
   int bwd_vpt2_max_vec = 1536;
 };
@@ -72,7 +73,9 @@ struct RowsPlan {
 // Longest row, in vectors, that the register-resident kernels take: forward 8 vectors per
 // thread at 512 threads, backward 4 (it holds x and dy, and LayerNorm also gamma and the
 // dgamma / dbeta accumulators of its columns).
-inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kFwd ? 4096 : 2048; }
+// The channel-first InstanceNorm backward has no such accumulators and goes as far as the
+// forward.
+inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kBwdCols ? 2048 : 4096; }
 
 // Which kernels take a contiguous-row problem.  vec = 16 / sizeof(T).
 //   V = vec: rows of at least one vector (a ragged end, D % vec != 0, is handled inside the
@@ -133,12 +136,21 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     } else if (n_vec <= 128) {
       p.tpr = 64;
       p.vpt = 2;
+    } else if (kind == RowsKind::kBwdCols && V > 1 && n_vec <= 512 && t.bwd_wave_groups &&
+               n_rows >= int64_t(cus) * (n_vec <= 256 ? 4 : 2)) {
+      // LayerNorm backward: 512-thread blocks with 2 or 4 waves per row, so that a block
+      // still covers several rows (one dgamma / dbeta partial row per block)
+      p.tpr = n_vec <= 256 ? 128 : 256;
+      p.vpt = 2;
     } else {
       p.tpr = 0;
       const int vpt2_max = kind == RowsKind::kFwd ? t.fwd_vpt2_max_vec : t.bwd_vpt2_max_vec;
       p.vpt = n_vec <= vpt2_max ? 2 : (n_vec <= 2048 ? 4 : 8);
     }
-    if (p.tpr == 0) {
+    if (p.tpr > 64) {
+      p.threads = 512;
+      p.rpb = p.threads / p.tpr;
+    } else if (p.tpr == 0) {
       p.threads = static_cast<int>(round_up(div_up(n_vec, p.vpt), 64));
       p.rpb = 1;
     } else {

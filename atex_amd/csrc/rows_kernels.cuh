@@ -20,7 +20,8 @@
 namespace atexn {
 
 // Geometry of the thread <-> row mapping.  TPR > 0: TPR (power of two <= 64) lanes per
-// row and blockDim.x / TPR rows per block.  TPR == 0: the whole block owns one row.
+// row and blockDim.x / TPR rows per block; TPR = 128 or 256 (backward only): a row is held
+// by 2 or 4 consecutive waves.  TPR == 0: the whole block owns one row.
 template <int TPR>
 struct RowMap {
   __device__ __forceinline__ static int tpr() { return TPR ? TPR : static_cast<int>(blockDim.x); }
@@ -43,6 +44,7 @@ constexpr int resident_fwd_max_threads() {
 template <int TPR, bool BWD_COLS, int RB, int VPT>
 constexpr int resident_bwd_max_threads() {
   if (TPR == 0 && VPT == 2) return 768;
+  if (TPR > 64) return 512;
   return (TPR != 0 && !BWD_COLS) ? 256 : 512;
 }
 
@@ -290,7 +292,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
   static_assert(!(RAGGED && (EXACT || RB != 1 || V == 1)), "ragged rows use the plain variant");
-  static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
+  static_assert((TPR != 0 && TPR <= kWave) || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float2 sum_buf[2][16];
   // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats
   extern __shared__ float fold_buf[];
@@ -409,9 +411,13 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
     }
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      if constexpr (TPR != 0) {
-        s1[r] = group_sum<(TPR ? TPR : 1)>(s1[r]);
-        s2[r] = group_sum<(TPR ? TPR : 1)>(s2[r]);
+      if constexpr (TPR > kWave) {
+        const float2 t = wavegroup_sum2<TPR / kWave>(s1[r], s2[r], sum_buf[it & 1]);
+        s1[r] = t.x;
+        s2[r] = t.y;
+      } else if constexpr (TPR != 0) {
+        s1[r] = group_sum<(TPR && TPR <= kWave ? TPR : 1)>(s1[r]);
+        s2[r] = group_sum<(TPR && TPR <= kWave ? TPR : 1)>(s2[r]);
       } else {
         const float2 t = block_sum2(s1[r], s2[r], sum_buf[it & 1]);
         s1[r] = t.x;
@@ -494,8 +500,10 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
       const int lane = threadIdx.x & (kWave - 1);
       const int wave = threadIdx.x / kWave;
       const int nw = blockDim.x / kWave;
-      // (at most kFoldWaves waves' worth of LDS is used per step)
-      for (int half = nw / 2; half >= 1; half >>= 1) {
+      // (at most kFoldWaves waves' worth of LDS is used per step); waves w and w + half own
+      // the same columns as long as half is a multiple of the waves per row
+      constexpr int WPG = TPR > kWave ? TPR / kWave : 1;
+      for (int half = nw / 2; half >= WPG; half >>= 1) {
         for (int base = 0; base < half; base += kFoldWaves) {
           const int src_wave = wave - half - base;  // index among the writers of this step
           if (src_wave >= 0 && src_wave < kFoldWaves && wave < 2 * half) {
@@ -519,7 +527,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
           __syncthreads();
         }
       }
-      if (wave == 0 && lane < tpr) {
+      if (wave < WPG && static_cast<int>(threadIdx.x) < tpr) {
 #pragma unroll
         for (int k = 0; k < VPT; ++k) {
           if (vec_ok[k]) {

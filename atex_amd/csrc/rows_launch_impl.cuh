@@ -35,7 +35,7 @@ template <typename T, int V, int TPR, int VPT, bool AFF>
 BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
     if (ragged) return rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF, true>;
-    if constexpr (TPR != 0) {
+    if constexpr (TPR != 0 && TPR <= 64) {
       if (rb == 2) return exact ? rows_bwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF>;
     }
     if (rb == 1 && exact) return rows_bwd_resident<T, V, TPR, VPT, 1, true, AFF>;
@@ -66,8 +66,15 @@ BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact,
   if (tpr == 32) return bwd_variant<T, V, 32, 1, AFF>(rb, exact, ragged);
   if (tpr == 64 && vpt == 1) return bwd_variant<T, V, 64, 1, AFF>(rb, exact, ragged);
   if (tpr == 64 && vpt == 2) return bwd_variant<T, V, 64, 2, AFF>(rb, exact, ragged);
+  if constexpr (!AFF) {  // LayerNorm: rows held by 2 or 4 waves of a 512-thread block
+    if (tpr == 128 && vpt == 2) return bwd_variant<T, V, 128, 2, AFF>(1, exact, ragged);
+    if (tpr == 256 && vpt == 2) return bwd_variant<T, V, 256, 2, AFF>(1, exact, ragged);
+  }
   if (tpr == 0 && vpt == 2) return bwd_variant<T, V, 0, 2, AFF>(rb, exact, ragged);
   if (tpr == 0 && vpt == 4) return bwd_variant<T, V, 0, 4, AFF>(rb, exact, ragged);
+  if constexpr (AFF) {
+    if (tpr == 0 && vpt == 8) return bwd_variant<T, V, 0, 8, AFF>(rb, exact, ragged);
+  }
   return nullptr;
 }
 

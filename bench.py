@@ -51,6 +51,12 @@ CASES = {
     "in3d_ncdhw": ("in", "f16", (2, 32, 128 ** 3, True)),
     # shapes of the reference's own benchmark tables (benchmark_layer_norm.py:53-63,
     # benchmark_instance_norm.py:58-69), not part of --case all
+    "ln_8192x1024_f32": ("ln", "f32", (8192, 1024)),
+    "ln_8192x2048_f16": ("ln", "f16", (8192, 2048)),
+    "ln_8192x768_f16": ("ln", "f16", (8192, 768)),
+    "ln_8192x1536_f16": ("ln", "f16", (8192, 1536)),
+    "in2d_nhwc_f32": ("in", "f32", (8, 64, 128 * 128, False)),
+    "in2d_nchw_f32": ("in", "f32", (8, 64, 128 * 128, True)),
     "ln_8192x10240": ("ln", "f16", (8192, 10240)),
     "ln_4096x16384": ("ln", "f16", (4096, 16384)),
     "lnref_10x1e7": ("ln", "f16", (10, 10000000)),
@@ -394,7 +400,7 @@ def main():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
     if args.case == "all":
         for name in CASES:
-            if "ref_" in name or "x1" in name:
+            if "ref_" in name or "x1" in name or "x2" in name or "x7" in name or name.endswith("_f32"):
                 continue
             steps = args.steps if "3d" not in name else max(10, args.steps // 10)
             r = run_case(name, steps, args.warmup, with_cpu=False)
