@@ -12,6 +12,7 @@
 #include <stdint.h>
 
 #include <algorithm>
+#include <climits>
 
 namespace atexn {
 
@@ -130,18 +131,29 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   p.ragged = D % V != 0;
   p.resident = n_vec <= resident_limit(kind);
   if (p.resident) {
-    if (n_vec <= 64) {
-      p.tpr = std::max(8, pow2_ceil(n_vec));
-      p.vpt = 1;
-    } else if (n_vec <= 128) {
-      p.tpr = 64;
-      p.vpt = 2;
+    // Rows of up to 192 vectors sit on a group of 8..64 lanes with 1, 2 or 3 vectors per lane:
+    // the candidate with the fewest slots wins (3 vectors per lane make the 3 * 2^k hidden
+    // sizes, 768, 1536, ..., exact), ties go to fewer vectors per lane.
+    int64_t best_slots = INT64_MAX;
+    if (V > 1 || n_vec <= 8) {
+      for (int vpt = 1; vpt <= (V > 1 ? 3 : 1); ++vpt) {
+        const int tpr = std::max(8, pow2_ceil(div_up(n_vec, vpt)));
+        if (tpr > 64 || (vpt == 2 && tpr != 64)) continue;
+        if (int64_t(tpr) * vpt < best_slots) {
+          best_slots = int64_t(tpr) * vpt;
+          p.tpr = tpr;
+          p.vpt = vpt;
+        }
+      }
+    }
+    if (best_slots != INT64_MAX) {
+      // chosen above
     } else if (kind == RowsKind::kBwdCols && V > 1 && n_vec <= 512 && t.bwd_wave_groups &&
                n_rows >= int64_t(cus) * (n_vec <= 256 ? 4 : 2)) {
       // LayerNorm backward: 512-thread blocks with 2 or 4 waves per row, so that a block
       // still covers several rows (one dgamma / dbeta partial row per block)
-      p.tpr = n_vec <= 256 ? 128 : 256;
-      p.vpt = 2;
+      p.tpr = n_vec <= 256 ? 128 : (n_vec <= 384 ? 128 : 256);
+      p.vpt = n_vec <= 256 ? 2 : (n_vec <= 384 ? 3 : 2);
     } else {
       p.tpr = 0;
       const int vpt2_max = kind == RowsKind::kFwd ? t.fwd_vpt2_max_vec : t.bwd_vpt2_max_vec;

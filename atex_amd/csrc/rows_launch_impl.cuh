@@ -46,7 +46,16 @@ BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact, bool ragged) {
 template <typename T, int V, bool AFF>
 FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb, bool exact, bool ragged) {
   // element-wise rows are only the ones shorter than a vector
-  if constexpr (V == 1) return tpr == 8 && vpt == 1 ? fwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  if constexpr (V == 1) {
+    return tpr == 8 && vpt == 1 ? fwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  } else {
+  if (vpt == 3) {
+    if (tpr == 8) return fwd_variant<T, V, 8, 3, AFF>(rb, exact, ragged);
+    if (tpr == 16) return fwd_variant<T, V, 16, 3, AFF>(rb, exact, ragged);
+    if (tpr == 32) return fwd_variant<T, V, 32, 3, AFF>(rb, exact, ragged);
+    if (tpr == 64) return fwd_variant<T, V, 64, 3, AFF>(rb, exact, ragged);
+    return nullptr;
+  }
   if (tpr == 8) return fwd_variant<T, V, 8, 1, AFF>(rb, exact, ragged);
   if (tpr == 16) return fwd_variant<T, V, 16, 1, AFF>(rb, exact, ragged);
   if (tpr == 32) return fwd_variant<T, V, 32, 1, AFF>(rb, exact, ragged);
@@ -56,11 +65,24 @@ FwdResidentFn<T, V, AFF> pick_fwd_resident(int tpr, int vpt, int rb, bool exact,
   if (tpr == 0 && vpt == 4) return fwd_variant<T, V, 0, 4, AFF>(rb, exact, ragged);
   if (tpr == 0 && vpt == 8) return fwd_variant<T, V, 0, 8, AFF>(rb, exact, ragged);
   return nullptr;
+  }
 }
 
 template <typename T, int V, bool AFF>
 BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact, bool ragged) {
-  if constexpr (V == 1) return tpr == 8 && vpt == 1 ? bwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  if constexpr (V == 1) {
+    return tpr == 8 && vpt == 1 ? bwd_variant<T, V, 8, 1, AFF>(rb, exact, false) : nullptr;
+  } else {
+  if (vpt == 3) {
+    if (tpr == 8) return bwd_variant<T, V, 8, 3, AFF>(rb, exact, ragged);
+    if (tpr == 16) return bwd_variant<T, V, 16, 3, AFF>(rb, exact, ragged);
+    if (tpr == 32) return bwd_variant<T, V, 32, 3, AFF>(rb, exact, ragged);
+    if (tpr == 64) return bwd_variant<T, V, 64, 3, AFF>(rb, exact, ragged);
+    if constexpr (!AFF) {
+      if (tpr == 128) return bwd_variant<T, V, 128, 3, AFF>(1, exact, ragged);
+    }
+    return nullptr;
+  }
   if (tpr == 8) return bwd_variant<T, V, 8, 1, AFF>(rb, exact, ragged);
   if (tpr == 16) return bwd_variant<T, V, 16, 1, AFF>(rb, exact, ragged);
   if (tpr == 32) return bwd_variant<T, V, 32, 1, AFF>(rb, exact, ragged);
@@ -76,6 +98,7 @@ BwdResidentFn<T, V, AFF> pick_bwd_resident(int tpr, int vpt, int rb, bool exact,
     if (tpr == 0 && vpt == 8) return bwd_variant<T, V, 0, 8, AFF>(rb, exact, ragged);
   }
   return nullptr;
+  }
 }
 
 template <typename T, int V, bool AFF>
