@@ -64,7 +64,8 @@ __device__ __forceinline__ void store_pack_n(T* p, const Pack<T, V>& v, int cnt)
   }
 }
 
-// Elements lo .. V-1 of a vector (lo == 0: the single wide access).
+// Elements lo .. V-1 of a vector (lo == 0: the single wide access).  The partial case is a
+// plain predicated element loop: a switch over lo with chunked stores measured slower.
 template <typename T, int V>
 __device__ __forceinline__ void store_pack_from(T* p, const Pack<T, V>& v, int lo) {
   if (lo == 0) {

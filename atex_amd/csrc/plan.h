@@ -167,7 +167,9 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.rpb = 1;
     } else {
       p.threads = 256;
-      if (V > 1 && !p.ragged) p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
+      if (V > 1 && (!p.ragged || p.vpt == 1)) {
+        p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
+      }
       if (kind == RowsKind::kBwdCols) {
         // bigger blocks -> fewer partial rows for the column reduction
         int th = std::min(t.bwd_ln_threads, 512);
@@ -227,6 +229,10 @@ struct TilePlan {
   int CT = 1;      // column tiles
   int RS = 1;      // row slabs
   int64_t R = 0;   // rows per slab
+  // backward sums stage: its own, possibly narrower, tiling
+  int sums_vpt = 4;
+  int sums_CT = 1, sums_RS = 1;
+  int64_t sums_R = 0;
   int S = 1;       // forward: chunks per row of the statistics stage
   int64_t chunk = 0;
   int stats_grid = 1;
@@ -258,12 +264,27 @@ inline TilePlan plan_tiles(bool bwd, int V, int64_t n_rows, int64_t D, int cus) 
     p.off_pairs = 0;
     bytes = align256(sizeof(float) * 2 * size_t(n_rows) * size_t(p.S));
   } else {
+    // sums stage: the widest tile whose partial rows (2 * D floats per row slab, written and
+    // read back) stay under about 5 % of the bytes of dy and x; the narrowest otherwise
+    for (int vpt = 4; vpt >= 1; vpt /= 2) {
+      const int64_t cw = int64_t(kPlanTileThreads) * vpt * V;
+      const int64_t ct = div_up(D, cw);
+      const int64_t want_rs = div_up(int64_t(cus) * t.tile_items_per_cu, ct);
+      int64_t rs2 = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want_rs, n_rows), 1024));
+      const int64_t r = div_up(n_rows, rs2);
+      rs2 = div_up(n_rows, r);
+      p.sums_vpt = vpt;
+      p.sums_CT = static_cast<int>(ct);
+      p.sums_RS = static_cast<int>(rs2);
+      p.sums_R = r;
+      if (rs2 == 1 || rs2 * 80 <= n_rows) break;
+    }
     p.off_pairs = 0;
-    bytes = align256(sizeof(float) * 2 * size_t(n_rows) * size_t(p.CT));
+    bytes = align256(sizeof(float) * 2 * size_t(n_rows) * size_t(p.sums_CT));
     p.off_rowsum = bytes;
     bytes += align256(sizeof(float) * 2 * size_t(n_rows));
     p.off_part = bytes;
-    if (p.RS > 1) bytes += align256(sizeof(float) * 2 * size_t(D) * size_t(p.RS));
+    if (p.sums_RS > 1) bytes += align256(sizeof(float) * 2 * size_t(D) * size_t(p.sums_RS));
   }
   p.ws_bytes = bytes;
   return p;

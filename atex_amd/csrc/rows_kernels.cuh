@@ -75,7 +75,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
                   int64_t n_rows, int d_elems, int C, float eps) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
-  static_assert(!(RAGGED && (EXACT || RB != 1 || V == 1)), "ragged rows use the plain variant");
+  static_assert(!(RAGGED && (EXACT || V == 1)), "ragged rows use the non-exact vector variants");
   // gamma / beta live in registers across rows unless that would exhaust the budget
   constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 4);
   static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
@@ -291,7 +291,7 @@ rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
                   float* __restrict__ part, int64_t n_rows, int d_elems, int C) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
-  static_assert(!(RAGGED && (EXACT || RB != 1 || V == 1)), "ragged rows use the plain variant");
+  static_assert(!(RAGGED && (EXACT || V == 1)), "ragged rows use the non-exact vector variants");
   static_assert((TPR != 0 && TPR <= kWave) || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float2 sum_buf[2][16];
   // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats

@@ -22,7 +22,14 @@ using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, c
 template <typename T, int V, int TPR, int VPT, bool AFF>
 FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
-    if (ragged) return rows_fwd_resident<T, V, TPR, VPT, 1, false, AFF, true>;
+    if (ragged) {
+      // short ragged rows (one vector per lane) keep their row batching
+      if constexpr (TPR != 0 && TPR <= 64 && VPT == 1) {
+        if (rb == 2) return rows_fwd_resident<T, V, TPR, VPT, 2, false, AFF, true>;
+        if (rb == 4) return rows_fwd_resident<T, V, TPR, VPT, 4, false, AFF, true>;
+      }
+      return rb == 1 ? rows_fwd_resident<T, V, TPR, VPT, 1, false, AFF, true> : nullptr;
+    }
     if constexpr (TPR != 0) {
       if (rb == 2) return exact ? rows_fwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 2, false, AFF>;
       if (rb == 4) return exact ? rows_fwd_resident<T, V, TPR, VPT, 4, true, AFF> : rows_fwd_resident<T, V, TPR, VPT, 4, false, AFF>;
@@ -34,7 +41,12 @@ FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact, bool ragged) {
 template <typename T, int V, int TPR, int VPT, bool AFF>
 BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
-    if (ragged) return rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF, true>;
+    if (ragged) {
+      if constexpr (TPR != 0 && TPR <= 64 && VPT == 1) {
+        if (rb == 2) return rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF, true>;
+      }
+      return rb == 1 ? rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF, true> : nullptr;
+    }
     if constexpr (TPR != 0 && TPR <= 64) {
       if (rb == 2) return exact ? rows_bwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF>;
     }
@@ -205,19 +217,24 @@ int tiles_bwd(const T* dy, const T* x, const float* gamma, const float* mean, co
   float2* rowsum = reinterpret_cast<float2*>(base + p.off_rowsum);
   float* part = reinterpret_cast<float*>(base + p.off_part);
   const dim3 grid(p.CT, p.RS);
-  const bool direct = p.RS == 1;  // one row slab: the column sums are final
-  tile_bwd_sums<T, V><<<grid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums,
-                                                    direct ? dgamma : part,
-                                                    direct ? dbeta : part + D,
-                                                    direct ? 0 : 2 * D, n_rows, D, p.R);
+  const dim3 sgrid(p.sums_CT, p.sums_RS);
+  const bool direct = p.sums_RS == 1;  // one row slab: the column sums are final
+  float* og = direct ? dgamma : part;
+  float* ob = direct ? dbeta : part + D;
+  const int64_t sstride = direct ? 0 : 2 * D;
+  switch (p.sums_vpt) {
+    case 4: tile_bwd_sums<T, V, 4><<<sgrid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, og, ob, sstride, n_rows, D, p.sums_R); break;
+    case 2: tile_bwd_sums<T, V, 2><<<sgrid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, og, ob, sstride, n_rows, D, p.sums_R); break;
+    default: tile_bwd_sums<T, V, 1><<<sgrid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, og, ob, sstride, n_rows, D, p.sums_R); break;
+  }
   ATEXN_CHECK_LAUNCH("tile_bwd_sums");
-  merge_row_sums<4><<<static_cast<unsigned>(div_up(n_rows, 4)), 256, 0, st>>>(sums, rowsum, n_rows, p.CT);
+  merge_row_sums<4><<<static_cast<unsigned>(div_up(n_rows, 4)), 256, 0, st>>>(sums, rowsum, n_rows, p.sums_CT);
   ATEXN_CHECK_LAUNCH("merge_row_sums");
   tile_bwd_apply<T, V><<<grid, kTileThreads, 0, st>>>(dy, x, gamma, mean, rstd, rowsum, dx, n_rows,
                                                      D, p.R, tuning().reverse_second_pass);
   ATEXN_CHECK_LAUNCH("tile_bwd_apply");
   if (direct) return ATEXN_OK;
-  return launch_col_reduce(part, dgamma, dbeta, p.RS, D, st);
+  return launch_col_reduce(part, dgamma, dbeta, p.sums_RS, D, st);
 }
 
 template <typename T, int V, bool AFF>

@@ -13,6 +13,10 @@
 // a row whose length is not a multiple of V is handled, element by element, by the single
 // thread that owns it ("tail slot"), outside the vector code of everybody else.
 //
+// The backward sums kernel also comes with narrower tiles (1 or 2 vectors per thread): with
+// few column tiles a launch needs many row slabs to fill the chip, and every slab costs a
+// partial dgamma / dbeta row of 2 * D floats; narrower tiles mean fewer slabs.
+//
 // Stages:  forward   split_fwd_stats -> merge_row_stats -> tile_fwd_apply
 //          backward  tile_bwd_sums -> merge_row_sums -> tile_bwd_apply [-> col_reduce]
 #pragma once
@@ -25,26 +29,26 @@ constexpr int kTileThreads = 256;
 constexpr int kTileVpt = 4;
 constexpr int kTileRowGroup = 64;  // rows whose wave sums are staged in LDS between barriers
 
-template <int V>
+template <int V, int VPT = kTileVpt>
 struct TileGeom {
   int64_t r0, r1;            // rows of the tile
-  int64_t col[kTileVpt];     // first column of each owned vector (clamped into the row)
-  bool full[kTileVpt];       // the vector lies wholly inside the row
+  int64_t col[VPT];          // first column of each owned vector (clamped into the row)
+  bool full[VPT];            // the vector lies wholly inside the row
   bool has_tail;             // this thread owns the row's partial last vector
   int64_t tail_col;
   int tail_cnt;
 };
 
 // Tiles are indexed (blockIdx.x = column tile, blockIdx.y = row slab).
-template <int V>
-__device__ __forceinline__ TileGeom<V> tile_geom(int64_t n_rows, int64_t D, int64_t R) {
-  TileGeom<V> g;
-  const int64_t CW = static_cast<int64_t>(kTileThreads) * kTileVpt * V;
+template <int V, int VPT = kTileVpt>
+__device__ __forceinline__ TileGeom<V, VPT> tile_geom(int64_t n_rows, int64_t D, int64_t R) {
+  TileGeom<V, VPT> g;
+  const int64_t CW = static_cast<int64_t>(kTileThreads) * VPT * V;
   const int64_t c0 = static_cast<int64_t>(blockIdx.x) * CW;
   g.r0 = static_cast<int64_t>(blockIdx.y) * R;
   g.r1 = g.r0 + R < n_rows ? g.r0 + R : n_rows;
 #pragma unroll
-  for (int k = 0; k < kTileVpt; ++k) {
+  for (int k = 0; k < VPT; ++k) {
     const int64_t c = c0 + (static_cast<int64_t>(threadIdx.x) + k * kTileThreads) * V;
     g.full[k] = c + V <= D;
     // vectors outside the row read (and ignore) the row's last full vector position
@@ -54,7 +58,7 @@ __device__ __forceinline__ TileGeom<V> tile_geom(int64_t n_rows, int64_t D, int6
   const int64_t jt = D / V;  // index of the partial vector among the row's vectors
   g.tail_cnt = rem;
   g.tail_col = jt * V;
-  g.has_tail = rem != 0 && jt / (kTileThreads * kTileVpt) == blockIdx.x &&
+  g.has_tail = rem != 0 && jt / (kTileThreads * VPT) == blockIdx.x &&
                jt % kTileThreads == threadIdx.x;
   return g;
 }
@@ -179,7 +183,7 @@ tile_fwd_apply(const T* x, const float* __restrict__ gamma, const float* __restr
 // sums[row * CT + tile]; per column of the tile: sum over the tile's rows of dy * xh and of
 // dy, into out_g / out_b (+ slab * slab_stride): the final dgamma / dbeta when there is one
 // row slab, the partial rows of col_reduce otherwise.
-template <typename T, int V>
+template <typename T, int V, int VPT>
 __global__ void __launch_bounds__(kTileThreads)
 tile_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
               const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
@@ -187,13 +191,13 @@ tile_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x, const float* __
               int64_t slab_stride, int64_t n_rows, int64_t D, int64_t R) {
   constexpr int NW = kTileThreads / kWave;
   __shared__ float2 wsum[kTileRowGroup][NW];
-  const TileGeom<V> g = tile_geom<V>(n_rows, D, R);
+  const TileGeom<V, VPT> g = tile_geom<V, VPT>(n_rows, D, R);
   const int CT = gridDim.x;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = threadIdx.x / kWave;
-  float gm[kTileVpt][V], ag[kTileVpt][V], ab[kTileVpt][V];
+  float gm[VPT][V], ag[VPT][V], ab[VPT][V];
 #pragma unroll
-  for (int k = 0; k < kTileVpt; ++k) {
+  for (int k = 0; k < VPT; ++k) {
     load_f32<V>(gamma + g.col[k], gm[k]);
 #pragma unroll
     for (int e = 0; e < V; ++e) {
@@ -212,16 +216,16 @@ tile_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     for (int64_t row = base; row < end; ++row) {
       const T* xr = x + row * D;
       const T* dr = dy + row * D;
-      Pack<T, V> px[kTileVpt], pd[kTileVpt];
+      Pack<T, V> px[VPT], pd[VPT];
 #pragma unroll
-      for (int k = 0; k < kTileVpt; ++k) {
+      for (int k = 0; k < VPT; ++k) {
         px[k] = load_pack<T, V>(xr + g.col[k]);
         pd[k] = load_pack<T, V>(dr + g.col[k]);
       }
       const float mean = mean_in[row], rstd = rstd_in[row];
       float s1 = 0.f, s2 = 0.f;
 #pragma unroll
-      for (int k = 0; k < kTileVpt; ++k) {
+      for (int k = 0; k < VPT; ++k) {
         float fx[V], fd[V];
         unpack<T, V>(px[k], fx);
         unpack<T, V>(pd[k], fd);
@@ -274,7 +278,7 @@ tile_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   float* og = out_g + static_cast<int64_t>(blockIdx.y) * slab_stride;
   float* ob = out_b + static_cast<int64_t>(blockIdx.y) * slab_stride;
 #pragma unroll
-  for (int k = 0; k < kTileVpt; ++k) {
+  for (int k = 0; k < VPT; ++k) {
     if (g.full[k]) {
       store_f32<V>(og + g.col[k], ag[k]);
       store_f32<V>(ob + g.col[k], ab[k]);
