@@ -192,14 +192,14 @@ __device__ __forceinline__ void cl_pivot(const T* xn_c, int64_t D, int C, float 
 }
 
 // ---------------------------------------------------------------- forward, stage 1
-// ps1 / ps2: [N * S, C] sums of (x - K) and (x - K)^2 over each slab, K = cl_pivot, which
+// psum: [N * S][2][C] sums of (x - K) and (x - K)^2 over each slab, K = cl_pivot, which
 // is saved to pivot[N, C].
 // U > 0: the slab is register-resident (slab_len <= U * pixel slots per block) and all its
 // loads are in flight at once; U == 0 streams the slab in batches.
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
-cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict__ ps2,
-             float* __restrict__ pivot, int64_t D, int C, int S, int tpp_shift,
+cl_fwd_stats(const T* __restrict__ x, float* __restrict__ psum, float* __restrict__ pivot,
+             int64_t D, int C, int S, int tpp_shift,
              int64_t slab_len) {
   __shared__ float lds[2 * V * kClThreads];
   const int CV = (C + V - 1) / V;
@@ -247,9 +247,9 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict
       t1[i] = acc[i];
       t2[i] = acc[V + i];
     }
-    const int64_t o = (g.n * S + g.s) * C + g.coff;
-    store_f32_from<V>(ps1 + o, t1, RG ? g.lo : 0);
-    store_f32_from<V>(ps2 + o, t2, RG ? g.lo : 0);
+    const int64_t o = ((g.n * S + g.s) * 2) * C + g.coff;
+    store_f32_from<V>(psum + o, t1, RG ? g.lo : 0);
+    store_f32_from<V>(psum + o + C, t2, RG ? g.lo : 0);
     // stage 2 must not re-read the pivot from x: y may alias x and be half written by then
     if (g.s == 0) store_f32_from<V>(pivot + g.n * C + g.coff, k0, RG ? g.lo : 0);
   }
@@ -260,8 +260,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ ps1, float* __restrict
 // every thread reads a vector before it writes the same vector.
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
-cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict__ ps2,
-             const float* __restrict__ pivot, const float* __restrict__ gamma,
+cl_fwd_apply(const T* x, const float* __restrict__ psum, const float* __restrict__ pivot, const float* __restrict__ gamma,
              const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
              float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
              int64_t slab_len, float eps, int rev) {
@@ -287,8 +286,8 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
     const bool in = cl < cap && c < C;
     float s1 = 0.f, s2 = 0.f, kc = 0.f;
     if (in) {
-      const float* q1 = ps1 + (g.n * S) * C + c;
-      const float* q2 = ps2 + (g.n * S) * C + c;
+      const float* q1 = psum + ((g.n * S) * 2) * C + c;
+      const float* q2 = q1 + C;
       if (sub == 0) kc = pivot[g.n * C + c];
       constexpr int B = 16;
       batched_for<B>(
@@ -297,8 +296,8 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
             float t1[B], t2[B];
 #pragma unroll
             for (int u = 0; u < B; ++u) {
-              t1[u] = q1[(sl + u * step) * C];
-              t2[u] = q2[(sl + u * step) * C];
+              t1[u] = q1[((sl + u * step) * 2) * C];
+              t2[u] = q2[((sl + u * step) * 2) * C];
             }
 #pragma unroll
             for (int u = 0; u < B; ++u) {
@@ -307,8 +306,8 @@ cl_fwd_apply(const T* x, const float* __restrict__ ps1, const float* __restrict_
             }
           },
           [&](int64_t sl) {
-            s1 += q1[sl * C];
-            s2 += q2[sl * C];
+            s1 += q1[(sl * 2) * C];
+            s2 += q2[(sl * 2) * C];
           });
     }
     for (int m = 1; m < fm.P; m <<= 1) {

@@ -14,19 +14,25 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   const ClPlan p = plan_cl(false, V, N, C, D, cu_count());
   ATEXN_REQUIRE(ws != nullptr && ws_bytes >= p.ws_bytes,
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
-  float* pmean = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
-  float* pm2 = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_b);
+  float* psum = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
   float* pivot = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_c);
+  float* folded = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_fold);
   const int Ci = static_cast<int>(C);
   ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_FWD(U_, RG_)                                                                  \
   do {                                                                                        \
-    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, D, Ci, p.S,   \
+    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, psum, pivot, D, Ci, p.S,         \
                                                        p.tpp_shift, p.slab_len);              \
     ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
-    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pmean, pm2, pivot, gamma, beta, y, \
-                                                       mean, rstd, D, Ci, p.S, p.tpp_shift,   \
+    if (p.fold) {                                                                             \
+      const int rc = launch_col_reduce(psum, folded, folded + C, p.S, C, st,                  \
+                                       static_cast<int>(N), int64_t(p.S) * 2 * C, 2 * C);     \
+      if (rc != ATEXN_OK) return rc;                                                          \
+    }                                                                                         \
+    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, p.fold ? folded : psum, pivot,   \
+                                                       gamma, beta, y, mean, rstd, D, Ci,     \
+                                                       p.fold ? 1 : p.S, p.tpp_shift,         \
                                                        p.slab_len, eps,                       \
                                                        tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \
@@ -52,6 +58,7 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   ATEXN_REQUIRE(ws != nullptr && ws_bytes >= p.ws_bytes,
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* part = static_cast<float*>(ws);
+  float* folded = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_fold);
   const int Ci = static_cast<int>(C);
   ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
@@ -60,8 +67,15 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
     cl_bwd_sums<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S, \
                                                       p.tpp_shift, p.slab_len);               \
     ATEXN_CHECK_LAUNCH("cl_bwd_sums");                                                        \
-    cl_bwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, part, dx, \
-                                                       dgamma, dbeta, N, D, Ci, p.S,          \
+    if (p.fold) {                                                                             \
+      const int rc = launch_col_reduce(part, folded, folded + C, p.S, C, st,                  \
+                                       static_cast<int>(N), int64_t(p.S) * 2 * C, 2 * C);     \
+      if (rc != ATEXN_OK) return rc;                                                          \
+    }                                                                                         \
+    cl_bwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd,           \
+                                                       p.fold ? folded : part, dx,            \
+                                                       dgamma, dbeta, N, D, Ci,               \
+                                                       p.fold ? 1 : p.S,                      \
                                                        p.tpp_shift, p.slab_len,               \
                                                        tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \

@@ -67,7 +67,7 @@ int fill_zero(float* out, int64_t n, hipStream_t st) {
 }
 
 int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_t W,
-                      hipStream_t st) {
+                      hipStream_t st, int batch, int64_t part_stride, int64_t out_stride) {
   ATEXN_REQUIRE(2 * W < (int64_t(1) << 31), "column count %lld too large", (long long)W);
   const int Wi = static_cast<int>(W);
   // Column groups per block (CX): the more, the longer the contiguous run a wave reads per
@@ -75,11 +75,12 @@ int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_
   // largest CX that still gives every CU a block and every row-lane at least two rows.
   const int cus = cu_count();
   auto fits = [&](int cw, int cx) {
-    return div_up(2 * W, int64_t(cw) * cx) >= cus && (256 / cx) * 2 <= std::max(G, 2);
+    return div_up(2 * W, int64_t(cw) * cx) * batch >= cus && (256 / cx) * 2 <= std::max(G, 2);
   };
 #define ATEXN_COL_REDUCE(CW_, CX_)                                                              \
-  col_reduce<CW_, CX_><<<static_cast<int>(div_up(2 * W, int64_t(CW_) * CX_)), kColReduceThreads, \
-                         0, st>>>(part, out0, out1, G, Wi)
+  col_reduce<CW_, CX_><<<dim3(static_cast<unsigned>(div_up(2 * W, int64_t(CW_) * CX_)), batch),  \
+                         kColReduceThreads, 0, st>>>(part, out0, out1, G, Wi, part_stride,      \
+                                                     out_stride)
   if (W % 4 == 0) {
     if (fits(4, 256) || G < 8) {
       ATEXN_COL_REDUCE(4, 256);

@@ -302,8 +302,13 @@ struct ClPlan {
   int64_t slab_len = 0;
   int64_t n_work = 0;
   int grid = 1;
-  size_t off_a = 0, off_b = 0, off_c = 0, ws_bytes = 0;
+  // More slabs per instance than kClFoldAbove: a small launch between the two stages adds up
+  // the slab partials of every instance once (folded[N][2][C]) instead of every stage-2
+  // workgroup doing it for itself.
+  bool fold = false;
+  size_t off_a = 0, off_b = 0, off_c = 0, off_fold = 0, ws_bytes = 0;
 };
+constexpr int kClFoldAbove = 64;
 
 inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
   const Tuning& t = tuning();
@@ -336,7 +341,9 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.off_b = sect;
   // fwd: slab sums S1, S2 [N*S, C] and the pivots [N, C]; bwd: part[N*S][2][C] (contiguous)
   p.off_c = 2 * sect;
-  p.ws_bytes = 2 * sect + align256(sizeof(float) * size_t(N) * size_t(C));
+  p.off_fold = 2 * sect + align256(sizeof(float) * size_t(N) * size_t(C));
+  p.fold = p.S > kClFoldAbove && N <= 65535;
+  p.ws_bytes = p.off_fold + align256(sizeof(float) * 2 * size_t(N) * size_t(C));
   return p;
 }
 

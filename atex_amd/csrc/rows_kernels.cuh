@@ -564,7 +564,11 @@ constexpr int kColReduceThreads = 256;
 template <int CW, int CX>
 __global__ void __launch_bounds__(kColReduceThreads)
 col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __restrict__ out1,
-           int G, int W) {
+           int G, int W, int64_t part_stride, int64_t out_stride) {
+  // blockIdx.y: independent problems part + y * part_stride -> out + y * out_stride
+  part += static_cast<int64_t>(blockIdx.y) * part_stride;
+  out0 += static_cast<int64_t>(blockIdx.y) * out_stride;
+  out1 += static_cast<int64_t>(blockIdx.y) * out_stride;
   // CX column groups of CW columns per block, CY = threads / CX partial rows in parallel:
   // CX = 4 for many partial rows, 64 for a few dozen, 256 (one thread per group, no
   // exchange) for a handful.

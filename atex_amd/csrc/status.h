@@ -52,9 +52,11 @@ int cl_bwd(int dtype, const void* dy, const void* x, const float* gamma, const f
 int fill_zero(float* out, int64_t n, hipStream_t st);
 
 // Launches the deterministic column reduction out0[j] = sum_g part[g][0][j],
-// out1[j] = sum_g part[g][1][j], j < W.
+// out1[j] = sum_g part[g][1][j], j < W; `batch` independent problems at the given strides
+// (in floats) in one launch.
 int launch_col_reduce(const float* part, float* out0, float* out1, int G, int64_t W,
-                      hipStream_t st);
+                      hipStream_t st, int batch = 1, int64_t part_stride = 0,
+                      int64_t out_stride = 0);
 
 inline int elem_size(int dtype) { return dtype == ATEXN_F32 ? 4 : 2; }
 

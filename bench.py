@@ -68,6 +68,8 @@ CASES = {
     "lnref_1e7x10": ("ln", "f16", (10000000, 10)),
     "lnref_4x400001": ("ln", "f16", (4, 400001)),
     "lnref_4x10000001": ("ln", "f16", (4, 10000001)),
+    "in_1x128x512x512_cl": ("in", "f16", (1, 128, 512 * 512, False)),
+    "in_1x32x128x128x128_cl": ("in", "f16", (1, 32, 128 ** 3, False)),
     "inref_8x64x64_cl": ("in", "f16", (8, 64, 64 ** 3, False)),
     "inref_8x64x64_cf": ("in", "f16", (8, 64, 64 ** 3, True)),
     "inref_4x256x32_cl": ("in", "f16", (4, 256, 32 ** 3, False)),
@@ -400,7 +402,7 @@ def main():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
     if args.case == "all":
         for name in CASES:
-            if "ref_" in name or "x1" in name or "x2" in name or "x7" in name or name.endswith("_f32"):
+            if "ref_" in name or "in_1x" in name or "x1" in name or "x2" in name or "x7" in name or name.endswith("_f32"):
                 continue
             steps = args.steps if "3d" not in name else max(10, args.steps // 10)
             r = run_case(name, steps, args.warmup, with_cpu=False)
