@@ -147,7 +147,7 @@ int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* 
     return ATEXN_OK;
   }
   ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
-  ATEXN_REQUIRE(dx != dy && dx != x, "dx must not alias dy or x");
+  ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
   ATEXN_REQUIRE(workspace != nullptr && ws_aligned(workspace), "workspace must be non-NULL and 256-byte aligned");
   return rows_bwd(dtype, false, dy, x, gamma, mean, inv_std, N, D, 1, dx, dgamma, dbeta, workspace,
                   workspace_bytes, st);
@@ -206,7 +206,7 @@ int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x
     return ATEXN_OK;
   }
   ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
-  ATEXN_REQUIRE(dx != dy && dx != x, "dx must not alias dy or x");
+  ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
   ATEXN_REQUIRE(workspace != nullptr && ws_aligned(workspace), "workspace must be non-NULL and 256-byte aligned");
   if (layout == ATEXN_LAYOUT_NC_) {
     return rows_bwd(dtype, true, dy, x, gamma, mean, inv_std, N * C, D, static_cast<int>(C), dx,

@@ -463,9 +463,9 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 // all N * S partial rows (fixed order, no atomics), which spares a third launch.
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
-cl_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
+cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
-             const float* __restrict__ part, T* __restrict__ dx, float* __restrict__ dgamma,
+             const float* __restrict__ part, T* dx, float* __restrict__ dgamma,
              float* __restrict__ dbeta, int64_t N, int64_t D, int C, int S, int tpp_shift,
              int64_t slab_len, int rev) {
   __shared__ float sm_a[kClMaxTileChannels];  // sum dy

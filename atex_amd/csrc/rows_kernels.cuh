@@ -281,13 +281,14 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // row % C, the two row sums a = sum dy, b = sum dy * xh give s1 = gamma a, s2 = gamma b and
 // are written to part[n][0][c] = b, part[n][1][c] = a  (n = row / C), i.e. `part` has
 // N * 2 * C floats and the same second kernel folds it over n.
-// dx must not alias dy or x.  RB / EXACT / prefetch as in the forward kernel.
+// dx may alias dy (a thread reads its elements of a row before it writes them), not x.
+// RB / EXACT / prefetch as in the forward kernel.
 template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
           bool RAGGED = false>
 __global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT>()))
-rows_bwd_resident(const T* __restrict__ dy, const T* __restrict__ x,
+rows_bwd_resident(const T* dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
-                  const float* __restrict__ rstd_in, T* __restrict__ dx,
+                  const float* __restrict__ rstd_in, T* dx,
                   float* __restrict__ part, int64_t n_rows, int d_elems, int C) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
@@ -908,11 +909,11 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
 // stage 2 backward: merge the row's chunk sums, write dx for the chunk.  ROW_AFFINE also
 // writes the per-(n, c) sums into `part` (layout as in rows_bwd_resident).
 template <typename T, int V, bool ROW_AFFINE>
-__global__ void split_bwd_apply(const T* __restrict__ dy, const T* __restrict__ x,
+__global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
                                 const float* __restrict__ gamma,
                                 const float* __restrict__ mean_in,
                                 const float* __restrict__ rstd_in,
-                                const float2* __restrict__ sums, T* __restrict__ dx,
+                                const float2* __restrict__ sums, T* dx,
                                 float* __restrict__ part, int64_t n_rows, int64_t D, int S,
                                 int64_t chunk, int C, int rev) {
   constexpr int B = ROW_AFFINE ? kSplitBatch : 2;

@@ -74,7 +74,7 @@ int atexn_layer_norm_fwd(int dtype, const void* x, const float* gamma, const flo
                          void* stream);
 
 /* Replaces functor::FusedLayerNormGrad<GPUDevice,T,U>::operator()
- * (cc/kernels/fused_layer_norm_op.cu:895-1030). dx must not alias dy or x. */
+ * (cc/kernels/fused_layer_norm_op.cu:895-1030). dx may alias dy (in-place gradient), not x. */
 size_t atexn_layer_norm_bwd_workspace_bytes(int dtype, int64_t N, int64_t D);
 int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* gamma,
                          const float* mean, const float* inv_std, int64_t N, int64_t D,
@@ -92,7 +92,8 @@ int atexn_instance_norm_fwd(int dtype, int layout, const void* x, const float* g
                             void* workspace, size_t workspace_bytes, void* stream);
 
 /* Replaces functor::FusedInstanceNormGrad<GPUDevice,T,U>::operator()
- * (cc/kernels/fused_instance_norm_op.cu:1519-1561). dgamma / dbeta are [C]. */
+ * (cc/kernels/fused_instance_norm_op.cu:1519-1561). dgamma / dbeta are [C]; dx may alias dy,
+ * not x. */
 size_t atexn_instance_norm_bwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
                                                int64_t D);
 int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x,

@@ -205,8 +205,8 @@ def test_kernel_level_validation(L):
     assert L.atexn_layer_norm_fwd(0, FAKE, FAKE, FAKE, 4, 8, 1e-3, FAKE, FAKE, FAKE, 0x1010, 4096, None) == 1
     assert b"256-byte aligned" in L.atexn_last_error()
     assert L.atexn_layer_norm_bwd(0, FAKE, FAKE, FAKE, FAKE, FAKE, 4, 8, FAKE, FAKE, FAKE, None, 0, None) == 1
-    assert L.atexn_layer_norm_bwd(0, FAKE, 0x2000, FAKE, FAKE, FAKE, 4, 8, FAKE, FAKE, FAKE, 0x4000, 1 << 20, None) == 1
-    assert b"dx must not alias" in L.atexn_last_error()
+    assert L.atexn_layer_norm_bwd(0, FAKE, 0x2000, FAKE, FAKE, FAKE, 4, 8, 0x2000, FAKE, FAKE, 0x4000, 1 << 20, None) == 1
+    assert b"dx must not alias x" in L.atexn_last_error()
     assert L.atexn_instance_norm_fwd(0, 5, FAKE, FAKE, FAKE, 1, 2, 3, 1e-3, FAKE, FAKE, FAKE, None, 0, None) == 1
     assert b"bad layout" in L.atexn_last_error()
     # too small a workspace is an argument error, not a launch

@@ -159,11 +159,11 @@ class Capi:
             self._p(rstd), wp, wb, self._stream(x.device)))
         return y, mean, rstd
 
-    def ln_bwd(self, dy, x, gamma, mean, rstd, dtype):
+    def ln_bwd(self, dy, x, gamma, mean, rstd, dtype, dx=None):
         t = self.torch
         N, D = x.shape
         code = O.DTYPE_CODE[dtype]
-        dx = t.empty_like(x)
+        dx = t.empty_like(x) if dx is None else dx
         dg = t.empty(D, dtype=t.float32, device=x.device)
         db = t.empty(D, dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_layer_norm_bwd_workspace_bytes(code, N, D), x.device)
@@ -190,12 +190,12 @@ class Capi:
             self._p(mean), self._p(rstd), wp, wb, self._stream(x.device)))
         return y, mean, rstd
 
-    def in_bwd(self, dy, x, gamma, mean, rstd, dtype, channel_first):
+    def in_bwd(self, dy, x, gamma, mean, rstd, dtype, channel_first, dx=None):
         t = self.torch
         N, C, D = self._ncd(x.shape, channel_first)
         code = O.DTYPE_CODE[dtype]
         layout = 0 if channel_first else 1
-        dx = t.empty_like(x)
+        dx = t.empty_like(x) if dx is None else dx
         dg = t.empty(C, dtype=t.float32, device=x.device)
         db = t.empty(C, dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_instance_norm_bwd_workspace_bytes(code, layout, N, C, D), x.device)
