@@ -17,7 +17,8 @@ Output: ONE JSON line on stdout.
                launch stream: algorithmic bytes of the backward / its average duration,
                against the 8 TB/s HBM peak
   cpu_baseline the C oracle's float flavour (OpenMP over rows) on the same workload, timed
-               on this machine's host cores
+               on this machine's host cores; `unfused_composite` inside it is the unfused op
+               sequence a framework would run instead (torch on the CPU, autograd backward)
 """
 from __future__ import annotations
 
@@ -267,7 +268,49 @@ def cpu_baseline(op, dtype, dims, max_seconds=20.0):
         "kind": "port",
         "sample": f"{sample}; median of {len(times)} steps, {med * 1e6:.0f} us/step",
         "us_per_step": med * 1e6,
+        "unfused_composite": composite_cpu(op, dtype, d, x, gamma, beta, dy, threads),
     }
+
+
+def composite_cpu(op, dtype, d, x, gamma, beta, dy, threads, max_seconds=8.0):
+    """What a framework without the fused op runs on the host: the unfused op sequence
+    (moments -> subtract -> rsqrt -> multiply -> add, statistics in float32, autograd for
+    the backward) in torch on the CPU.  A composite restatement, not tf.keras itself
+    (TensorFlow is not installed); reported beside the fused C port for orientation."""
+    import torch
+
+    torch.set_num_threads(threads)
+    tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
+    xt = torch.from_numpy(np.ascontiguousarray(x, dtype=np.float32)).to(tdt).requires_grad_(True)
+    g = torch.from_numpy(gamma).requires_grad_(True)
+    b = torch.from_numpy(beta).requires_grad_(True)
+    dyt = torch.from_numpy(np.ascontiguousarray(dy, dtype=np.float32)).to(tdt)
+    if op == "ln":
+        axes, wshape = (-1,), (1, -1)
+    elif d[3]:   # channel-first [N, C, D]
+        axes, wshape = (2,), (1, -1, 1)
+    else:        # channels-last [N, D, C]
+        axes, wshape = (1,), (1, 1, -1)
+
+    def step():
+        xf = xt.float()
+        mean = xf.mean(dim=axes, keepdim=True)
+        var = (xf - mean).square().mean(dim=axes, keepdim=True)
+        y = ((xf - mean) * torch.rsqrt(var + 1e-3) * g.view(wshape) + b.view(wshape)).to(tdt)
+        torch.autograd.grad(y, (xt, g, b), dyt)
+
+    step()
+    times = []
+    t_end = time.perf_counter() + max_seconds
+    while len(times) < 10 and (time.perf_counter() < t_end or len(times) < 2):
+        t0 = time.perf_counter()
+        step()
+        times.append(time.perf_counter() - t0)
+    med = float(np.median(times))
+    fb, bb = algorithmic_bytes(op, dtype, d)
+    return {"value": (fb + bb) / med / 1e9, "unit": "GB/s", "threads": threads,
+            "us_per_step": med * 1e6,
+            "note": "torch CPU, unfused op sequence with autograd; composite restatement, not tf.keras"}
 
 
 def roofline_kernel(op, dims):
