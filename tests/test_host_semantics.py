@@ -264,3 +264,27 @@ def test_python_layer_semantics_on_cpu():
     assert set(n for n in dir(nv_norms) if not n.startswith("__")) >= {
         "LayerNormalization", "InstanceNormalization", "fused_layer_norm_op", "fused_layer_norm_grad_op",
         "fused_instance_norm_op", "fused_instance_norm_grad_op", "_layer_norm_grad", "_instance_norm_grad"}
+
+
+def test_header_is_plain_c_and_links_from_c(tmp_path):
+    """include/atex_norms.h compiles as C99 and as C++, and a C program linked against the
+    library can use the host-side entry points (no Python, no torch, no GPU)."""
+    import shutil
+    import subprocess
+
+    from atex_amd.nv_norms import _capi
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    inc = os.path.join(root, "include")
+    hdr = os.path.join(inc, "atex_norms.h")
+    subprocess.run(["gcc", "-std=c99", "-pedantic", "-Wall", "-Werror", "-fsyntax-only", "-x", "c", hdr],
+                   check=True)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", hdr], check=True)
+    exe = str(tmp_path / "capi_host_check")
+    libdir = os.path.dirname(_capi.LIB_PATH)
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Werror", "-I", inc,
+                    os.path.join(root, "tests", "capi_host_check.c"), "-o", exe,
+                    "-L", libdir, "-latex_norms_hip", f"-Wl,-rpath,{libdir}"], check=True)
+    out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
+    assert out.returncode == 0, out.stderr + out.stdout
+    assert "capi host check ok" in out.stdout
