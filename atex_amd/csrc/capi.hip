@@ -155,7 +155,7 @@ int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* 
 
 size_t atexn_instance_norm_fwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
                                                int64_t D) {
-  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt) return 0;
+  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt || N > kMaxInt) return 0;
   return layout == ATEXN_LAYOUT_NC_ ? rows_fwd_ws(dtype, true, N * C, D, static_cast<int>(C))
                                     : cl_fwd_ws(dtype, N, C, D);
 }
@@ -167,7 +167,7 @@ int atexn_instance_norm_fwd(int dtype, int layout, const void* x, const float* g
   ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
   ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
   ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
-  ATEXN_REQUIRE(C <= kMaxInt, "C=%lld too large", (long long)C);
+  ATEXN_REQUIRE(C <= kMaxInt && N <= kMaxInt, "N=%lld or C=%lld too large", (long long)N, (long long)C);
   if (N == 0 || C == 0 || D == 0) return ATEXN_OK;
   ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
   ATEXN_REQUIRE(workspace == nullptr || ws_aligned(workspace), "workspace must be 256-byte aligned");
@@ -182,7 +182,7 @@ int atexn_instance_norm_fwd(int dtype, int layout, const void* x, const float* g
 
 size_t atexn_instance_norm_bwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
                                                int64_t D) {
-  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt) return 0;
+  if (!dtype_ok(dtype) || N <= 0 || C <= 0 || D <= 0 || C > kMaxInt || N > kMaxInt) return 0;
   return layout == ATEXN_LAYOUT_NC_ ? rows_bwd_ws(dtype, true, N * C, D, static_cast<int>(C))
                                     : cl_bwd_ws(dtype, N, C, D);
 }
@@ -195,7 +195,7 @@ int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x
   ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
   ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
   ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
-  ATEXN_REQUIRE(C <= kMaxInt, "C=%lld too large", (long long)C);
+  ATEXN_REQUIRE(C <= kMaxInt && N <= kMaxInt, "N=%lld or C=%lld too large", (long long)N, (long long)C);
   hipStream_t st = static_cast<hipStream_t>(stream);
   if (N == 0 || C == 0 || D == 0) {
     if (C > 0) {

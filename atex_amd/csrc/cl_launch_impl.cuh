@@ -18,7 +18,9 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   float* pivot = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_c);
   float* folded = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_fold);
   const int Ci = static_cast<int>(C);
-  ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
+  // one workgroup column per instance: the launch's x extent N * 256 must stay below 2^32
+  ATEXN_REQUIRE(N < (int64_t(1) << 24), "batch size %lld too large (channels-last limit 2^24 - 1)",
+                (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_FWD(U_, RG_)                                                                  \
   do {                                                                                        \
@@ -60,7 +62,9 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   float* part = static_cast<float*>(ws);
   float* folded = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_fold);
   const int Ci = static_cast<int>(C);
-  ATEXN_REQUIRE(N < (int64_t(1) << 31), "batch size %lld too large", (long long)N);
+  // one workgroup column per instance: the launch's x extent N * 256 must stay below 2^32
+  ATEXN_REQUIRE(N < (int64_t(1) << 24), "batch size %lld too large (channels-last limit 2^24 - 1)",
+                (long long)N);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_BWD(U_, RG_)                                                                  \
   do {                                                                                        \
