@@ -161,7 +161,7 @@ __device__ __forceinline__ void cl_for_pixels(const ClGeom& g, Full&& full, Tail
 // are unconditional so that they are all in flight at once: a lane whose pixel or channel
 // vector lies outside the slab reads the slab's first pixel / the last channel vector
 // instead (always valid memory) and is masked out of the arithmetic.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool LAST = false>
 __device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, int CV, int C,
                                              Pack<T, V> (&raw)[U], bool (&ok)[U]) {
   const T* b = base_n + g.coff;
@@ -169,7 +169,8 @@ __device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, i
   for (int u = 0; u < U; ++u) {
     const int64_t p = g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb;
     ok[u] = g.ch_ok && p < g.p1;
-    raw[u] = load_pack<T, V>(b + (p < g.p1 ? p : g.p0) * C);
+    const T* src = b + (p < g.p1 ? p : g.p0) * C;
+    raw[u] = LAST ? load_pack_last<T, V>(src) : load_pack<T, V>(src);
   }
 }
 
@@ -275,7 +276,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ psum, const float* __restrict
   // resident slab: its loads are issued first and fly while the partials are folded
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
-  if constexpr (U > 0) cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, raw, ok);
   // phase A: add up the S slab partials of every channel of the tile, finish the
   // statistics around the pivot
   const int c_base = g.ct * cap;
@@ -369,14 +370,14 @@ cl_fwd_apply(const T* x, const float* __restrict__ psum, const float* __restrict
 #pragma unroll
             for (int u = 0; u < B; ++u) {
               q[u] = rev ? flip - (p + u * step) : p + u * step;
-              pk[u] = load_pack<T, V>(x + boff + q[u] * C);
+              pk[u] = load_pack_last<T, V>(x + boff + q[u] * C);
             }
 #pragma unroll
             for (int u = 0; u < B; ++u) apply(pk[u], q[u]);
           },
           [&](int64_t p) {
             const int64_t q = rev ? flip - p : p;
-            apply(load_pack<T, V>(x + boff + q * C), q);
+            apply(load_pack_last<T, V>(x + boff + q * C), q);
           });
     }
   }
@@ -481,8 +482,8 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool okp[U > 0 ? U : 1];
   if constexpr (U > 0) {
-    cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, okp);
-    cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, okp);
+    cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, rx, okp);
+    cl_load_slab<T, V, U, true>(dy + (g.n * D) * C, g, CV, C, rd, okp);
   }
   const int c_base = g.ct * cap;
   for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
@@ -589,15 +590,15 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
 #pragma unroll
             for (int u = 0; u < B; ++u) {
               q[u] = rev ? flip - (p + u * step) : p + u * step;
-              px[u] = load_pack<T, V>(x + boff + q[u] * C);
-              pd[u] = load_pack<T, V>(dy + boff + q[u] * C);
+              px[u] = load_pack_last<T, V>(x + boff + q[u] * C);
+              pd[u] = load_pack_last<T, V>(dy + boff + q[u] * C);
             }
 #pragma unroll
             for (int u = 0; u < B; ++u) apply(px[u], pd[u], q[u]);
           },
           [&](int64_t p) {
             const int64_t q = rev ? flip - p : p;
-            apply(load_pack<T, V>(x + boff + q * C), load_pack<T, V>(dy + boff + q * C), q);
+            apply(load_pack_last<T, V>(x + boff + q * C), load_pack_last<T, V>(dy + boff + q * C), q);
           });
     }
   }

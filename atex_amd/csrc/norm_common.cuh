@@ -50,6 +50,21 @@ template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p) {
   return *reinterpret_cast<const Pack<T, V>*>(p);
 }
+// The last read of an input by the second stage of a two-stage kernel: the non-temporal hint
+// keeps these lines from displacing what is still to be read (measured: 0-3 % off the
+// backward of the 268 MB cases, 9 % off [10, 10^7]).
+template <typename T, int V>
+__device__ __forceinline__ Pack<T, V> load_pack_last(const T* p) {
+  if constexpr (sizeof(T) * V == 16) {
+    using u32x4_u = typename Bits16<sizeof(T)>::type;
+    const u32x4 bits = __builtin_nontemporal_load(reinterpret_cast<const u32x4_u*>(p));
+    Pack<T, V> r;
+    __builtin_memcpy(&r, &bits, 16);
+    return r;
+  } else {
+    return load_pack<T, V>(p);
+  }
+}
 // Output tensors (y, dx) are written once and never read back by these kernels, so their
 // stores carry the non-temporal hint: the lines do not compete with the inputs for L2 and
 // drain as a stream.  Measured on MI355X against plain stores: forward 8.7 -> 6.3 us at

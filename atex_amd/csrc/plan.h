@@ -23,7 +23,7 @@ struct Tuning {
   int bwd_waves_per_cu = 8;       // resident LayerNorm backward: waves kept resident per CU
                                   //   (each block adds a partial row to the column reduction)
   int bwd_affine_waves_per_cu = 32;  // resident channel-first backward (no partial rows)
-  int split_items_per_cu = 4;     // split rows: (row, chunk) work items per CU
+  int split_items_per_cu = 2;     // split rows: (row, chunk) work items per CU
   int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
   int tile_items_per_cu = 4;      // LayerNorm long rows: (row slab, column tile) tiles per CU
   int fwd_rows_batch = 4;         // resident kernels, rows <= one wave: rows per batch of a

@@ -804,14 +804,14 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
 #pragma unroll
           for (int u = 0; u < B; ++u) {
             i[u] = split_pos(v + u * step, n_vec, rev) * V;
-            pk[u] = load_pack<T, V>(xp + i[u]);
+            pk[u] = load_pack_last<T, V>(xp + i[u]);
           }
 #pragma unroll
           for (int u = 0; u < B; ++u) one(pk[u], i[u]);
         },
         [&](int64_t v) {
           const int64_t i = split_pos(v, n_vec, rev) * V;
-          one(load_pack<T, V>(xp + i), i);
+          one(load_pack_last<T, V>(xp + i), i);
         });
     // ragged row end (last chunk only): the elements after the last full vector
     const int rem = static_cast<int>(len % V);
@@ -970,15 +970,15 @@ __global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
 #pragma unroll
           for (int u = 0; u < B; ++u) {
             i[u] = split_pos(v + u * step, n_vec, rev) * V;
-            px[u] = load_pack<T, V>(xp + i[u]);
-            pd[u] = load_pack<T, V>(dp + i[u]);
+            px[u] = load_pack_last<T, V>(xp + i[u]);
+            pd[u] = load_pack_last<T, V>(dp + i[u]);
           }
 #pragma unroll
           for (int u = 0; u < B; ++u) one(px[u], pd[u], i[u]);
         },
         [&](int64_t v) {
           const int64_t i = split_pos(v, n_vec, rev) * V;
-          one(load_pack<T, V>(xp + i), load_pack<T, V>(dp + i), i);
+          one(load_pack_last<T, V>(xp + i), load_pack_last<T, V>(dp + i), i);
         });
     const int rem = static_cast<int>(len % V);
     if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {

@@ -155,7 +155,7 @@ tile_fwd_apply(const T* x, const float* __restrict__ gamma, const float* __restr
     T* yr = y + row * D;
     Pack<T, V> pk[kTileVpt];
 #pragma unroll
-    for (int k = 0; k < kTileVpt; ++k) pk[k] = load_pack<T, V>(xr + g.col[k]);
+    for (int k = 0; k < kTileVpt; ++k) pk[k] = load_pack_last<T, V>(xr + g.col[k]);
     const float mean = mean_in[row], rstd = rstd_in[row];
 #pragma unroll
     for (int k = 0; k < kTileVpt; ++k) {
@@ -314,8 +314,8 @@ tile_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ g
     Pack<T, V> px[kTileVpt], pd[kTileVpt];
 #pragma unroll
     for (int k = 0; k < kTileVpt; ++k) {
-      px[k] = load_pack<T, V>(xr + g.col[k]);
-      pd[k] = load_pack<T, V>(dr + g.col[k]);
+      px[k] = load_pack_last<T, V>(xr + g.col[k]);
+      pd[k] = load_pack_last<T, V>(dr + g.col[k]);
     }
     const float mean = mean_in[row], rstd = rstd_in[row];
     const float2 rs = rowsum[row];

@@ -84,10 +84,10 @@ DEFAULT_CASE = "ln_bert"
 # WRITE_SIZE x 1.0).  Summaries: profiles/<case>_hbm_traffic.txt.  Cases without a run: None.
 MEASURED_TRAFFIC = {
     "ln_bert": 52.78e6,                 # rows_bwd_resident
-    "in2d_nchw": 50.48e6,               # rows_bwd_resident (row-affine)
+    "in2d_nchw": 50.51e6,               # rows_bwd_resident (row-affine)
     "in2d_nhwc": 33.99e6 + 52.59e6,     # cl_bwd_sums + cl_bwd_apply
-    "in3d_ndhwc": 537.01e6 + 805.31e6,  # cl_bwd_sums + cl_bwd_apply
-    "in3d_ncdhw": 536.86e6 + 805.41e6,  # split_bwd_sums + split_bwd_apply
+    "in3d_ndhwc": 537.01e6 + 805.34e6,  # cl_bwd_sums + cl_bwd_apply
+    "in3d_ncdhw": 536.84e6 + 805.38e6,  # split_bwd_sums + split_bwd_apply
 }
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
