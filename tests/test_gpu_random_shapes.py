@@ -1,6 +1,8 @@
 """Seeded sweep over random shapes, dtypes, layouts, alignments and in-place use: every kernel
 family and every boundary between them (resident / tiles / small / split / channels-last,
 exact / non-exact / ragged) is crossed many times, each case checked against the oracle."""
+import os
+
 import numpy as np
 import pytest
 
@@ -10,6 +12,8 @@ from tests.util import TOL, assert_close
 pytestmark = pytest.mark.gpu
 
 EPS = 1e-3
+# cases per op; a longer sweep: ATEXN_RANDOM_SEEDS=1000 python -m pytest tests/test_gpu_random_shapes.py
+N_SEEDS = int(os.environ.get("ATEXN_RANDOM_SEEDS", "48"))
 
 
 def _pick_d(rng):
@@ -40,7 +44,7 @@ def _check(got, ref, dy, gamma, rstd, dtype):
     assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(N_SEEDS))
 def test_layer_norm_random(coracle, seed):
     import torch
 
@@ -70,7 +74,7 @@ def test_layer_norm_random(coracle, seed):
     _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
 
 
-@pytest.mark.parametrize("seed", range(48))
+@pytest.mark.parametrize("seed", range(N_SEEDS))
 def test_instance_norm_random(coracle, seed):
     import torch
 
