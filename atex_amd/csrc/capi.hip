@@ -71,7 +71,8 @@ int atexn_abi_version(void) { return kAbiVersion; }
  * name or a value out of range. */
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
-  ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass"), "value must be >= 1");
+  ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused"),
+                "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_ln_threads")) {
@@ -98,6 +99,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_vpt2_max_vec")) {
     ATEXN_REQUIRE(value >= 1024 && value <= 1536, "bwd_vpt2_max_vec must be in [1024, 1536]");
     t.bwd_vpt2_max_vec = value;
+  } else if (!strcmp(name, "cl_fused")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "cl_fused must be 0 or 1");
+    t.cl_fused = value;
   } else if (!strcmp(name, "reverse_second_pass")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "reverse_second_pass must be 0 or 1");
     t.reverse_second_pass = value;

@@ -604,4 +604,144 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   }
 }
 
+// ------------------------------------------------------------------ single pass
+// An instance whose pixels fit the registers of one workgroup per channel tile (D <= U pixel
+// slots per thread x pixel slots per block) and a grid that is already wide enough with one
+// slab per instance: one launch, x read once.  Counterpart of the reference's single-kernel
+// shared-memory variant for channels-last (fused_instance_norm_op.cu:1066-1165), with the
+// instance in registers instead of shared memory and an exact two-pass over them (mean, then
+// centred squares) instead of Welford merges.  Grid = (N, 1, channel tiles).
+// y may alias x: a workgroup loads all of its elements before it stores any.
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta, T* y,
+             float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t D, int C,
+             int tpp_shift, float eps) {
+  __shared__ float lds[V * kClThreads];
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
+  Pack<T, V> raw[U];
+  bool ok[U];
+  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  float gm[V], bt[V];
+  load_f32<V>(gamma + g.coff, gm);
+  load_f32<V>(beta + g.coff, bt);
+  float mean[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) mean[i] = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) mean[i] += ok[u] ? to_f32(raw[u].v[i]) : 0.f;
+  }
+  cl_block_sum<V>(mean, lds, TPP);
+  float q[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    mean[i] *= inv_d;
+    q[i] = 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
+      q[i] += d * d;
+    }
+  }
+  __syncthreads();  // the first sum's LDS reads are done
+  cl_block_sum<V>(q, lds, TPP);
+  float rs[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    rs[i] = rsqrtf(q[i] * inv_d + eps);
+    gm[i] *= rs[i];
+  }
+  const int64_t boff = (g.n * D) * C + g.coff;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (ok[u]) {
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) o.v[i] = from_f32<T>((to_f32(raw[u].v[i]) - mean[i]) * gm[i] + bt[i]);
+      store_pack<T, V>(y + boff + (g.slot + static_cast<int64_t>(u) * g.ppb) * C, o);
+    }
+  }
+  if (g.ch_ok && g.slot == 0) {
+    store_f32<V>(mean_out + g.n * C + g.coff, mean);
+    store_f32<V>(rstd_out + g.n * C + g.coff, rs);
+  }
+}
+
+// Backward counterpart: x and dy of the instance in registers (U <= 8 each).  The per-instance
+// sums go to part[n][0][c] = sum dy * xh, part[n][1][c] = sum dy for the column reduction over
+// n that follows; with a single instance they are dgamma / dbeta themselves (out0 / out1 then
+// point at dgamma / dbeta and `stride` is 0).  dx may alias dy.
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads)
+cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
+             const float* __restrict__ mean_in, const float* __restrict__ rstd_in, T* dx,
+             float* __restrict__ out0, float* __restrict__ out1, int64_t stride, int64_t D, int C,
+             int tpp_shift) {
+  __shared__ float lds[2 * V * kClThreads];
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
+  Pack<T, V> rx[U], rd[U];
+  bool ok[U];
+  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
+  cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+  float mu[V], rs[V], sc[V];
+  load_f32<V>(mean_in + g.n * C + g.coff, mu);
+  load_f32<V>(rstd_in + g.n * C + g.coff, rs);
+  load_f32<V>(gamma + g.coff, sc);
+  float acc[2 * V];
+#pragma unroll
+  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = ok[u] ? to_f32(rd[u].v[i]) : 0.f;
+      const float h = ok[u] ? (to_f32(rx[u].v[i]) - mu[i]) * rs[i] : 0.f;
+      acc[i] += d * h;
+      acc[V + i] += d;
+    }
+  }
+  cl_block_sum<2 * V>(acc, lds, TPP);
+  float ca[V], cb[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    sc[i] *= rs[i];
+    ca[i] = -sc[i] * (acc[i] * inv_d);
+    cb[i] = -sc[i] * (acc[V + i] * inv_d);
+  }
+  const int64_t boff = (g.n * D) * C + g.coff;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    if (ok[u]) {
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float h = (to_f32(rx[u].v[i]) - mu[i]) * rs[i];
+        o.v[i] = from_f32<T>(sc[i] * to_f32(rd[u].v[i]) + (ca[i] * h + cb[i]));
+      }
+      store_pack<T, V>(dx + boff + (g.slot + static_cast<int64_t>(u) * g.ppb) * C, o);
+    }
+  }
+  if (g.ch_ok && g.slot == 0) {
+    float t0[V], t1[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      t0[i] = acc[i];
+      t1[i] = acc[V + i];
+    }
+    store_f32<V>(out0 + g.n * stride + g.coff, t0);
+    store_f32<V>(out1 + g.n * stride + g.coff, t1);
+  }
+}
+
 }  // namespace atexn

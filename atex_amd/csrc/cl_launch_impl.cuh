@@ -40,6 +40,22 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
     ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
+    if (p.fused) {
+      const dim3 fgrid(static_cast<unsigned>(N), 1, p.CT);
+#define ATEXN_CL_FWD_FUSED(U_)                                                                 \
+  cl_fwd_fused<T, V, U_><<<fgrid, kClThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, D, Ci,   \
+                                                        p.tpp_shift, eps)
+      switch (p.fused_u) {
+        case 1: ATEXN_CL_FWD_FUSED(1); break;
+        case 2: ATEXN_CL_FWD_FUSED(2); break;
+        case 4: ATEXN_CL_FWD_FUSED(4); break;
+        case 8: ATEXN_CL_FWD_FUSED(8); break;
+        default: ATEXN_CL_FWD_FUSED(16); break;
+      }
+#undef ATEXN_CL_FWD_FUSED
+      ATEXN_CHECK_LAUNCH("cl_fwd_fused");
+      return ATEXN_OK;
+    }
     // a channel count that is not a multiple of V: streaming kernels with an overlapping
     // last channel vector
     if (C % V != 0) { ATEXN_CL_FWD(0, true); return ATEXN_OK; }
@@ -85,6 +101,26 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
     ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
+    if (p.fused) {
+      const dim3 fgrid(static_cast<unsigned>(N), 1, p.CT);
+      // a single instance: its sums are dgamma / dbeta; else per-instance rows for col_reduce
+      float* o0 = N == 1 ? dgamma : part;
+      float* o1 = N == 1 ? dbeta : part + C;
+      const int64_t stride = N == 1 ? 0 : 2 * C;
+#define ATEXN_CL_BWD_FUSED(U_)                                                                 \
+  cl_bwd_fused<T, V, U_><<<fgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, o0, o1,   \
+                                                        stride, D, Ci, p.tpp_shift)
+      switch (p.fused_u) {
+        case 1: ATEXN_CL_BWD_FUSED(1); break;
+        case 2: ATEXN_CL_BWD_FUSED(2); break;
+        case 4: ATEXN_CL_BWD_FUSED(4); break;
+        default: ATEXN_CL_BWD_FUSED(8); break;
+      }
+#undef ATEXN_CL_BWD_FUSED
+      ATEXN_CHECK_LAUNCH("cl_bwd_fused");
+      if (N > 1) return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N), C, st);
+      return ATEXN_OK;
+    }
     if (C % V != 0) { ATEXN_CL_BWD(0, true); return ATEXN_OK; }
     if (p.U == 4) { ATEXN_CL_BWD(4, false); return ATEXN_OK; }
     if (p.U == 8) { ATEXN_CL_BWD(8, false); return ATEXN_OK; }

@@ -36,6 +36,7 @@ struct Tuning {
   int reverse_second_pass = 1;
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
+  int cl_fused = 1;        // channels-last: single-pass kernels when an instance fits a workgroup
   int bwd_wave_groups = 1;  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   int fwd_vpt2_max_vec = 1024;
   int bwd_vpt2_max_vec = 1536;
@@ -306,6 +307,8 @@ struct ClPlan {
   // the slab partials of every instance once (folded[N][2][C]) instead of every stage-2
   // workgroup doing it for itself.
   bool fold = false;
+  bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
+  int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
   size_t off_a = 0, off_b = 0, off_c = 0, off_fold = 0, ws_bytes = 0;
 };
 constexpr int kClFoldAbove = 64;
@@ -343,6 +346,11 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.off_c = 2 * sect;
   p.off_fold = 2 * sect + align256(sizeof(float) * size_t(N) * size_t(C));
   p.fold = p.S > kClFoldAbove && N <= 65535;
+  // (the backward holds x and dy: 16 pixels per thread of both measured no better than two stages)
+  if (t.cl_fused && V > 1 && C % V == 0 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
+    p.fused = true;
+    p.fused_u = std::max(1, pow2_ceil(per_thread));
+  }
   p.ws_bytes = p.off_fold + align256(sizeof(float) * 2 * size_t(N) * size_t(C));
   return p;
 }

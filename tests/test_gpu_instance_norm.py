@@ -177,3 +177,48 @@ def test_deterministic(capi):
             outs.append([t.clone() for t in (y, m, r, dx, dg, db)])
         for a, b in zip(*outs):
             assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("N,C,S", [
+    (1, 32, 216),      # a single instance: its sums are dgamma / dbeta directly
+    (2, 32, 216),
+    (600, 8, 20),      # 1 pixel slot per thread
+    (600, 16, 200),    # 2
+    (300, 64, 100),    # 4
+    (40, 64, 250),     # 8
+    (40, 128, 250),    # 16 forward, two stages backward
+    (3, 4096, 4),      # two channel tiles
+    (5, 520, 31),      # channel vectors not a power of two
+])
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
+    """Instances that fit one workgroup's registers take single-pass kernels; the two-stage
+    kernels stay reachable through the tuning hook.  Both must meet the oracle."""
+    import torch
+
+    capi = util.Capi()
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 77)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, m_ref.astype(np.float32), r_ref.astype(np.float32),
+                                            dtype, False)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    md = torch.from_numpy(m_ref.astype(np.float32)).cuda()
+    rd = torch.from_numpy(r_ref.astype(np.float32)).cuda()
+    tol = TOL[dtype]
+    try:
+        for fused in (1, 0):
+            print(f"IN channels-last N={N} C={C} spatial={S} {dtype} single_pass={fused}", flush=True)
+            assert capi.L.atexn_set_tuning(b"cl_fused", fused) == 0
+            y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+            dx, dg, db = capi.in_bwd(dyd, xd, gd, md, rd, dtype, False)
+            torch.cuda.synchronize()
+            assert_close(util.to_host(m), m_ref, tol["stat"], "mean")
+            assert_close(util.to_host(r), r_ref, tol["stat"], "inv_std")
+            assert_close(util.to_host(y), y_ref, tol["y"], "y")
+            scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), r_ref, dtype)
+            assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx", scale=scale)
+            assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+            assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+    finally:
+        capi.L.atexn_set_tuning(b"cl_fused", 1)
