@@ -8,8 +8,9 @@
 // channels, TPP lanes cover a pixel, and a block of 256 threads sweeps 256 / TPP pixels
 // per step, so every wave-load is a contiguous 1 KiB.  The spatial extent of one
 // instance is cut into S slabs, one block per (instance, slab, channel tile), two launches:
-//   stage 1  per-slab per-channel partial sums -> workspace
-//   stage 2  every block first folds the S partials of its instance and channel tile
+//   stage 1  per-slab per-channel partials (forward: mean and sum of squared deviations;
+//            backward: the two sums) -> workspace
+//   stage 2  every block first merges the S partials of its instance and channel tile
 //            (a few KiB from L2) into LDS, then applies; no separate finalize launch.
 // Small slabs stay in registers between their (single, fully overlapped) batch of loads
 // and their use.
@@ -174,97 +175,165 @@ __device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, i
   }
 }
 
-// Pivot of an instance, per channel: the median of the channel's values at the first, the
-// middle and the last pixel.  Forward statistics are accumulated as sum(x - K) and
-// sum((x - K)^2) around this pivot K, which every slab of the instance shares, so slabs
-// (and threads) combine by plain addition, and
-//     mean = K + S1 / D,   var = S2 / D - (S1 / D)^2
-// loses only a factor (1 + (K - mean)^2 / var) of precision; the median of three samples
-// keeps K within the bulk of the data even when one sample is an outlier.
-template <typename T, int V>
-__device__ __forceinline__ void cl_pivot(const T* xn_c, int64_t D, int C, float (&k)[V]) {
-  const Pack<T, V> a = load_pack<T, V>(xn_c);
-  const Pack<T, V> b = load_pack<T, V>(xn_c + (D / 2) * C);
-  const Pack<T, V> c = load_pack<T, V>(xn_c + (D - 1) * C);
-#pragma unroll
-  for (int i = 0; i < V; ++i) {
-    k[i] = __builtin_amdgcn_fmed3f(to_f32(a.v[i]), to_f32(b.v[i]), to_f32(c.v[i]));
-  }
+// Count of pixels of slab s when an instance of D pixels is cut into slabs of slab_len.
+__device__ __forceinline__ float cl_slab_count(int s, int64_t D, int64_t slab_len) {
+  const int64_t beg = static_cast<int64_t>(s) * slab_len;
+  return static_cast<float>(beg + slab_len <= D ? slab_len : D - beg);
 }
 
 // ---------------------------------------------------------------- forward, stage 1
-// psum: [N * S][2][C] sums of (x - K) and (x - K)^2 over each slab, K = cl_pivot, which
-// is saved to pivot[N, C].
-// U > 0: the slab is register-resident (slab_len <= U * pixel slots per block) and all its
-// loads are in flight at once; U == 0 streams the slab in batches.
+// pstat: [N * S][2][C], the (mean, m2 = sum of squared deviations from that mean) of every
+// channel over each slab; the slab's pixel count follows from the geometry.  Nothing is
+// accumulated around a pivot or around zero, so the result keeps float32 accuracy whatever
+// the data look like (an instance whose border pixels are far from the bulk, a large common
+// offset): the counterpart of the reference's Welford pushes (norm_util.h:182-211).
+// U > 0: the slab is register-resident (slab_len <= U * pixel slots per block), all its
+// loads are in flight at once and the statistics are an exact two-pass over the registers
+// (block-wide sum -> slab mean, block-wide sum of squared deviations from it).
+// U == 0 streams the slab in batches of 8 pixels per thread: per-thread running (mean, m2)
+// by batch-wise Chan updates (wf_lanes_push), combined over the block around the slab mean
+// (m2 = sum over threads of m2_t + n_t (mean_t - mean)^2, every term non-negative).
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
-cl_fwd_stats(const T* __restrict__ x, float* __restrict__ psum, float* __restrict__ pivot,
-             int64_t D, int C, int S, int tpp_shift,
-             int64_t slab_len) {
-  __shared__ float lds[2 * V * kClThreads];
+cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int C, int S,
+             int tpp_shift, int64_t slab_len) {
+  __shared__ float lds[V * kClThreads];
   const int CV = (C + V - 1) / V;
   const int TPP = 1 << tpp_shift;
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   const T* xn = x + (g.n * D) * C;
-  float k0[V];
-  cl_pivot<T, V>(xn + g.coff, D, C, k0);
-  float acc[2 * V];
-#pragma unroll
-  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
-  auto add = [&](const Pack<T, V>& pk, bool valid) {
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const float d = valid ? to_f32(pk.v[i]) - k0[i] : 0.f;
-      acc[i] += d;
-      acc[V + i] += d * d;
-    }
-  };
+  const float inv_n = 1.0f / static_cast<float>(g.p1 - g.p0);
+  float mean[V], m2[V];
   if constexpr (U > 0) {
     Pack<T, V> raw[U];
     bool ok[U];
     cl_load_slab<T, V, U>(xn, g, CV, C, raw, ok);
 #pragma unroll
-    for (int u = 0; u < U; ++u) add(raw[u], ok[u]);
-  } else if (g.ch_ok) {
-    const T* base = xn + g.coff;
-    constexpr int B = 8;
-    cl_for_pixels<B>(
-        g,
-        [&](int64_t p, int64_t step) {
-          Pack<T, V> pk[B];
+    for (int i = 0; i < V; ++i) mean[i] = 0.f;
 #pragma unroll
-          for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(base + (p + u * step) * C);
+    for (int u = 0; u < U; ++u) {
 #pragma unroll
-          for (int u = 0; u < B; ++u) add(pk[u], true);
-        },
-        [&](int64_t p) { add(load_pack<T, V>(base + p * C), true); });
-  }
-  cl_block_sum<2 * V>(acc, lds, TPP);
-  if (g.ch_ok && g.slot == 0) {
-    float t1[V], t2[V];
+      for (int i = 0; i < V; ++i) mean[i] += ok[u] ? to_f32(raw[u].v[i]) : 0.f;
+    }
+    cl_block_sum<V>(mean, lds, TPP);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      t1[i] = acc[i];
-      t2[i] = acc[V + i];
+      mean[i] *= inv_n;
+      m2[i] = 0.f;
     }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
+        m2[i] += d * d;
+      }
+    }
+  } else {
+    WfLanes<V> run;
+    wf_lanes_init<V>(run);
+    if (g.ch_ok) {
+      const T* base = xn + g.coff;
+      constexpr int B = 8;
+      cl_for_pixels<B>(
+          g,
+          [&](int64_t p, int64_t step) {
+            Pack<T, V> pk[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(base + (p + u * step) * C);
+            float f[B][V];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+#pragma unroll
+              for (int i = 0; i < V; ++i) f[u][i] = to_f32(pk[u].v[i]);
+            }
+            wf_lanes_push<V, B>(run, f);
+          },
+          [&](int64_t p) {
+            const Pack<T, V> pk = load_pack<T, V>(base + p * C);
+            float f[1][V];
+#pragma unroll
+            for (int i = 0; i < V; ++i) f[0][i] = to_f32(pk.v[i]);
+            wf_lanes_push<V, 1>(run, f);
+          });
+    }
+#pragma unroll
+    for (int i = 0; i < V; ++i) mean[i] = run.mean[i] * run.n;
+    cl_block_sum<V>(mean, lds, TPP);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      mean[i] *= inv_n;
+      const float d = run.mean[i] - mean[i];
+      m2[i] = run.m2[i] + run.n * (d * d);
+    }
+  }
+  __syncthreads();  // the first sum's LDS reads are done
+  cl_block_sum<V>(m2, lds, TPP);
+  if (g.ch_ok && g.slot == 0) {
     const int64_t o = ((g.n * S + g.s) * 2) * C + g.coff;
-    store_f32_from<V>(psum + o, t1, RG ? g.lo : 0);
-    store_f32_from<V>(psum + o + C, t2, RG ? g.lo : 0);
-    // stage 2 must not re-read the pivot from x: y may alias x and be half written by then
-    if (g.s == 0) store_f32_from<V>(pivot + g.n * C + g.coff, k0, RG ? g.lo : 0);
+    store_f32_from<V>(pstat + o, mean, RG ? g.lo : 0);
+    store_f32_from<V>(pstat + o + C, m2, RG ? g.lo : 0);
+  }
+}
+
+// Between the stages, only when an instance has more than kClFoldAbove slabs: merges the S slab
+// statistics of every (instance, channel) once, in a fixed order, into folded[N][2][C] = (mean,
+// m2 of the whole instance), so that the stage-2 workgroups need not each do it.  Block =
+// kClMergeChannels channels x (256 / kClMergeChannels) slab phases; grid = (channel groups, N).
+constexpr int kClMergeChannels = 16;
+__global__ void __launch_bounds__(kClThreads)
+cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int64_t D, int C, int S,
+               int64_t slab_len) {
+  constexpr int PH = kClThreads / kClMergeChannels;
+  __shared__ Wf buf[PH][kClMergeChannels];
+  const int cx = threadIdx.x % kClMergeChannels;
+  const int ph = threadIdx.x / kClMergeChannels;
+  const int c = blockIdx.x * kClMergeChannels + cx;
+  const int64_t n = blockIdx.y;
+  Wf w{0.f, 0.f, 0.f};
+  if (c < C) {
+    const float* q = pstat + ((n * S) * 2) * C + c;
+    constexpr int B = 8;
+    batched_for<B>(
+        ph, S, PH,
+        [&](int64_t sl, int64_t step) {
+          float tm[B], tq[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            tm[u] = q[((sl + u * step) * 2) * C];
+            tq[u] = q[((sl + u * step) * 2 + 1) * C];
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, slab_len)});
+          }
+        },
+        [&](int64_t sl) {
+          w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
+                             cl_slab_count(static_cast<int>(sl), D, slab_len)});
+        });
+  }
+  buf[ph][cx] = w;
+  __syncthreads();
+  if (ph == 0 && c < C) {
+    Wf r = buf[0][cx];
+    for (int k = 1; k < PH; ++k) r = wf_merge(r, buf[k][cx]);
+    folded[(n * 2) * C + c] = r.mean;
+    folded[(n * 2 + 1) * C + c] = r.m2;
   }
 }
 
 // ---------------------------------------------------------------- forward, stage 2
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
+// pstat holds S partial (mean, m2) rows per instance whose counts follow from cnt_len (the
+// slab length; after cl_merge_stats: S == 1 and cnt_len == D).
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
-cl_fwd_apply(const T* x, const float* __restrict__ psum, const float* __restrict__ pivot, const float* __restrict__ gamma,
+cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restrict__ gamma,
              const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
-             float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
-             int64_t slab_len, float eps, int rev) {
+             float* __restrict__ rstd_out, int64_t D, int C, int S, int64_t cnt_len,
+             int tpp_shift, int64_t slab_len, float eps, int rev) {
   __shared__ float sm_mean[kClMaxTileChannels];
   __shared__ float sm_rstd[kClMaxTileChannels];
   const int CV = (C + V - 1) / V;
@@ -273,57 +342,55 @@ cl_fwd_apply(const T* x, const float* __restrict__ psum, const float* __restrict
   const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
-  // resident slab: its loads are issued first and fly while the partials are folded
+  // resident slab: its loads are issued first and fly while the partials are merged
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, raw, ok);
-  // phase A: add up the S slab partials of every channel of the tile, finish the
-  // statistics around the pivot
+  // phase A: Chan-merge the S slab statistics of every channel of the tile (each of the
+  // fm.P lanes of a channel takes every P-th slab in order, then the lanes merge pairwise;
+  // the merge is bitwise symmetric, so every workgroup of the instance gets the same bits)
   const int c_base = g.ct * cap;
   for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
     const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
     const int sub = static_cast<int>(threadIdx.x) % fm.P;
     const int c = c_base + cl;
     const bool in = cl < cap && c < C;
-    float s1 = 0.f, s2 = 0.f, kc = 0.f;
+    Wf w{0.f, 0.f, 0.f};
     if (in) {
-      const float* q1 = psum + ((g.n * S) * 2) * C + c;
-      const float* q2 = q1 + C;
-      if (sub == 0) kc = pivot[g.n * C + c];
-      constexpr int B = 16;
+      const float* q = pstat + ((g.n * S) * 2) * C + c;
+      constexpr int B = 8;
       batched_for<B>(
           sub, S, fm.P,
           [&](int64_t sl, int64_t step) {
-            float t1[B], t2[B];
+            float tm[B], tq[B];
 #pragma unroll
             for (int u = 0; u < B; ++u) {
-              t1[u] = q1[((sl + u * step) * 2) * C];
-              t2[u] = q2[((sl + u * step) * 2) * C];
+              tm[u] = q[((sl + u * step) * 2) * C];
+              tq[u] = q[((sl + u * step) * 2 + 1) * C];
             }
 #pragma unroll
             for (int u = 0; u < B; ++u) {
-              s1 += t1[u];
-              s2 += t2[u];
+              w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, cnt_len)});
             }
           },
           [&](int64_t sl) {
-            s1 += q1[(sl * 2) * C];
-            s2 += q2[(sl * 2) * C];
+            w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
+                               cl_slab_count(static_cast<int>(sl), D, cnt_len)});
           });
     }
     for (int m = 1; m < fm.P; m <<= 1) {
-      s1 += lane_xor(s1, m);
-      s2 += lane_xor(s2, m);
+      Wf o;
+      o.mean = lane_xor(w.mean, m);
+      o.m2 = lane_xor(w.m2, m);
+      o.n = lane_xor(w.n, m);
+      w = wf_merge(w, o);
     }
     if (sub == 0 && in) {
-      const float dm = s1 * inv_d;
-      const float mean = kc + dm;
-      const float var = fmaxf(s2 * inv_d - dm * dm, 0.f);
-      const float rs = rsqrtf(var + eps);
-      sm_mean[cl] = mean;
+      const float rs = rsqrtf(w.m2 * inv_d + eps);
+      sm_mean[cl] = w.mean;
       sm_rstd[cl] = rs;
       if (g.s == 0) {
-        mean_out[g.n * C + c] = mean;
+        mean_out[g.n * C + c] = w.mean;
         rstd_out[g.n * C + c] = rs;
       }
     }

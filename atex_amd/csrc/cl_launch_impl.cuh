@@ -14,8 +14,7 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   const ClPlan p = plan_cl(false, V, N, C, D, cu_count());
   ATEXN_REQUIRE(ws != nullptr && ws_bytes >= p.ws_bytes,
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
-  float* psum = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
-  float* pivot = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_c);
+  float* pstat = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_a);
   float* folded = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_fold);
   const int Ci = static_cast<int>(C);
   // one workgroup column per instance: the launch's x extent N * 256 must stay below 2^32
@@ -24,17 +23,19 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_FWD(U_, RG_)                                                                  \
   do {                                                                                        \
-    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, psum, pivot, D, Ci, p.S,         \
-                                                       p.tpp_shift, p.slab_len);              \
+    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pstat, D, Ci, p.S, p.tpp_shift,  \
+                                                       p.slab_len);                           \
     ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
     if (p.fold) {                                                                             \
-      const int rc = launch_col_reduce(psum, folded, folded + C, p.S, C, st,                  \
-                                       static_cast<int>(N), int64_t(p.S) * 2 * C, 2 * C);     \
-      if (rc != ATEXN_OK) return rc;                                                          \
+      const dim3 mgrid(static_cast<unsigned>(div_up(C, kClMergeChannels)),                    \
+                       static_cast<unsigned>(N));                                             \
+      cl_merge_stats<<<mgrid, kClThreads, 0, st>>>(pstat, folded, D, Ci, p.S, p.slab_len);    \
+      ATEXN_CHECK_LAUNCH("cl_merge_stats");                                                   \
     }                                                                                         \
-    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, p.fold ? folded : psum, pivot,   \
-                                                       gamma, beta, y, mean, rstd, D, Ci,     \
-                                                       p.fold ? 1 : p.S, p.tpp_shift,         \
+    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, p.fold ? folded : pstat, gamma,  \
+                                                       beta, y, mean, rstd, D, Ci,            \
+                                                       p.fold ? 1 : p.S,                      \
+                                                       p.fold ? D : p.slab_len, p.tpp_shift,  \
                                                        p.slab_len, eps,                       \
                                                        tuning().reverse_second_pass);         \
     ATEXN_CHECK_LAUNCH("cl_fwd_apply");                                                       \

@@ -371,6 +371,73 @@ __device__ __forceinline__ float block_sum1(float a, float* buf) {
   return r;
 }
 
+// Streaming statistics without a pivot: a thread takes its values in small register-resident
+// batches, gets each batch's (mean, m2) by an exact two-pass over the registers and merges it
+// into its running triple with Chan's update (reference: norm_util.h:190-210, whose per-element
+// push is the batch-of-one case).  No term is a difference of large sums, so an outlier
+// anywhere in the data costs no precision; per element it is one add, one subtract and one
+// FMA, the merge (a reciprocal and ten operations) is shared by the whole batch.
+__device__ __forceinline__ void wf_push_batch(Wf& run, float batch_mean, float batch_m2, float nb) {
+  const float n = run.n + nb;
+  const float w = nb * fast_rcp(n);
+  const float d = batch_mean - run.mean;
+  run.m2 += batch_m2 + (d * d) * (run.n * w);
+  run.mean += d * w;
+  run.n = n;
+}
+template <int N>
+__device__ __forceinline__ void wf_push(Wf& run, const float (&f)[N]) {
+  float s = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) s += f[i];
+  const float mb = s * (1.0f / N);
+  float q = 0.f;
+#pragma unroll
+  for (int i = 0; i < N; ++i) {
+    const float d = f[i] - mb;
+    q += d * d;
+  }
+  wf_push_batch(run, mb, q, static_cast<float>(N));
+}
+
+// The same for V independent streams that advance together (the V channels of a thread's
+// channel vector): one count, one reciprocal per batch.
+template <int V>
+struct WfLanes {
+  float mean[V], m2[V];
+  float n;
+};
+template <int V>
+__device__ __forceinline__ void wf_lanes_init(WfLanes<V>& w) {
+#pragma unroll
+  for (int i = 0; i < V; ++i) w.mean[i] = w.m2[i] = 0.f;
+  w.n = 0.f;
+}
+// f[u][i]: value u of stream i; all B values of every stream are valid.
+template <int V, int B>
+__device__ __forceinline__ void wf_lanes_push(WfLanes<V>& run, const float (&f)[B][V]) {
+  const float n = run.n + static_cast<float>(B);
+  const float w = static_cast<float>(B) * fast_rcp(n);
+  const float cross = run.n * w;
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    float s = 0.f;
+#pragma unroll
+    for (int u = 0; u < B; ++u) s += f[u][i];
+    const float mb = s * (1.0f / B);
+    float q = 0.f;
+#pragma unroll
+    for (int u = 0; u < B; ++u) {
+      const float d = f[u][i] - mb;
+      q += d * d;
+    }
+    const float d = mb - run.mean[i];
+    run.m2[i] += q + (d * d) * cross;
+    run.mean[i] += d * w;
+  }
+  run.n = n;
+}
+
 // Statistics of the V*NV register-resident values of one thread (exact two-pass, the
 // data is on chip), as a Welford triple.  valid[k] tells whether vector k is inside the
 // row; elements of a valid vector are all valid.

@@ -309,7 +309,7 @@ struct ClPlan {
   bool fold = false;
   bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
   int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
-  size_t off_a = 0, off_b = 0, off_c = 0, off_fold = 0, ws_bytes = 0;
+  size_t off_a = 0, off_fold = 0, ws_bytes = 0;
 };
 constexpr int kClFoldAbove = 64;
 
@@ -340,11 +340,10 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
     }
   }
   const size_t sect = align256(sizeof(float) * size_t(N) * size_t(p.S) * size_t(C));
+  // fwd: slab statistics [N*S][2][C] (mean, m2); bwd: part[N*S][2][C]; then the per-instance
+  // merge of either, folded[N][2][C]
   p.off_a = 0;
-  p.off_b = sect;
-  // fwd: slab sums S1, S2 [N*S, C] and the pivots [N, C]; bwd: part[N*S][2][C] (contiguous)
-  p.off_c = 2 * sect;
-  p.off_fold = 2 * sect + align256(sizeof(float) * size_t(N) * size_t(C));
+  p.off_fold = 2 * sect;
   p.fold = p.S > kClFoldAbove && N <= 65535;
   // (the backward holds x and dy: 16 pixels per thread of both measured no better than two stages)
   if (t.cl_fused && V > 1 && C % V == 0 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {

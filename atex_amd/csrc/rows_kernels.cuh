@@ -661,58 +661,42 @@ __device__ __forceinline__ int64_t split_pos(int64_t p, int64_t n_vec, bool rev)
   return rev ? n_vec - 1 - p : p;
 }
 
-// Statistics of a chunk as a Welford triple.  Each thread accumulates sum(x - K) and
-// sum((x - K)^2) around its own pivot K = the first element it owns (two FMAs per element,
-// no division), converts to (mean, m2, n) at the end, and the block merges the threads'
-// triples with Chan's formula.  A thread's pivot is one of its own samples, so the shifted
-// sums lose precision only when that sample is an outlier of the thread's data, and then
-// only in that thread's share.
+// Statistics of a chunk as a Welford triple.  Each thread takes its vectors in batches of
+// kSplitBatch (all loads in flight), gets each batch's (mean, m2) from an exact two-pass over
+// the registers and merges it into its running triple (wf_push); the block then merges the
+// threads' triples with Chan's formula.  There is no pivot: no sample, however far from the
+// rest, costs the others any precision.
 template <typename T, int V>
 __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
   const int64_t n_vec = len / V;
   const int rem = static_cast<int>(len % V);  // only the last chunk of a ragged row
   const int64_t tid = threadIdx.x;
   const bool has_tail = rem != 0 && n_vec % blockDim.x == tid;
-  if (tid >= n_vec && !has_tail) return Wf{0.f, 0.f, 0.f};
-  const float K = to_f32(p[tid < n_vec ? tid * V : n_vec * V]);
-  float s1 = 0.f, s2 = 0.f;
-  int64_t cnt = 0;
-  auto acc = [&](const Pack<T, V>& pk) {
-#pragma unroll
-    for (int k = 0; k < V; ++k) {
-      const float d = to_f32(pk.v[k]) - K;
-      s1 += d;
-      s2 += d * d;
-    }
-  };
+  Wf w{0.f, 0.f, 0.f};
   batched_for<kSplitBatch>(
       tid, n_vec, blockDim.x,
       [&](int64_t v, int64_t step) {
         Pack<T, V> pk[kSplitBatch];
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u) pk[u] = load_pack<T, V>(p + (v + u * step) * V);
+        float f[kSplitBatch * V];
 #pragma unroll
-        for (int u = 0; u < kSplitBatch; ++u) acc(pk[u]);
-        cnt += kSplitBatch * V;
+        for (int u = 0; u < kSplitBatch; ++u) {
+#pragma unroll
+          for (int k = 0; k < V; ++k) f[u * V + k] = to_f32(pk[u].v[k]);
+        }
+        wf_push<kSplitBatch * V>(w, f);
       },
       [&](int64_t v) {
-        acc(load_pack<T, V>(p + v * V));
-        cnt += V;
+        const Pack<T, V> pk = load_pack<T, V>(p + v * V);
+        float f[V];
+#pragma unroll
+        for (int k = 0; k < V; ++k) f[k] = to_f32(pk.v[k]);
+        wf_push<V>(w, f);
       });
   if (has_tail) {
-    for (int k = 0; k < rem; ++k) {
-      const float d = to_f32(p[n_vec * V + k]) - K;
-      s1 += d;
-      s2 += d * d;
-    }
-    cnt += rem;
+    for (int k = 0; k < rem; ++k) wf_push_batch(w, to_f32(p[n_vec * V + k]), 0.f, 1.f);
   }
-  Wf w;
-  w.n = static_cast<float>(cnt);
-  const float inv = 1.0f / w.n;
-  const float dm = s1 * inv;
-  w.mean = K + dm;
-  w.m2 = fmaxf(s2 - s1 * dm, 0.f);
   return w;
 }
 

@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 from tests import util
+from tests.util import assert_close
 
 pytestmark = pytest.mark.gpu
 
@@ -61,6 +62,61 @@ def test_instance_norm_offset(coracle, N, C, S, channel_first, kappa):
     assert np.max(np.abs(util.to_host(m) - m_ref) / np.abs(m_ref)) <= b["mean"]
     assert np.max(np.abs(util.to_host(r) - r_ref) / r_ref) <= b["rstd"]
     assert np.max(np.abs(util.to_host(y) - y_ref)) <= b["y"] * 2.0
+
+
+# Kernel families whose statistics stream through the data (everything that is not an exact
+# two-pass over a register-resident row): name -> (layout, N, C, D).  "cl" = channels-last.
+OUTLIER_CASES = {
+    "channels-last, register slabs, 64 slabs merged by stage 2": ("cl", 8, 64, 16384),
+    "channels-last, streaming slabs merged by stage 2": ("cl", 8, 32, 1 << 17),
+    "channels-last, register slabs, merge launch": ("cl", 1, 8, 1 << 19),
+    "channels-last, streaming slabs, merge launch": ("cl", 1, 32, 1 << 19),
+    "channels-last, C not a multiple of the vector": ("cl", 16, 6, 5000),
+    "channels-last, C not a multiple of the vector, merge launch": ("cl", 2, 6, 50000),
+    "channels-last, single pass": ("cl", 512, 32, 256),
+    "channel-first, planes split over workgroups": ("cf", 1, 3, 1 << 19),
+    "LayerNorm tiles (rows too long for registers)": ("ln", 6, 1, 70001),
+}
+
+
+@pytest.mark.parametrize("kappa", [100.0, 1000.0])
+@pytest.mark.parametrize("case", sorted(OUTLIER_CASES))
+def test_outlier_samples(coracle, case, kappa):
+    """The bulk of every instance / row is N(kappa, 1) while the places a kernel could take a
+    pivot or a first sample from are 0, i.e. kappa standard deviations away: the first, middle
+    and last pixel of an instance (an image with zero-padded corners), and the first element of
+    the first few threads' shares of a row.  Statistics must keep the float32 tolerance: the
+    reference's Welford pushes do (norm_util.h:182-211)."""
+    import torch
+
+    layout, N, C, D = OUTLIER_CASES[case]
+    capi = util.Capi()
+    rng = util.rng_for(302)
+    print(f"outlier samples: {case} kappa={kappa} N={N} C={C} D={D}", flush=True)
+    if layout == "ln":
+        x = (rng.standard_normal((N, D)) + kappa).astype(np.float32)
+        x[:, [0, 4, 8, 12, D // 2, D - 1]] = 0
+        gamma, beta = util.affine_params(rng, D)
+        y_ref, m_ref, r_ref = coracle.ln_fwd(x, gamma, beta, EPS, "f32")
+        y, m, r = capi.ln_fwd(torch.from_numpy(x).cuda(), torch.from_numpy(gamma).cuda(),
+                              torch.from_numpy(beta).cuda(), EPS, "f32")
+    else:
+        x = (rng.standard_normal((N, D, C)) + kappa).astype(np.float32)
+        x[:, [0, 1, 2, 3, D // 2, D - 1], :] = 0
+        cf = layout == "cf"
+        if cf:
+            x = np.ascontiguousarray(np.transpose(x, (0, 2, 1)))
+            x[:, :, [4, 8, 12]] = 0
+        gamma, beta = util.affine_params(rng, C)
+        y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, "f32", cf)
+        y, m, r = capi.in_fwd(torch.from_numpy(x).cuda(), torch.from_numpy(gamma).cuda(),
+                              torch.from_numpy(beta).cuda(), EPS, "f32", cf)
+    torch.cuda.synchronize()
+    tol = util.TOL["f32"]["stat"]
+    assert_close(util.to_host(m), m_ref, tol, "mean")
+    assert_close(util.to_host(r), r_ref, tol, "inv_std")
+    # y = (x - mean) * r: x - mean carries the float32 rounding of mean, 6e-8 * kappa
+    assert np.max(np.abs(util.to_host(y) - y_ref) / (1.0 + np.abs(y_ref))) <= 1e-5 + 40 * 6e-8 * kappa
 
 
 def test_constant_rows_and_extremes():

@@ -1,5 +1,13 @@
-"""Benchmark configuration 4 at its full size, x fp16 [2, 128, 128, 128, 32] (both layouts),
-through the op-level entry points.  The oracle still runs in a few seconds on the box's
+"""Benchmark configurations 2 and 4 at their full sizes.
+
+Configuration 2 (LayerNorm hidden-size sweep, [262144, 128], [16384, 4096], [2048, 12288] in
+fp16 and bf16) runs through the kernel-level entry points against the oracle's float64
+flavour on every element: the launch plan depends on the row count (rows per lane group,
+block size, grid), so the instantiations that run at the full row counts are not the ones a
+reduced row count selects.
+
+Configuration 4, x fp16 [2, 128, 128, 128, 32] (both layouts), runs through the op-level
+entry points.  The oracle still runs in a few seconds on the box's
 cores for one forward + backward, so the values are compared directly; on top of that come
 the size-independent properties the statistics must satisfy whatever the size:
 
@@ -8,8 +16,8 @@ the size-independent properties the statistics must satisfy whatever the size:
 * dbeta = sum(dy), dgamma = sum(dy * xhat) recomputed from the returned statistics;
 * the two layouts give the same statistics and weight gradients for transposed inputs.
 
-The other configurations already run at full size in test_gpu_layer_norm.py
-(configs 0-2) and test_gpu_instance_norm.py (config 3).
+Configurations 0 and 1 run at full size in test_gpu_layer_norm.py, configuration 3 in
+test_gpu_instance_norm.py.
 """
 import numpy as np
 import pytest
@@ -21,6 +29,14 @@ pytestmark = pytest.mark.gpu
 
 EPS = 1e-3
 N, C, SP = 2, 32, (128, 128, 128)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16"])
+@pytest.mark.parametrize("rows,D", [(262144, 128), (16384, 4096), (2048, 12288)])
+def test_config2_full_row_counts(coracle, rows, D, dtype):
+    from tests.test_gpu_layer_norm import run_case
+
+    run_case(util.Capi(), coracle, "scaled_rows", rows, D, dtype, 2)
 
 
 @pytest.fixture(scope="module")
