@@ -7,12 +7,19 @@
 // which stays with the caller.
 #include <algorithm>
 #include <cstring>
+#include <mutex>
 #include <vector>
 
 #include "plan.h"
 #include "status.h"
 
 using namespace atexn;
+
+// Device scratch of atexn_layer_norm_bwd_static: part of the library's code object, so every
+// GPU the library runs on holds its own copy from module load until the process ends.  In host
+// code the array's name is only a handle; its device address comes from hipGetSymbolAddress,
+// once per device, and only that address is ever handed to a kernel.
+static __device__ __align__(256) unsigned char scratch[ATEXN_STATIC_SCRATCH_BYTES];
 
 namespace {
 
@@ -49,6 +56,32 @@ int check_tensor(const atexn_tensor* t, const char* name) {
     int s_ = (expr);                \
     if (s_ != ATEXN_OK) return s_;  \
   } while (0)
+
+constexpr int kMaxDevices = 64;
+std::mutex g_scratch_mutex;
+void* g_scratch_ptr[kMaxDevices] = {};
+
+// Address of `scratch` on the current device (looked up on the first call per device).
+int static_scratch(void** out) {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "hipGetDevice: %s", hipGetErrorString(e));
+  ATEXN_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d not supported (limit %d)", dev,
+                kMaxDevices);
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || p == nullptr) {
+      (void)hipGetLastError();
+      return set_error(ATEXN_LAUNCH_ERROR, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                       hipGetErrorString(e));
+    }
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return ATEXN_OK;
+}
 
 }  // namespace
 
@@ -155,6 +188,24 @@ int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* 
   ATEXN_REQUIRE(workspace != nullptr && ws_aligned(workspace), "workspace must be non-NULL and 256-byte aligned");
   return rows_bwd(dtype, false, dy, x, gamma, mean, inv_std, N, D, 1, dx, dgamma, dbeta, workspace,
                   workspace_bytes, st);
+}
+
+int atexn_layer_norm_bwd_static(int dtype, const void* dy, const void* x, const float* gamma,
+                                const float* mean, const float* inv_std, int64_t N, int64_t D,
+                                void* dx, float* dgamma, float* dbeta, void* stream) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
+  const size_t need = rows_bwd_ws(dtype, false, N, D, 1);
+  ATEXN_REQUIRE(need <= sizeof(scratch),
+                "LayerNorm backward of [%lld, %lld] needs %zu bytes of scratch, more than the %zu "
+                "bytes of the static buffer: use atexn_layer_norm_bwd with a workspace",
+                (long long)N, (long long)D, need, sizeof(scratch));
+  void* ws = nullptr;
+  if (need > 0) ATEXN_TRY(static_scratch(&ws));
+  // the kernels overwrite every scratch word they later read (one partial dgamma / dbeta row
+  // per workgroup, per-row sums), so nothing has to be cleared between calls
+  return atexn_layer_norm_bwd(dtype, dy, x, gamma, mean, inv_std, N, D, dx, dgamma, dbeta, ws,
+                              sizeof(scratch), stream);
 }
 
 size_t atexn_instance_norm_fwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,

@@ -52,6 +52,7 @@ SIGNATURES = {
     "atexn_layer_norm_fwd": (_i, [_i, _vp, _vp, _vp, _i64, _i64, _f, _vp, _vp, _vp, _vp, _sz, _vp]),
     "atexn_layer_norm_bwd_workspace_bytes": (_sz, [_i, _i64, _i64]),
     "atexn_layer_norm_bwd": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "atexn_layer_norm_bwd_static": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp, _vp]),
     "atexn_instance_norm_fwd_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64]),
     "atexn_instance_norm_fwd": (_i, [_i, _i, _vp, _vp, _vp, _i64, _i64, _i64, _f, _vp, _vp, _vp, _vp, _sz, _vp]),
     "atexn_instance_norm_bwd_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64]),

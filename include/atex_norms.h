@@ -19,7 +19,10 @@
  *   - the saved statistics are the mean and the INVERSE STANDARD DEVIATION
  *     rsqrt(biased_variance + epsilon) (reference: cc/kernels/norm_util.h:253-258);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); every call is
- *     asynchronous on it, re-entrant, allocates nothing and keeps no device state;
+ *     asynchronous on it, re-entrant, allocates nothing and keeps no device state
+ *     (atexn_layer_norm_bwd_static is the one exception, see there);
+ *   - the device the stream belongs to must be the calling thread's current device: launch
+ *     plans and workspace sizes are made for the current device's compute-unit count;
  *   - data pointers need only the alignment of their element type (2 or 4 bytes): the
  *     kernels' 16-byte accesses work at any element offset, so slices of larger tensors
  *     can be passed as they are;
@@ -80,6 +83,24 @@ int atexn_layer_norm_bwd(int dtype, const void* dy, const void* x, const float* 
                          const float* mean, const float* inv_std, int64_t N, int64_t D,
                          void* dx, float* dgamma, float* dbeta, void* workspace,
                          size_t workspace_bytes, void* stream);
+
+/* atexn_layer_norm_bwd without a workspace argument, for callers that cannot allocate device
+ * memory at the point of the call (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  It has no counterpart in the reference, whose functor allocates its
+ * scratch through the framework.  The scratch is a static device array of
+ * ATEXN_STATIC_SCRATCH_BYTES inside the library (every GPU the library runs on holds it from
+ * module load to process exit); the call allocates and frees nothing.  Problems whose
+ * atexn_layer_norm_bwd_workspace_bytes exceeds that size are rejected with
+ * ATEXN_INVALID_ARGUMENT.  All calls on one GPU share the one array: calls that overlap in
+ * time on the same GPU (two streams, two threads) race; serialise them or use
+ * atexn_layer_norm_bwd with separate workspaces.  Nothing has to be cleared between calls
+ * (the kernels write every scratch word before they read it).  The first call on a device
+ * looks the array's address up (hipGetSymbolAddress); make that call outside stream capture.
+ * Results are bit-identical to atexn_layer_norm_bwd. */
+#define ATEXN_STATIC_SCRATCH_BYTES (8u << 20)
+int atexn_layer_norm_bwd_static(int dtype, const void* dy, const void* x, const float* gamma,
+                                const float* mean, const float* inv_std, int64_t N, int64_t D,
+                                void* dx, float* dgamma, float* dbeta, void* stream);
 
 /* Replaces functor::FusedInstanceNorm<GPUDevice,T,U>::operator()
  * (cc/kernels/fused_instance_norm_op.cu:1458-1517). mean / inv_std are [N, C] in both
