@@ -1,10 +1,15 @@
 """Builds libatex_norms_hip.so in-tree with hipcc for gfx950.
 
-    python -m atex_amd.build [--force]
+    python -m atex_amd.build [--force] [--product-only]
 
 Each .hip translation unit is compiled to an object (in parallel), then linked into
 atex_amd/lib/libatex_norms_hip.so.  No CMake, no torch: the library depends only on the HIP
 runtime.
+
+A second library, libatex_norms_hip_bench.so, is the same sources compiled with
+-DATEXN_BENCH_BUILD: it adds one tuning switch ("bwd_stage_mask", run only the row kernel of
+a backward call) that bench.py uses to time the dominant kernel alone.  Nothing but bench.py
+loads it.
 """
 from __future__ import annotations
 
@@ -18,6 +23,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ_DIR = os.path.join(HERE, "build")
 LIB_DIR = os.path.join(HERE, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libatex_norms_hip.so")
+BENCH_LIB_PATH = os.path.join(LIB_DIR, "libatex_norms_hip_bench.so")
 
 SOURCES = [
     "capi.hip",
@@ -57,12 +63,12 @@ def _deps_mtime() -> float:
     return m
 
 
-def _compile(src: str, force: bool, dep_m: float) -> str:
-    obj = os.path.join(OBJ_DIR, src.replace(".hip", ".o"))
+def _compile(src: str, force: bool, dep_m: float, bench: bool) -> str:
+    obj = os.path.join(OBJ_DIR, src.replace(".hip", "_bench.o" if bench else ".o"))
     s = os.path.join(CSRC, src)
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(s), dep_m):
         return obj
-    cmd = [_hipcc(), *HIPCC_FLAGS, "-c", s, "-o", obj]
+    cmd = [_hipcc(), *HIPCC_FLAGS, *(["-DATEXN_BENCH_BUILD"] if bench else []), "-c", s, "-o", obj]
     r = subprocess.run(cmd, capture_output=True, text=True)
     err = "\n".join(l for l in r.stderr.splitlines() if "packed-fp32-ops" not in l)
     if r.returncode != 0:
@@ -72,19 +78,27 @@ def _compile(src: str, force: bool, dep_m: float) -> str:
     return obj
 
 
-def build(force: bool = False, jobs: int = 6) -> str:
-    os.makedirs(OBJ_DIR, exist_ok=True)
-    os.makedirs(LIB_DIR, exist_ok=True)
-    dep_m = _deps_mtime()
-    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
-        objs = list(ex.map(lambda s: _compile(s, force, dep_m), SOURCES))
-    if force or not os.path.exists(LIB_PATH) or any(os.path.getmtime(o) > os.path.getmtime(LIB_PATH) for o in objs):
-        cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", LIB_PATH]
+def _link(objs, path: str, force: bool) -> None:
+    if force or not os.path.exists(path) or any(os.path.getmtime(o) > os.path.getmtime(path) for o in objs):
+        cmd = [_hipcc(), "--offload-arch=gfx950", "-shared", "-fPIC", "-fno-gpu-rdc", *objs, "-o", path]
         r = subprocess.run(cmd, capture_output=True, text=True)
         if r.returncode != 0:
             raise RuntimeError("link failed:\n" + r.stderr)
+
+
+def build(force: bool = False, jobs: int = 8, bench: bool = True) -> str:
+    """Compiles the product library and (bench=True) the benchmark variant."""
+    os.makedirs(OBJ_DIR, exist_ok=True)
+    os.makedirs(LIB_DIR, exist_ok=True)
+    dep_m = _deps_mtime()
+    units = [(s, False) for s in SOURCES] + ([(s, True) for s in SOURCES] if bench else [])
+    with concurrent.futures.ThreadPoolExecutor(max_workers=jobs) as ex:
+        objs = list(ex.map(lambda u: _compile(u[0], force, dep_m, u[1]), units))
+    _link(objs[:len(SOURCES)], LIB_PATH, force)
+    if bench:
+        _link(objs[len(SOURCES):], BENCH_LIB_PATH, force)
     return LIB_PATH
 
 
 if __name__ == "__main__":
-    print(build(force="--force" in sys.argv))
+    print(build(force="--force" in sys.argv, bench="--product-only" not in sys.argv))

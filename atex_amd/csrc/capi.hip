@@ -99,9 +99,10 @@ const char* atexn_status_string(int status) {
 const char* atexn_last_error(void) { return last_error(); }
 int atexn_abi_version(void) { return kAbiVersion; }
 
-/* Benchmark / tuning hook, not part of the drop-in contract: sets a launch-planning
- * parameter by name for the whole process.  Returns ATEXN_INVALID_ARGUMENT for an unknown
- * name or a value out of range. */
+/* Debugging / benchmarking hook (declared in the header): sets a launch-planning parameter by
+ * name for the whole process.  Returns ATEXN_INVALID_ARGUMENT for an unknown name or a value
+ * out of range.  Every setting computes complete, correct results; the one switch that does
+ * not (running only part of a backward call) exists in the benchmark build alone. */
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused"),
@@ -120,9 +121,11 @@ int atexn_set_tuning(const char* name, int value) {
     ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),
                   "rows batch must be 1, 2 (or 4, forward only)");
     (name[0] == 'f' ? t.fwd_rows_batch : t.bwd_rows_batch) = value;
+#ifdef ATEXN_BENCH_BUILD
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
     t.bwd_stage_mask = value;
+#endif
   } else if (!strcmp(name, "bwd_wave_groups")) {
     ATEXN_REQUIRE(value == 1 || value == 2, "bwd_wave_groups must be 1 (on) or 2 (off)");
     t.bwd_wave_groups = value == 1;

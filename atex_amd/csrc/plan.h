@@ -12,36 +12,52 @@
 #include <stdint.h>
 
 #include <algorithm>
+#include <atomic>
 #include <climits>
 
 namespace atexn {
 
-// Tunables (process-wide; defaults chosen by measurement on MI355X).
+// Launch-planning parameters (process-wide; defaults chosen by measurement on MI355X).  They are
+// only ever changed through atexn_set_tuning, a debugging / benchmarking hook; each is an atomic
+// so that a change made while other threads plan launches is a clean switch, not a data race.
+// (A workspace query and the call it sizes must still see the same values.)
+using TuneInt = std::atomic<int>;
 struct Tuning {
-  int fwd_waves_per_cu = 16;      // resident forward: waves kept resident per CU
-  int bwd_ln_threads = 512;       // resident LayerNorm backward, rows <= one wave: block size
-  int bwd_waves_per_cu = 8;       // resident LayerNorm backward: waves kept resident per CU
-                                  //   (each block adds a partial row to the column reduction)
-  int bwd_affine_waves_per_cu = 32;  // resident channel-first backward (no partial rows)
-  int split_items_per_cu = 2;     // split rows: (row, chunk) work items per CU
-  int cl_items_per_cu = 2;        // channels-last: (n, slab, tile) work items per CU
-  int tile_items_per_cu = 4;      // LayerNorm long rows: (row slab, column tile) tiles per CU
-  int fwd_rows_batch = 4;         // resident kernels, rows <= one wave: rows per batch of a
-  int bwd_rows_batch = 1;         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
-  // Benchmark hook: which stages of a backward call run (bit 0: the row / slab kernels,
-  // bit 1: the final column reduction).  Anything but 3 gives incomplete results.
-  int bwd_stage_mask = 3;
+  TuneInt fwd_waves_per_cu{16};      // resident forward: waves kept resident per CU
+  TuneInt bwd_ln_threads{512};       // resident LayerNorm backward, rows <= one wave: block size
+  TuneInt bwd_waves_per_cu{8};       // resident LayerNorm backward: waves kept resident per CU
+                                     //   (each block adds a partial row to the column reduction)
+  TuneInt bwd_affine_waves_per_cu{32};  // resident channel-first backward (no partial rows)
+  TuneInt split_items_per_cu{2};     // split rows: (row, chunk) work items per CU
+  TuneInt cl_items_per_cu{2};        // channels-last: (n, slab, tile) work items per CU
+  TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
+  TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
+  TuneInt bwd_rows_batch{1};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
-  int reverse_second_pass = 1;
+  TuneInt reverse_second_pass{1};
+  TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
+  TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
-  int cl_fused = 1;        // channels-last: single-pass kernels when an instance fits a workgroup
-  int bwd_wave_groups = 1;  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
-  int fwd_vpt2_max_vec = 1024;
-  int bwd_vpt2_max_vec = 1536;
+  TuneInt fwd_vpt2_max_vec{1024};
+  TuneInt bwd_vpt2_max_vec{1536};
+#ifdef ATEXN_BENCH_BUILD
+  // Only in the benchmark build of the library (libatex_norms_hip_bench.so): which stages of a
+  // backward call over resident rows run (bit 0: the row kernel, bit 1: the column reduction),
+  // so that the row kernel can be timed alone.  Anything but 3 gives incomplete results, which
+  // is why the product library has no such switch.
+  TuneInt bwd_stage_mask{3};
+#endif
 };
 Tuning& tuning();
+inline int bwd_stage_mask() {
+#ifdef ATEXN_BENCH_BUILD
+  return tuning().bwd_stage_mask;
+#else
+  return 3;
+#endif
+}
 
 enum class RowsKind { kFwd, kBwdCols /*LayerNorm: per-column dgamma/dbeta*/, kBwdAffine };
 
@@ -173,7 +189,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       }
       if (kind == RowsKind::kBwdCols) {
         // bigger blocks -> fewer partial rows for the column reduction
-        int th = std::min(t.bwd_ln_threads, 512);
+        int th = std::min<int>(t.bwd_ln_threads, 512);
         while (th > 256 && div_up(n_rows, int64_t(th / p.tpr) * p.rb) < cus) th /= 2;
         p.threads = th;
       }

@@ -169,7 +169,7 @@ int small_bwd_launch(const T* dy, const T* x, const float* gamma, const float* m
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* part = static_cast<float*>(ws);
   const int Di = static_cast<int>(D);
-  if (tuning().bwd_stage_mask & 1) {
+  if (bwd_stage_mask() & 1) {
     switch (p.NV) {
       case 1: small_bwd<T, V, 1, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
       case 2: small_bwd<T, V, 2, AFF><<<p.grid, kSmallThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di, C); break;
@@ -178,7 +178,7 @@ int small_bwd_launch(const T* dy, const T* x, const float* gamma, const float* m
     }
     ATEXN_CHECK_LAUNCH("small_bwd");
   }
-  if (!(tuning().bwd_stage_mask & 2)) return ATEXN_OK;
+  if (!(bwd_stage_mask() & 2)) return ATEXN_OK;
   return launch_col_reduce(part, dgamma, dbeta, p.part_rows, AFF ? C : D, st);
 }
 
@@ -250,7 +250,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   if (p.resident) {
     auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact, p.ragged);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
-    const int stages = tuning().bwd_stage_mask;
+    const int stages = bwd_stage_mask();
     if (stages & 1) {
       fn<<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
                                                 static_cast<int>(D), C);

@@ -67,7 +67,7 @@ SIGNATURES = {
     "atexn_fused_instance_norm": (_i, [_tp, _tp, _tp, _f, ctypes.c_char_p, _tp, _tp, _tp, _vp, _sz, _vp]),
     "atexn_fused_instance_norm_grad_workspace_bytes": (_sz, [_tp, ctypes.c_char_p]),
     "atexn_fused_instance_norm_grad": (_i, [_tp, _tp, _tp, _tp, _tp, ctypes.c_char_p, _tp, _tp, _tp, _vp, _sz, _vp]),
-    # tuning hook (benchmarks only; not in the public header)
+    # debugging / benchmarking hook
     "atexn_set_tuning": (_i, [ctypes.c_char_p, _i]),
 }
 

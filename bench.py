@@ -15,7 +15,11 @@ Output: ONE JSON line on stdout.
   value        algorithmic bytes of fwd + bwd / wall time per step, in GB/s
   roofline     the dominant kernel (the backward row kernel), timed alone with events on the
                launch stream: algorithmic bytes of the backward / its average duration,
-               against the 8 TB/s HBM peak
+               against the 8 TB/s HBM peak.  "Alone" needs the benchmark build of the library
+               (libatex_norms_hip_bench.so, same sources plus a switch that skips the column
+               reduction); every other figure comes from the product library
+  targets      (default case only) the second target shape, InstanceNorm x fp16 [8,128,128,64]
+               in both layouts: us per call, GB/s, fraction of peak, roofline of its backward
   cpu_baseline the C oracle's float flavour (OpenMP over rows) on the same workload, timed
                on this machine's host cores; `unfused_composite` inside it is the unfused op
                sequence a framework would run instead (torch on the CPU, autograd backward)
@@ -77,6 +81,8 @@ CASES = {
     "inref_4x256x32_cf": ("in", "f16", (4, 256, 32 ** 3, True)),
 }
 DEFAULT_CASE = "ln_bert"
+# the two shapes the throughput target is stated on, reported on the default run's line
+TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
 
 # Bytes between L2 and memory per launch of the kernel(s) the roofline object is quoted on,
 # from `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this file, each scaled by
@@ -126,6 +132,29 @@ def make_host_inputs(op, dtype, dims, seed):
     gamma = rng.uniform(0.5, 1.5, size=P).astype(np.float32)
     beta = (rng.standard_normal(P) * 0.1).astype(np.float32)
     return x, gamma, beta, dy
+
+
+_BENCH_LIB = None
+
+
+def bench_lib():
+    """The benchmark build of the library (adds the "bwd_stage_mask" switch), or None."""
+    global _BENCH_LIB
+    if _BENCH_LIB is None:
+        import ctypes
+
+        from atex_amd.nv_norms import _capi
+
+        path = _capi.LIB_PATH.replace(".so", "_bench.so")
+        if not os.path.exists(path):
+            return None
+        L = ctypes.CDLL(path)
+        for name, (res, args) in _capi.SIGNATURES.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _BENCH_LIB = L
+    return _BENCH_LIB
 
 
 class GpuCase:
@@ -313,12 +342,26 @@ def composite_cpu(op, dtype, d, x, gamma, beta, dy, threads, max_seconds=8.0):
             "note": "torch CPU, unfused op sequence with autograd; composite restatement, not tf.keras"}
 
 
-def roofline_kernel(op, dims):
+def resident_rows_bwd(op, dtype, dims):
+    """Whether the backward of the case runs the register-resident row kernel followed by the
+    column reduction (rows of at most 2048 vectors for LayerNorm, planes of at most 4096 for
+    channel-first InstanceNorm; a vector is 16 bytes)."""
+    vec = 16 // ESIZE[dtype]
+    if op == "ln":
+        return dims[1] <= 2048 * vec
+    return bool(dims[3]) and dims[2] <= 4096 * vec
+
+
+def roofline_kernel(op, dtype, dims, alone):
     if op == "in" and not dims[3]:
         return "cl_bwd_sums + cl_bwd_apply (channels-last backward, the whole call)"
-    if op == "in" and dims[2] > 16384:
-        return "split_bwd_sums + split_bwd_apply (backward of rows too long for registers)"
-    return "rows_bwd_resident (backward row kernel: dx and the dgamma / dbeta partials)"
+    if op == "in" and not resident_rows_bwd(op, dtype, dims):
+        return "split_bwd_sums + split_bwd_apply + col_reduce (backward of planes too long for registers, the whole call)"
+    if op == "ln" and not resident_rows_bwd(op, dtype, dims):
+        return "tile_bwd_sums + merge_row_sums + tile_bwd_apply (backward of rows too long for registers, the whole call)"
+    if alone:
+        return "rows_bwd_resident (backward row kernel: dx and the dgamma / dbeta partials), timed without col_reduce"
+    return "rows_bwd_resident + col_reduce (the whole backward call)"
 
 
 def torch_mod():
@@ -327,11 +370,33 @@ def torch_mod():
     return torch
 
 
-def run_case(name, steps, warmup, with_cpu=True):
+def time_row_kernel_alone(case, steps, warmup):
+    """Average ms of the backward call without its final column reduction (the dominant kernel
+    alone), through the benchmark build of the library; None if that build is missing or the
+    case's backward has no separate column reduction to switch off."""
+    if not resident_rows_bwd(case.op, case.dtype, case.dims):
+        return None
+    LB = bench_lib()
+    if LB is None:
+        return None
+    product = case.L
+    case.L = LB
+    try:
+        if LB.atexn_set_tuning(b"bwd_stage_mask", 1) != 0:
+            return None
+        try:
+            return case.time_loop(case.bwd, steps, warmup)
+        finally:
+            LB.atexn_set_tuning(b"bwd_stage_mask", 3)
+    finally:
+        case.L = product
+
+
+def measure(name, steps, warmup, extras=True):
+    """Times one case; returns (result dict, GpuCase)."""
     op, dtype, dims = CASES[name]
     fb, bb = algorithmic_bytes(op, dtype, dims)
     case = GpuCase(op, dtype, dims)
-    L = case.L
 
     def step(i):
         case.fwd(i)
@@ -340,15 +405,38 @@ def run_case(name, steps, warmup, with_cpu=True):
     ms_step = case.time_loop(step, steps, warmup)
     ms_fwd = case.time_loop(case.fwd, steps, warmup)
     ms_bwd = case.time_loop(case.bwd, steps, warmup)
-    # the dominant kernel alone: backward without its final column reduction
-    L.atexn_set_tuning(b"bwd_stage_mask", 1)
-    ms_bwd_main = case.time_loop(case.bwd, steps, warmup)
-    L.atexn_set_tuning(b"bwd_stage_mask", 3)
+    ms_alone = time_row_kernel_alone(case, steps, warmup)
+    ms_roof = ms_alone if ms_alone is not None else ms_bwd
+    achieved = bb / (ms_roof * 1e-3) / 1e9
+    value = (fb + bb) / (ms_step * 1e-3) / 1e9
+    if op == "ln":
+        workload = f"LayerNorm fwd+bwd x {dtype} [{dims[0]},{dims[1]}] axis=-1 eps=1e-3, gamma/beta fp32"
+    else:
+        N, C, D, cf = dims
+        workload = (f"InstanceNorm fwd+bwd x {dtype} N={N} C={C} spatial={D} "
+                    f"{'channel-first' if cf else 'channels-last'} eps=1e-3")
+    res = {
+        "workload": workload, "case": name, "rotating_buffer_sets": case.n_sets,
+        "algorithmic_bytes_fwd": fb, "algorithmic_bytes_bwd": bb,
+        "value": value, "ms_per_step": ms_step,
+        "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
+        "us_per_call": {"fwd": ms_fwd * 1e3, "bwd": ms_bwd * 1e3, "fwd_bwd": ms_step * 1e3},
+        "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9},
+        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
+                     "kernel": roofline_kernel(op, dtype, dims, ms_alone is not None),
+                     "us": ms_roof * 1e3},
+    }
+    if not extras:
+        return res, case
+
     # hot-cache figure (one buffer set reused), labelled as such
     n_sets = case.n_sets
     case.n_sets = 1
     ms_step_hot = case.time_loop(step, steps, warmup)
     case.n_sets = n_sets
+    res["us_per_call"]["fwd_bwd_hot_cache"] = ms_step_hot * 1e3
+    res["gbps"]["fwd_bwd_hot_cache"] = (fb + bb) / (ms_step_hot * 1e-3) / 1e9
 
     # the same fwd + bwd steps captured once into a HIP graph (one pass over all buffer sets)
     # and replayed: what a caller that captures its step gets
@@ -371,6 +459,7 @@ def run_case(name, steps, warmup, with_cpu=True):
         ms_step_graph = case.time_loop(lambda i: graph.replay(), reps, 2) / case.n_sets
     except Exception as e:  # graph capture is an extra, never fatal
         print(f"hip graph timing skipped: {e}", file=sys.stderr)
+    res["us_per_call"]["fwd_bwd_hip_graph"] = None if ms_step_graph is None else ms_step_graph * 1e3
 
     # what plain streaming kernels reach on the same tensors and rotation (torch's elementwise
     # kernels): a copy (1 read + 1 write, the forward's traffic) and an add (2 reads + 1 write,
@@ -381,44 +470,54 @@ def run_case(name, steps, warmup, with_cpu=True):
     torch = case.torch
     ms_add = case.time_loop(lambda i: torch.add(case.sets[i % case.n_sets]["x"], case.sets[i % case.n_sets]["dy"],
                                                 out=case.sets[i % case.n_sets]["dx"]), steps, warmup)
+    res["streaming_reference"] = {
+        "copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
+        "add_us": ms_add * 1e3, "add_gbps": 3 * tensor_bytes / (ms_add * 1e-3) / 1e9,
+        "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"}
+    return res, case
 
-    value = (fb + bb) / (ms_step * 1e-3) / 1e9
-    achieved = bb / (ms_bwd_main * 1e-3) / 1e9
-    if op == "ln":
-        workload = f"LayerNorm fwd+bwd x {dtype} [{dims[0]},{dims[1]}] axis=-1 eps=1e-3, gamma/beta fp32"
-    else:
-        N, C, D, cf = dims
-        workload = (f"InstanceNorm fwd+bwd x {dtype} N={N} C={C} spatial={D} "
-                    f"{'channel-first' if cf else 'channels-last'} eps=1e-3")
+
+def run_case(name, steps, warmup, with_cpu=True, with_targets=False):
+    op, dtype, dims = CASES[name]
+    m, case = measure(name, steps, warmup)
     out = {
         "metric": "LN/IN fwd+bwd achieved HBM GB/s",
-        "value": value,
+        "value": m["value"],
         "unit": "GB/s",
         "n_gpus": 1,
         "steps": steps,
         "warmup": warmup,
-        "ms_per_step": ms_step,
+        "ms_per_step": m["ms_per_step"],
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": dtype,
         "data": "synthetic",
-        "config": {"workload": workload, "case": name, "rotating_buffer_sets": n_sets,
-                   "algorithmic_bytes_fwd": fb, "algorithmic_bytes_bwd": bb},
-        "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBPS,
-        "us_per_call": {"fwd": ms_fwd * 1e3, "bwd": ms_bwd * 1e3, "fwd_bwd": ms_step * 1e3,
-                        "fwd_bwd_hot_cache": ms_step_hot * 1e3,
-                        "fwd_bwd_hip_graph": None if ms_step_graph is None else ms_step_graph * 1e3},
-        "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9,
-                 "fwd_bwd_hot_cache": (fb + bb) / (ms_step_hot * 1e-3) / 1e9},
-        "streaming_reference": {"copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
-                                "add_us": ms_add * 1e3, "add_gbps": 3 * tensor_bytes / (ms_add * 1e-3) / 1e9,
-                                "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"},
-        "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
-                     "kernel": roofline_kernel(op, dims),
-                     "us": ms_bwd_main * 1e3},
+        "config": {"workload": m["workload"], "case": name, "rotating_buffer_sets": m["rotating_buffer_sets"],
+                   "algorithmic_bytes_fwd": m["algorithmic_bytes_fwd"],
+                   "algorithmic_bytes_bwd": m["algorithmic_bytes_bwd"]},
+        "pct_of_hbm_peak": m["pct_of_hbm_peak"],
+        "us_per_call": m["us_per_call"],
+        "gbps": m["gbps"],
+        "streaming_reference": m["streaming_reference"],
+        "roofline": m["roofline"],
     }
+    del case
+    if with_targets:
+        # the second target shape, on the same driver-run line
+        out["targets"] = {}
+        for tname in TARGET_CASES:
+            if tname == name:
+                continue
+            t, tcase = measure(tname, steps, warmup, extras=False)
+            del tcase
+            torch_mod().cuda.empty_cache()
+            out["targets"][tname] = {
+                "workload": t["workload"], "dtype": CASES[tname][1],
+                "us_per_call": t["us_per_call"], "gbps": t["gbps"],
+                "value": t["value"], "pct_of_hbm_peak": t["pct_of_hbm_peak"],
+                "roofline": t["roofline"],
+            }
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline(op, dtype, dims)
     return out
@@ -431,6 +530,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--case", default=DEFAULT_CASE, choices=sorted(CASES) + ["all"])
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-targets", action="store_true",
+                    help="default case only: skip the InstanceNorm target shapes")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
                          "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
@@ -451,7 +552,8 @@ def main():
             r = run_case(name, steps, args.warmup, with_cpu=False)
             print(json.dumps(r), flush=True)
         return
-    print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu)), flush=True)
+    print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu,
+                              with_targets=args.case == DEFAULT_CASE and not args.no_targets)), flush=True)
     if args.copy_calibration:
         src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
         dst = torch.empty_like(src)

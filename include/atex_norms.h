@@ -32,7 +32,9 @@
  *     ATEXN_LAUNCH_ERROR (a HIP call failed); atexn_last_error() gives the detail of the
  *     calling thread's last failure.  Nothing aborts or throws across this boundary
  *     (the reference aborts on a launch failure, norm_util.h:77);
- *   - empty inputs (N * D == 0 or N * C * D == 0) succeed without reading anything; the
+ *   - empty inputs (N * D == 0 or N * C * D == 0) succeed without reading or writing anything
+ *     (mean / inv_std stay unwritten even when N > 0, as in the reference, whose functors
+ *     return at once on an empty x, fused_layer_norm_op.cu:811-813); the
  *     backward entry points then zero-fill dgamma / dbeta, as the reference's CPU functor
  *     does (fused_layer_norm_op.cc:96-103) -- its GPU functor leaves them unwritten
  *     (fused_layer_norm_op.cu:904-906).
@@ -64,6 +66,16 @@ const char* atexn_status_string(int status);
 const char* atexn_last_error(void);
 /* ABI version of this header: bumps when a signature changes. */
 int atexn_abi_version(void);
+
+/* Debugging / benchmarking hook, not needed by a drop-in user: sets one launch-planning
+ * parameter (resident waves per CU, rows per batch, work items per CU of the two-stage kernels,
+ * single-pass channels-last on / off, ...) for the whole process; the names are listed in
+ * csrc/plan.h (struct Tuning).  Every value it accepts still gives complete and correct results,
+ * only a different launch plan.  The parameters are the one piece of process-wide HOST state of
+ * the library: a *_workspace_bytes query and the call it sizes must run under the same
+ * settings, so change them only while no other thread is between the two.  Returns
+ * ATEXN_INVALID_ARGUMENT for an unknown name or a value out of range. */
+int atexn_set_tuning(const char* name, int value);
 
 /* ------------------------------------------------------------------ kernel level */
 

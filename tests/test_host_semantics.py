@@ -6,6 +6,7 @@ the axis cases of tests/fused_layer_norm_test.py:250-260."""
 import ctypes
 import os
 import re
+import subprocess
 
 import pytest
 
@@ -44,6 +45,12 @@ def test_every_declared_symbol_is_exported(L):
     for n in names:
         assert hasattr(L, n), f"{n} is declared in atex_norms.h but not exported"
     assert set(names) <= set(_capi.SIGNATURES), set(names) - set(_capi.SIGNATURES)
+    # and nothing beyond the header: every exported atexn_* symbol of the product library (and
+    # of its benchmark variant) is declared
+    for path in (_capi.LIB_PATH, _capi.LIB_PATH.replace(".so", "_bench.so")):
+        out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
+        exported = {line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("atexn_")}
+        assert exported == set(names), (path, exported ^ set(names))
     assert L.atexn_abi_version() == 1
     assert L.atexn_status_string(0) == b"OK"
     assert L.atexn_status_string(1) == b"INVALID_ARGUMENT"
@@ -216,6 +223,14 @@ def test_kernel_level_validation(L):
                                   0x4000, need - 256, None) == 1
     assert b"workspace too small" in L.atexn_last_error()
     assert L.atexn_set_tuning(b"no_such_parameter", 1) == 1
+    # running only part of a backward call is not something the product library can be told
+    assert L.atexn_set_tuning(b"bwd_stage_mask", 1) == 1
+    assert b"unknown tuning parameter" in L.atexn_last_error()
+    # the static-scratch backward refuses what does not fit its buffer before it touches a device
+    assert L.atexn_layer_norm_bwd_workspace_bytes(1, 2048, 12288) > (8 << 20)
+    assert L.atexn_layer_norm_bwd_static(1, FAKE, 0x2000, FAKE, FAKE, FAKE, 2048, 12288, 0x3000, FAKE,
+                                         FAKE, None) == 1
+    assert b"static buffer" in L.atexn_last_error()
 
 
 def test_workspace_queries_without_gpu(L):
