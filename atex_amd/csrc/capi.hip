@@ -105,7 +105,8 @@ int atexn_abi_version(void) { return kAbiVersion; }
  * not (running only part of a backward call) exists in the benchmark build alone. */
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
-  ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused"),
+  ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
+                    !strcmp(name, "cl_coop"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -138,6 +139,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "cl_fused")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_fused must be 0 or 1");
     t.cl_fused = value;
+  } else if (!strcmp(name, "cl_coop")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "cl_coop must be 0 or 1");
+    t.cl_coop = value;
   } else if (!strcmp(name, "reverse_second_pass")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "reverse_second_pass must be 0 or 1");
     t.reverse_second_pass = value;

@@ -16,6 +16,8 @@
 // and their use.
 #pragma once
 
+#include <hip/hip_cooperative_groups.h>
+
 #include "norm_common.cuh"
 
 namespace atexn {
@@ -181,6 +183,259 @@ __device__ __forceinline__ float cl_slab_count(int s, int64_t D, int64_t slab_le
   return static_cast<float>(beg + slab_len <= D ? slab_len : D - beg);
 }
 
+// ------------------------------------------------------- building blocks of the stages
+// Statistics of a register-resident slab: an exact two-pass over the registers (block-wide
+// sum -> slab mean, block-wide sum of squared deviations from it).  lds: V * 256 floats.
+template <typename T, int V, int U>
+__device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], const bool (&ok)[U],
+                                                  float inv_n, int TPP, float* lds,
+                                                  float (&mean)[V], float (&m2)[V]) {
+#pragma unroll
+  for (int i = 0; i < V; ++i) mean[i] = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) mean[i] += ok[u] ? to_f32(raw[u].v[i]) : 0.f;
+  }
+  cl_block_sum<V>(mean, lds, TPP);
+#pragma unroll
+  for (int i = 0; i < V; ++i) {
+    mean[i] *= inv_n;
+    m2[i] = 0.f;
+  }
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
+      m2[i] += d * d;
+    }
+  }
+  __syncthreads();  // the first sum's LDS reads are done
+  cl_block_sum<V>(m2, lds, TPP);
+}
+
+// Chan-merge of the S slab statistics pstat[(n * S + s)][2][C] of every channel of the
+// block's tile into sm_mean / sm_rstd (and, from the block of slab 0, into the op's outputs).
+// Each of the fm.P lanes of a channel takes every P-th slab in order, then the lanes merge
+// pairwise; the merge is bitwise symmetric, so every workgroup of the instance gets the same
+// bits.  The counts follow from cnt_len (the slab length; after cl_merge_stats S == 1 and
+// cnt_len == D).  The caller synchronises the block before it reads sm_mean / sm_rstd.
+__device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& g, int S,
+                                              int64_t cnt_len, int64_t D, int C, int cap,
+                                              float eps, float* sm_mean, float* sm_rstd,
+                                              float* __restrict__ mean_out,
+                                              float* __restrict__ rstd_out) {
+  const FoldMap fm = fold_map(cap);
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const int c_base = g.ct * cap;
+  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
+    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
+    const int sub = static_cast<int>(threadIdx.x) % fm.P;
+    const int c = c_base + cl;
+    const bool in = cl < cap && c < C;
+    Wf w{0.f, 0.f, 0.f};
+    if (in) {
+      const float* q = pstat + ((g.n * S) * 2) * C + c;
+      constexpr int B = 8;
+      batched_for<B>(
+          sub, S, fm.P,
+          [&](int64_t sl, int64_t step) {
+            float tm[B], tq[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+              tm[u] = q[((sl + u * step) * 2) * C];
+              tq[u] = q[((sl + u * step) * 2 + 1) * C];
+            }
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+              w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, cnt_len)});
+            }
+          },
+          [&](int64_t sl) {
+            w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
+                               cl_slab_count(static_cast<int>(sl), D, cnt_len)});
+          });
+    }
+    for (int m = 1; m < fm.P; m <<= 1) {
+      Wf o;
+      o.mean = lane_xor(w.mean, m);
+      o.m2 = lane_xor(w.m2, m);
+      o.n = lane_xor(w.n, m);
+      w = wf_merge(w, o);
+    }
+    if (sub == 0 && in) {
+      const float rs = rsqrtf(w.m2 * inv_d + eps);
+      sm_mean[cl] = w.mean;
+      sm_rstd[cl] = rs;
+      if (g.s == 0) {
+        mean_out[g.n * C + c] = w.mean;
+        rstd_out[g.n * C + c] = rs;
+      }
+    }
+  }
+}
+
+// Per-thread constants of the forward apply: mean and gamma * rstd of the thread's channels.
+template <int V, bool RG>
+struct ClFwdCoef {
+  float mean[V], sc[V], bt[V];
+  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, const float* gamma,
+                                       const float* beta, const float* sm_mean,
+                                       const float* sm_rstd) {
+    // channel of element i inside the tile; elements the thread does not own may fall before
+    // the tile (their results are never stored)
+    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
+    load_f32<V>(gamma + g.coff, sc);
+    load_f32<V>(beta + g.coff, bt);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      mean[i] = sm_mean[RG && cl0 + i < 0 ? 0 : cl0 + i];
+      sc[i] *= sm_rstd[RG && cl0 + i < 0 ? 0 : cl0 + i];
+    }
+  }
+  template <typename T>
+  __device__ __forceinline__ Pack<T, V> apply(const Pack<T, V>& pk) const {
+    Pack<T, V> o;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      // subtract the mean first: x * scale - mean * scale would cancel badly when |mean| >> std
+      o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * sc[i] + bt[i]);
+    }
+    return o;
+  }
+};
+
+// Sums of a register-resident slab for the backward: acc[i] = sum dy * xh, acc[V + i] = sum dy
+// over the block's pixels, per channel of the thread.  lds: 2 * V * 256 floats.
+template <typename T, int V, int U>
+__device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], const Pack<T, V> (&rd)[U],
+                                                 const bool (&ok)[U], const float (&mu)[V],
+                                                 const float (&rs)[V], int TPP, float* lds,
+                                                 float (&acc)[2 * V]) {
+#pragma unroll
+  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float d = ok[u] ? to_f32(rd[u].v[i]) : 0.f;
+      const float xh = ok[u] ? (to_f32(rx[u].v[i]) - mu[i]) * rs[i] : 0.f;
+      acc[i] += d * xh;
+      acc[V + i] += d;
+    }
+  }
+  cl_block_sum<2 * V>(acc, lds, TPP);
+}
+
+// Backward counterpart of cl_fold_stats: adds up the S slab partials part[(n * S + s)][2][C]
+// of the block's instance and channel tile into sm_b (sum dy * xh) and sm_a (sum dy), and
+// produces the block's share of dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C])
+// is the sum of one column of all N * S partial rows (fixed order, no atomics); block w of the
+// grid takes outputs w, w + #blocks, ...  Ends with a block-wide barrier.
+__device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g, int64_t N, int S,
+                                             int C, int cap, float* sm_a, float* sm_b,
+                                             float (*red_buf)[16], float* __restrict__ dgamma,
+                                             float* __restrict__ dbeta) {
+  const FoldMap fm = fold_map(cap);
+  const int c_base = g.ct * cap;
+  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
+    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;
+    const int sub = static_cast<int>(threadIdx.x) % fm.P;
+    const int c = c_base + cl;
+    const bool in = cl < cap && c < C;
+    float a = 0.f, b = 0.f;
+    if (in) {
+      const float* pr = part + ((g.n * S) * 2) * C + c;
+      constexpr int B = 16;
+      batched_for<B>(
+          sub, S, fm.P,
+          [&](int64_t sl, int64_t step) {
+            float tb[B], ta[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+              tb[u] = pr[((sl + u * step) * 2) * C];
+              ta[u] = pr[((sl + u * step) * 2 + 1) * C];
+            }
+#pragma unroll
+            for (int u = 0; u < B; ++u) {
+              b += tb[u];
+              a += ta[u];
+            }
+          },
+          [&](int64_t sl) {
+            b += pr[(sl * 2) * C];
+            a += pr[(sl * 2 + 1) * C];
+          });
+    }
+    for (int m = 1; m < fm.P; m <<= 1) {
+      a += lane_xor(a, m);
+      b += lane_xor(b, m);
+    }
+    if (sub == 0 && in) {
+      sm_a[cl] = a;
+      sm_b[cl] = b;
+    }
+  }
+  const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
+  const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  int red_it = 0;
+  for (int64_t o = w; o < 2 * static_cast<int64_t>(C); o += n_blocks) {
+    const int which = o < C ? 0 : 1;
+    const int c = static_cast<int>(o < C ? o : o - C);
+    const int64_t rows = N * S;
+    float t = 0.f;
+    const float* pc = part + static_cast<int64_t>(which) * C + c;
+    batched_for<4>(
+        threadIdx.x, rows, kClThreads,
+        [&](int64_t r, int64_t step) {
+          float v[4];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) v[u] = pc[((r + u * step) * 2) * C];
+#pragma unroll
+          for (int u = 0; u < 4; ++u) t += v[u];
+        },
+        [&](int64_t r) { t += pc[(r * 2) * C]; });
+    t = block_sum1(t, red_buf[red_it & 1]);
+    ++red_it;
+    if (threadIdx.x == 0) (which == 0 ? dgamma : dbeta)[c] = t;
+  }
+  __syncthreads();
+}
+
+// Per-thread constants of the backward apply:
+// dx = r * gamma * (dy - (A + xh * B) / D) with A = sum dy, B = sum dy * xh over the whole
+// (n, c) instance (norm_util.h:599-615 in s1 / s2 form) = sc * dy + (ca * xh + cb).
+template <int V, bool RG>
+struct ClBwdCoef {
+  float mu[V], rs[V], sc[V], ca[V], cb[V];
+  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, int C, float inv_d,
+                                       const float* gamma, const float* mean_in,
+                                       const float* rstd_in, const float* sm_a,
+                                       const float* sm_b) {
+    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
+    load_f32<V>(mean_in + g.n * C + g.coff, mu);
+    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
+    load_f32<V>(gamma + g.coff, sc);
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      sc[i] *= rs[i];
+      ca[i] = -sc[i] * (sm_b[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
+      cb[i] = -sc[i] * (sm_a[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
+    }
+  }
+  template <typename T>
+  __device__ __forceinline__ Pack<T, V> apply(const Pack<T, V>& px, const Pack<T, V>& pd) const {
+    Pack<T, V> o;
+#pragma unroll
+    for (int i = 0; i < V; ++i) {
+      const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
+      o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * xh + cb[i]));
+    }
+    return o;
+  }
+};
+
 // ---------------------------------------------------------------- forward, stage 1
 // pstat: [N * S][2][C], the (mean, m2 = sum of squared deviations from that mean) of every
 // channel over each slab; the slab's pixel count follows from the geometry.  Nothing is
@@ -188,8 +443,7 @@ __device__ __forceinline__ float cl_slab_count(int s, int64_t D, int64_t slab_le
 // the data look like (an instance whose border pixels are far from the bulk, a large common
 // offset): the counterpart of the reference's Welford pushes (norm_util.h:182-211).
 // U > 0: the slab is register-resident (slab_len <= U * pixel slots per block), all its
-// loads are in flight at once and the statistics are an exact two-pass over the registers
-// (block-wide sum -> slab mean, block-wide sum of squared deviations from it).
+// loads are in flight at once and the statistics are an exact two-pass over the registers.
 // U == 0 streams the slab in batches of 8 pixels per thread: per-thread running (mean, m2)
 // by batch-wise Chan updates (wf_lanes_push), combined over the block around the slab mean
 // (m2 = sum over threads of m2_t + n_t (mean_t - mean)^2, every term non-negative).
@@ -208,27 +462,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
     Pack<T, V> raw[U];
     bool ok[U];
     cl_load_slab<T, V, U>(xn, g, CV, C, raw, ok);
-#pragma unroll
-    for (int i = 0; i < V; ++i) mean[i] = 0.f;
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int i = 0; i < V; ++i) mean[i] += ok[u] ? to_f32(raw[u].v[i]) : 0.f;
-    }
-    cl_block_sum<V>(mean, lds, TPP);
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      mean[i] *= inv_n;
-      m2[i] = 0.f;
-    }
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
-        m2[i] += d * d;
-      }
-    }
+    cl_resident_stats<T, V, U>(raw, ok, inv_n, TPP, lds, mean, m2);
   } else {
     WfLanes<V> run;
     wf_lanes_init<V>(run);
@@ -266,9 +500,9 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
       const float d = run.mean[i] - mean[i];
       m2[i] = run.m2[i] + run.n * (d * d);
     }
+    __syncthreads();  // the first sum's LDS reads are done
+    cl_block_sum<V>(m2, lds, TPP);
   }
-  __syncthreads();  // the first sum's LDS reads are done
-  cl_block_sum<V>(m2, lds, TPP);
   if (g.ch_ok && g.slot == 0) {
     const int64_t o = ((g.n * S + g.s) * 2) * C + g.coff;
     store_f32_from<V>(pstat + o, mean, RG ? g.lo : 0);
@@ -326,8 +560,6 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
 // ---------------------------------------------------------------- forward, stage 2
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
-// pstat holds S partial (mean, m2) rows per instance whose counts follow from cnt_len (the
-// slab length; after cl_merge_stats: S == 1 and cnt_len == D).
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restrict__ gamma,
@@ -337,88 +569,20 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
   __shared__ float sm_mean[kClMaxTileChannels];
   __shared__ float sm_rstd[kClMaxTileChannels];
   const int CV = (C + V - 1) / V;
-  const int TPP = 1 << tpp_shift;
-  const int cap = TPP * V;
-  const FoldMap fm = fold_map(cap);
-  const float inv_d = 1.0f / static_cast<float>(D);
+  const int cap = (1 << tpp_shift) * V;
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   // resident slab: its loads are issued first and fly while the partials are merged
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, raw, ok);
-  // phase A: Chan-merge the S slab statistics of every channel of the tile (each of the
-  // fm.P lanes of a channel takes every P-th slab in order, then the lanes merge pairwise;
-  // the merge is bitwise symmetric, so every workgroup of the instance gets the same bits)
-  const int c_base = g.ct * cap;
-  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
-    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
-    const int sub = static_cast<int>(threadIdx.x) % fm.P;
-    const int c = c_base + cl;
-    const bool in = cl < cap && c < C;
-    Wf w{0.f, 0.f, 0.f};
-    if (in) {
-      const float* q = pstat + ((g.n * S) * 2) * C + c;
-      constexpr int B = 8;
-      batched_for<B>(
-          sub, S, fm.P,
-          [&](int64_t sl, int64_t step) {
-            float tm[B], tq[B];
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              tm[u] = q[((sl + u * step) * 2) * C];
-              tq[u] = q[((sl + u * step) * 2 + 1) * C];
-            }
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, cnt_len)});
-            }
-          },
-          [&](int64_t sl) {
-            w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
-                               cl_slab_count(static_cast<int>(sl), D, cnt_len)});
-          });
-    }
-    for (int m = 1; m < fm.P; m <<= 1) {
-      Wf o;
-      o.mean = lane_xor(w.mean, m);
-      o.m2 = lane_xor(w.m2, m);
-      o.n = lane_xor(w.n, m);
-      w = wf_merge(w, o);
-    }
-    if (sub == 0 && in) {
-      const float rs = rsqrtf(w.m2 * inv_d + eps);
-      sm_mean[cl] = w.mean;
-      sm_rstd[cl] = rs;
-      if (g.s == 0) {
-        mean_out[g.n * C + c] = w.mean;
-        rstd_out[g.n * C + c] = rs;
-      }
-    }
-  }
+  cl_fold_stats(pstat, g, S, cnt_len, D, C, cap, eps, sm_mean, sm_rstd, mean_out, rstd_out);
   __syncthreads();
-  // phase B: apply
   if (g.ch_ok) {
-    // channel of element i inside the tile; elements the thread does not own may fall before
-    // the tile (their results are never stored)
-    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
-    float mean[V], sc[V], bt[V];
-    load_f32<V>(gamma + g.coff, sc);
-    load_f32<V>(beta + g.coff, bt);
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      mean[i] = sm_mean[RG && cl0 + i < 0 ? 0 : cl0 + i];
-      sc[i] *= sm_rstd[RG && cl0 + i < 0 ? 0 : cl0 + i];
-    }
+    ClFwdCoef<V, RG> k;
+    k.load(g, tpp_shift, gamma, beta, sm_mean, sm_rstd);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& pk, int64_t p) {
-      Pack<T, V> o;
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        // subtract the mean first: x * scale - mean * scale would cancel badly when
-        // |mean| >> std
-        o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * sc[i] + bt[i]);
-      }
-      store_pack_from<T, V>(y + boff + p * C, o, RG ? g.lo : 0);
+      store_pack_from<T, V>(y + boff + p * C, k.template apply<T>(pk), RG ? g.lo : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll
@@ -463,8 +627,6 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
   const int TPP = 1 << tpp_shift;
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   float acc[2 * V];
-#pragma unroll
-  for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) {
@@ -478,38 +640,41 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
     load_f32<V>(mean_in + g.n * C + g.coff, mu);
     load_f32<V>(rstd_in + g.n * C + g.coff, rs);
   }
-  auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, bool valid) {
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      const float d = valid ? to_f32(pd.v[i]) : 0.f;
-      const float xh = valid ? (to_f32(px.v[i]) - mu[i]) * rs[i] : 0.f;
-      acc[i] += d * xh;
-      acc[V + i] += d;
-    }
-  };
   if constexpr (U > 0) {
+    cl_resident_sums<T, V, U>(rx, rd, ok, mu, rs, TPP, lds, acc);
+  } else {
 #pragma unroll
-    for (int u = 0; u < U; ++u) add(rx[u], rd[u], ok[u]);
-  } else if (g.ch_ok) {
-    const int64_t boff = (g.n * D) * C + g.coff;
-    constexpr int B = 4;
-    cl_for_pixels<B>(
-        g,
-        [&](int64_t p, int64_t step) {
-          Pack<T, V> px[B], pd[B];
+    for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
+    auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd) {
 #pragma unroll
-          for (int u = 0; u < B; ++u) {
-            px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
-            pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
-          }
+      for (int i = 0; i < V; ++i) {
+        const float d = to_f32(pd.v[i]);
+        const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
+        acc[i] += d * xh;
+        acc[V + i] += d;
+      }
+    };
+    if (g.ch_ok) {
+      const int64_t boff = (g.n * D) * C + g.coff;
+      constexpr int B = 4;
+      cl_for_pixels<B>(
+          g,
+          [&](int64_t p, int64_t step) {
+            Pack<T, V> px[B], pd[B];
 #pragma unroll
-          for (int u = 0; u < B; ++u) add(px[u], pd[u], true);
-        },
-        [&](int64_t p) {
-          add(load_pack<T, V>(x + boff + p * C), load_pack<T, V>(dy + boff + p * C), true);
-        });
+            for (int u = 0; u < B; ++u) {
+              px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
+              pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
+            }
+#pragma unroll
+            for (int u = 0; u < B; ++u) add(px[u], pd[u]);
+          },
+          [&](int64_t p) {
+            add(load_pack<T, V>(x + boff + p * C), load_pack<T, V>(dy + boff + p * C));
+          });
+    }
+    cl_block_sum<2 * V>(acc, lds, TPP);
   }
-  cl_block_sum<2 * V>(acc, lds, TPP);
   if (g.ch_ok && g.slot == 0) {
     float* o = part + ((g.n * S + g.s) * 2) * C + g.coff;
     float t0[V], t1[V];
@@ -524,11 +689,9 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 }
 
 // --------------------------------------------------------------- backward, stage 2
-// dx = r * gamma * (dy - (A + xh * B) / D) with A = sum dy, B = sum dy * xh over the
-// whole (n, c) instance (norm_util.h:599-615 in s1 / s2 form).  Every block first folds
-// the S slab partials of its instance and channel tile into LDS.  The 2 C outputs of
-// dgamma / dbeta are dealt out over the blocks, each a block-wide sum of one column of
-// all N * S partial rows (fixed order, no atomics), which spares a third launch.
+// Every block first folds the S slab partials of its instance and channel tile into LDS and
+// produces its share of dgamma / dbeta (cl_fold_sums), which spares a third launch, then
+// writes dx for its slab.
 template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
@@ -540,9 +703,7 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   __shared__ float sm_b[kClMaxTileChannels];  // sum dy * xh
   __shared__ float red_buf[2][16];
   const int CV = (C + V - 1) / V;
-  const int TPP = 1 << tpp_shift;
-  const int cap = TPP * V;
-  const FoldMap fm = fold_map(cap);
+  const int cap = (1 << tpp_shift) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   // resident slab: its loads are issued first and fly while the partials are folded
@@ -552,94 +713,13 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, rx, okp);
     cl_load_slab<T, V, U, true>(dy + (g.n * D) * C, g, CV, C, rd, okp);
   }
-  const int c_base = g.ct * cap;
-  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
-    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;
-    const int sub = static_cast<int>(threadIdx.x) % fm.P;
-    const int c = c_base + cl;
-    const bool in = cl < cap && c < C;
-    float a = 0.f, b = 0.f;
-    if (in) {
-      const float* pr = part + ((g.n * S) * 2) * C + c;
-      constexpr int B = 16;
-      batched_for<B>(
-          sub, S, fm.P,
-          [&](int64_t sl, int64_t step) {
-            float tb[B], ta[B];
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              tb[u] = pr[((sl + u * step) * 2) * C];
-              ta[u] = pr[((sl + u * step) * 2 + 1) * C];
-            }
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              b += tb[u];
-              a += ta[u];
-            }
-          },
-          [&](int64_t sl) {
-            b += pr[(sl * 2) * C];
-            a += pr[(sl * 2 + 1) * C];
-          });
-    }
-    for (int m = 1; m < fm.P; m <<= 1) {
-      a += lane_xor(a, m);
-      b += lane_xor(b, m);
-    }
-    if (sub == 0 && in) {
-      sm_a[cl] = a;
-      sm_b[cl] = b;
-    }
-  }
-  // dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C]) is the sum of one column
-  // of all N * S partial rows; block w of the grid takes outputs w, w + #blocks, ...
-  const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
-  const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
-  int red_it = 0;
-  for (int64_t o = w; o < 2 * static_cast<int64_t>(C); o += n_blocks) {
-    const int which = o < C ? 0 : 1;
-    const int c = static_cast<int>(o < C ? o : o - C);
-    const int64_t rows = N * S;
-    float t = 0.f;
-    const float* pc = part + static_cast<int64_t>(which) * C + c;
-    batched_for<4>(
-        threadIdx.x, rows, kClThreads,
-        [&](int64_t r, int64_t step) {
-          float v[4];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) v[u] = pc[((r + u * step) * 2) * C];
-#pragma unroll
-          for (int u = 0; u < 4; ++u) t += v[u];
-        },
-        [&](int64_t r) { t += pc[(r * 2) * C]; });
-    t = block_sum1(t, red_buf[red_it & 1]);
-    ++red_it;
-    if (threadIdx.x == 0) (which == 0 ? dgamma : dbeta)[c] = t;
-  }
-  __syncthreads();
+  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, dgamma, dbeta);
   if (g.ch_ok) {
-    // channel of element i inside the tile; elements the thread does not own may fall before
-    // the tile (their results are never stored)
-    const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
-    float mu[V], rs[V], sc[V], ca[V], cb[V];
-    load_f32<V>(mean_in + g.n * C + g.coff, mu);
-    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
-    load_f32<V>(gamma + g.coff, sc);
-#pragma unroll
-    for (int i = 0; i < V; ++i) {
-      sc[i] *= rs[i];
-      ca[i] = -sc[i] * (sm_b[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
-      cb[i] = -sc[i] * (sm_a[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
-    }
+    ClBwdCoef<V, RG> k;
+    k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t p) {
-      Pack<T, V> o;
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
-        o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * xh + cb[i]));
-      }
-      store_pack_from<T, V>(dx + boff + p * C, o, RG ? g.lo : 0);
+      store_pack_from<T, V>(dx + boff + p * C, k.template apply<T>(px, pd), RG ? g.lo : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll
@@ -667,6 +747,125 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
             const int64_t q = rev ? flip - p : p;
             apply(load_pack_last<T, V>(x + boff + q * C), load_pack_last<T, V>(dy + boff + q * C), q);
           });
+    }
+  }
+}
+
+// ------------------------------------------------- one cooperative launch per direction
+// When every slab of the launch is register-resident and the whole grid can be co-resident on
+// the chip, the two stages run as ONE cooperative kernel: a workgroup loads its slab once,
+// publishes the slab's partials, crosses a grid-wide barrier (cooperative_groups; the runtime
+// checks co-residency at launch and owns the barrier state, so no counter needs clearing and no
+// wave spins on a workgroup that cannot be scheduled), folds the partials of its instance and
+// applies from registers.  x (and dy) are read once.  Counterpart of the reference's
+// single-kernel channels-last variant (fused_instance_norm_op.cu:1066-1165), which only takes
+// instances that fit one block's shared memory.
+// The partials are written by workgroups on other XCDs, whose L2s are not coherent with this
+// one: the barrier's device-scope release / acquire makes them visible, and they are read
+// through pointers the compiler may not assume unaliased.
+// y may alias x (dx may alias dy): a workgroup holds all of its elements before it stores any.
+// At least two waves per SIMD (two workgroups per CU): the register budget that keeps a grid
+// of two workgroups per CU co-resident.
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads, 2)
+cl_fwd_coop(const T* x, float* pstat, const float* __restrict__ gamma,
+            const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
+            float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
+            int64_t slab_len, float eps) {
+  __shared__ float lds[V * kClThreads];
+  __shared__ float sm_mean[kClMaxTileChannels];
+  __shared__ float sm_rstd[kClMaxTileChannels];
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  Pack<T, V> raw[U];
+  bool ok[U];
+  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  float mean[V], m2[V];
+  cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(g.p1 - g.p0), TPP, lds, mean, m2);
+  if (g.ch_ok && g.slot == 0) {
+    const int64_t o = ((g.n * S + g.s) * 2) * C + g.coff;
+    store_f32<V>(pstat + o, mean);
+    store_f32<V>(pstat + o + C, m2);
+  }
+  cooperative_groups::this_grid().sync();
+#pragma unroll
+  for (int u = 0; u < U; ++u) forget_derived<T, V>(raw[u]);
+  cl_fold_stats(pstat, g, S, slab_len, D, C, cap, eps, sm_mean, sm_rstd, mean_out, rstd_out);
+  __syncthreads();
+  if (g.ch_ok) {
+    ClFwdCoef<V, false> k;
+    k.load(g, tpp_shift, gamma, beta, sm_mean, sm_rstd);
+    const int64_t boff = (g.n * D) * C + g.coff;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        store_pack<T, V>(y + boff + (g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb) * C,
+                         k.template apply<T>(raw[u]));
+      }
+    }
+  }
+}
+
+template <typename T, int V, int U>
+__global__ void __launch_bounds__(kClThreads, 2)
+cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
+            const float* __restrict__ mean_in, const float* __restrict__ rstd_in, float* part,
+            T* dx, float* __restrict__ dgamma, float* __restrict__ dbeta, int64_t N, int64_t D,
+            int C, int S, int tpp_shift, int64_t slab_len) {
+  __shared__ float lds[2 * V * kClThreads];
+  __shared__ float sm_a[kClMaxTileChannels];
+  __shared__ float sm_b[kClMaxTileChannels];
+  __shared__ float red_buf[2][16];
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  Pack<T, V> rx[U], rd[U];
+  bool ok[U];
+  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
+  cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+  {
+    float mu[V], rs[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
+    if (g.ch_ok) {
+      load_f32<V>(mean_in + g.n * C + g.coff, mu);
+      load_f32<V>(rstd_in + g.n * C + g.coff, rs);
+    }
+    float acc[2 * V];
+    cl_resident_sums<T, V, U>(rx, rd, ok, mu, rs, TPP, lds, acc);
+    if (g.ch_ok && g.slot == 0) {
+      float* o = part + ((g.n * S + g.s) * 2) * C + g.coff;
+      float t0[V], t1[V];
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        t0[i] = acc[i];
+        t1[i] = acc[V + i];
+      }
+      store_f32<V>(o, t0);
+      store_f32<V>(o + C, t1);
+    }
+  }
+  cooperative_groups::this_grid().sync();
+#pragma unroll
+  for (int u = 0; u < U; ++u) {
+    forget_derived<T, V>(rx[u]);
+    forget_derived<T, V>(rd[u]);
+  }
+  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, dgamma, dbeta);
+  if (g.ch_ok) {
+    ClBwdCoef<V, false> k;
+    k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);
+    const int64_t boff = (g.n * D) * C + g.coff;
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        store_pack<T, V>(dx + boff + (g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb) * C,
+                         k.template apply<T>(rx[u], rd[u]));
+      }
     }
   }
 }

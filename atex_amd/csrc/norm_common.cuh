@@ -90,6 +90,19 @@ __device__ __forceinline__ void store_pack(T* p, const Pack<T, V>& v) {
   }
 }
 
+// Makes the compiler forget what it knows about a register-resident vector: values derived
+// from it before this point (its float conversions) cannot be kept alive in its place, so only
+// the raw 16 bytes stay in registers across a long wait.
+template <typename T, int V>
+__device__ __forceinline__ void forget_derived(Pack<T, V>& v) {
+  if constexpr (sizeof(T) * V == 16) {
+    u32x4 bits;
+    __builtin_memcpy(&bits, &v, 16);
+    asm volatile("" : "+v"(bits));
+    __builtin_memcpy(&v, &bits, 16);
+  }
+}
+
 // The first cnt (0 <= cnt <= V) elements of a vector; the rest read as zero / are not written.
 // cnt == V takes the single wide access.
 template <typename T, int V>

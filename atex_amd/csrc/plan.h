@@ -37,6 +37,10 @@ struct Tuning {
   // is what the memory-side cache still holds).
   TuneInt reverse_second_pass{1};
   TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
+  // channels-last: both stages in one cooperative launch when every slab is register-resident
+  // and the grid fits the chip at once.  Off: the grid-wide barrier of the cooperative-groups
+  // runtime measured 50 us on MI355X (the whole two-stage forward takes 15 us).
+  TuneInt cl_coop{0};
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
@@ -325,6 +329,10 @@ struct ClPlan {
   bool fold = false;
   bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
   int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
+  // Several register-resident slabs per instance, few enough workgroups to be on the chip
+  // together: candidates for the single cooperative launch (the runtime has the last word on
+  // co-residency; the two-stage kernels remain the fallback, on the same workspace).
+  bool coop = false;
   size_t off_a = 0, off_fold = 0, ws_bytes = 0;
 };
 constexpr int kClFoldAbove = 64;
@@ -366,6 +374,8 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
     p.fused = true;
     p.fused_u = std::max(1, pow2_ceil(per_thread));
   }
+  p.coop = t.cl_coop && !p.fused && !p.fold && V > 1 && C % V == 0 && p.S > 1 && p.U > 0 &&
+           p.n_work <= int64_t(cus) * 4;
   p.ws_bytes = p.off_fold + align256(sizeof(float) * 2 * size_t(N) * size_t(C));
   return p;
 }

@@ -530,6 +530,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--case", default=DEFAULT_CASE, choices=sorted(CASES) + ["all"])
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--tune", action="append", default=[], metavar="NAME=VALUE",
+                    help="set a launch-planning parameter (atexn_set_tuning) before measuring, "
+                         "in the product and the benchmark build of the library; for A/B runs")
     ap.add_argument("--no-targets", action="store_true",
                     help="default case only: skip the InstanceNorm target shapes")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -544,6 +547,13 @@ def main():
 
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
+    for item in args.tune:
+        from atex_amd.nv_norms import _capi
+
+        key, _, val = item.partition("=")
+        for L in (_capi.lib(), bench_lib()):
+            if L is not None and L.atexn_set_tuning(key.encode(), int(val)) != 0:
+                sys.exit(f"--tune {item}: {L.atexn_last_error().decode()}")
     if args.case == "all":
         for name in CASES:
             if "ref_" in name or "in_1x" in name or "x1" in name or "x2" in name or "x7" in name or name.endswith("_f32"):

@@ -222,3 +222,37 @@ def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
             assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
     finally:
         capi.L.atexn_set_tuning(b"cl_fused", 1)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (4, 32, 4096), (16, 128, 2048), (3, 8, 30000)])
+def test_channels_last_cooperative_launch_matches_two_stage(coracle, N, C, S, dtype):
+    """Both stages in one cooperative launch (switched on through the tuning hook; where the
+    runtime refuses the launch the two-stage kernels run): the same arithmetic on the same
+    partials, so every output must have the bits of the two-stage result."""
+    import torch
+
+    capi = util.Capi()
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 78)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    print(f"IN channels-last cooperative N={N} C={C} spatial={S} {dtype}", flush=True)
+    ref = None
+    try:
+        for coop in (0, 1):
+            assert capi.L.atexn_set_tuning(b"cl_coop", coop) == 0
+            y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+            dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
+            torch.cuda.synchronize()
+            if ref is None:
+                ref = (y, m, r, dx, dg, db)
+            else:
+                for name, a, b in zip(("y", "mean", "inv_std", "dx", "dgamma", "dbeta"), (y, m, r, dx, dg, db), ref):
+                    assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
+    finally:
+        capi.L.atexn_set_tuning(b"cl_coop", 0)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
+    tol = TOL[dtype]
+    assert_close(util.to_host(ref[1]), m_ref, tol["stat"], "mean")
+    assert_close(util.to_host(ref[2]), r_ref, tol["stat"], "inv_std")
+    assert_close(util.to_host(ref[0]), y_ref, tol["y"], "y")
