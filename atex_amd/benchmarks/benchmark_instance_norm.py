@@ -2,7 +2,7 @@
 table of the reference's benchmark (benchmark_instance_norm.py:58-69), both layouts, fp16
 activations with float32 weights.
 
-    python -m atex_amd.benchmarks.benchmark_instance_norm
+    python -m atex_amd.benchmarks.benchmark_instance_norm [--json FILE]
 
 Columns: torch's group_norm with one group per channel on the same GPU (the role
 tensorflow_addons plays in the reference's table; channels-last inputs are handed to it as a
@@ -16,7 +16,7 @@ import torch
 import torch.nn.functional as F
 
 from atex_amd import nv_norms
-from atex_amd.benchmarks.common import fmt, time_train_step
+from atex_amd.benchmarks.common import REPEAT, WARMUP, fmt, one_step_outputs, time_train_step, write_json
 
 # (N, C, spatial extent) -> ((A100, H100) channels-last, (A100, H100) channel-first)
 SHAPES = {
@@ -38,35 +38,66 @@ def expand(s, channel_last):
     return (n, d, d, d, c) if channel_last else (n, c, d, d, d)
 
 
-def benchmark(shape, channel_last: bool, use_fused: bool) -> float:
+def _case(shape, channel_last: bool, use_fused: bool):
+    """(x, fn, params) of one column of the table."""
     torch.manual_seed(0)
     x = torch.randn(shape, device="cuda", dtype=torch.float16, requires_grad=True)
     c = shape[-1] if channel_last else shape[1]
     if use_fused:
         layer = nv_norms.InstanceNormalization(axis=-1 if channel_last else 1)
         layer.build(shape, device="cuda")
-        return time_train_step(x, layer, [layer.gamma, layer.beta])
+        return x, layer, [layer.gamma, layer.beta]
     gamma = torch.ones(c, device="cuda", requires_grad=True)
     beta = torch.zeros(c, device="cuda", requires_grad=True)
     if channel_last:
-        fn = lambda t: F.group_norm(t.permute(0, 4, 1, 2, 3), c, gamma.half(), beta.half(), 1e-3)  # noqa: E731
+        fn = lambda t: F.group_norm(t.permute(0, 4, 1, 2, 3), c, gamma.half(), beta.half(), 1e-3).permute(0, 2, 3, 4, 1)  # noqa: E731
     else:
         fn = lambda t: F.group_norm(t, c, gamma.half(), beta.half(), 1e-3)  # noqa: E731
-    return time_train_step(x, fn, [gamma, beta])
+    return x, fn, [gamma, beta]
+
+
+def benchmark(shape, channel_last: bool, use_fused: bool, warmup: int = WARMUP, repeat: int = REPEAT) -> float:
+    x, fn, params = _case(shape, channel_last, use_fused)
+    return time_train_step(x, fn, params, warmup, repeat)
+
+
+def outputs(shape, channel_last: bool, use_fused: bool):
+    """(y, dx, dgamma, dbeta) of one train step of a column."""
+    return one_step_outputs(*_case(shape, channel_last, use_fused))
+
+
+def run(shapes=None, warmup: int = WARMUP, repeat: int = REPEAT, echo=None):
+    rows = []
+    for channel_last in (True, False):
+        for s, pub in SHAPES.items():
+            if shapes is not None and s not in shapes:
+                continue
+            shape = expand(s, channel_last)
+            a100, h100 = pub[0] if channel_last else pub[1]
+            row = {"shape": list(shape), "layout": "channels_last" if channel_last else "channels_first",
+                   "torch_ms": benchmark(shape, channel_last, False, warmup, repeat),
+                   "fused_ms": benchmark(shape, channel_last, True, warmup, repeat),
+                   "a100_nv_ms": a100, "h100_nv_ms": h100}
+            rows.append(row)
+            if echo:
+                echo(row)
+    return rows
 
 
 def main():
+    import argparse
+
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--json", metavar="FILE", help="also write the table as JSON")
+    args = ap.parse_args()
     if not torch.cuda.is_available():
         raise SystemExit("needs a GPU")
-    for channel_last in (True, False):
-        print(f"InstanceNorm fwd+bwd, fp16, {'channels_last (N, D, H, W, C)' if channel_last else 'channels_first (N, C, D, H, W)'}, ms per train step")
-        print(f"{'shape':>24} | {'torch':>7} {'fused':>7} | A100 NV  H100 NV (published, other hardware)")
-        for s, pub in SHAPES.items():
-            shape = expand(s, channel_last)
-            a100, h100 = pub[0] if channel_last else pub[1]
-            t_native = benchmark(shape, channel_last, False)
-            t_fused = benchmark(shape, channel_last, True)
-            print(f"{str(shape):>24} | {t_native:7.3f} {t_fused:7.3f} | {fmt(a100)}   {fmt(h100)}", flush=True)
+    print("InstanceNorm fwd+bwd, fp16, ms per train step; channels_last (N, D, H, W, C) then channels_first (N, C, D, H, W)")
+    print(f"{'shape':>24} | {'torch':>7} {'fused':>7} | A100 NV  H100 NV (published, other hardware)")
+    rows = run(echo=lambda r: print(f"{str(tuple(r['shape'])):>24} | {r['torch_ms']:7.3f} {r['fused_ms']:7.3f} | "
+                                    f"{fmt(r['a100_nv_ms'])}   {fmt(r['h100_nv_ms'])}", flush=True))
+    if args.json:
+        write_json(args.json, "InstanceNorm 3-D volumes, fp16 activations, float32 weights", rows)
 
 
 if __name__ == "__main__":

@@ -32,3 +32,32 @@ def time_train_step(x, fn, params, warmup=WARMUP, repeat=REPEAT) -> float:
 
 def fmt(v):
     return "   -  " if v is None else f"{v:6.2f}"
+
+
+def one_step_outputs(x, fn, params):
+    """(y, dx, dparams...) of a single step, for comparing two columns of a table.  The loss is
+    a fixed random weighting of y rather than the timed step's plain sum: with dy = 1 the scale
+    gradient is sum(xhat) = 0 and would compare rounding noise only."""
+    y = fn(x)
+    g = torch.Generator(device=y.device).manual_seed(1)
+    w = torch.randn(y.shape, device=y.device, dtype=torch.float32, generator=g).to(y.dtype)
+    grads = torch.autograd.grad((y * w).sum(), [x] + list(params))
+    return (y.detach(),) + tuple(g.detach() for g in grads)
+
+
+def write_json(path, table, rows):
+    """rows: list of dicts.  Adds what is needed to read the file on its own."""
+    import json
+
+    doc = {
+        "table": table,
+        "unit": "ms per train step (layer forward, sum loss, gradients of x, gamma, beta; eager)",
+        "warmup": WARMUP, "repeat": REPEAT,
+        "device": torch.cuda.get_device_name(0) if torch.cuda.is_available() else "cpu",
+        "columns": {"torch_ms": "torch's own op on the same GPU", "fused_ms": "this library's layer",
+                    "a100_nv_ms / h100_nv_ms": "the reference's published figures for its fused op (other hardware)"},
+        "rows": rows,
+    }
+    with open(path, "w") as f:
+        json.dump(doc, f, indent=1)
+        f.write("\n")

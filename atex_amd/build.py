@@ -32,6 +32,7 @@ SOURCES = [
     "rows_launch_f16.hip",
     "rows_launch_bf16.hip",
     "cl_launch.hip",
+    "cpu_kernels.cc",
 ]
 
 # -packed-fp32-ops off: hipcc must not form v_pk_*_f32 from ordinary float code.
@@ -64,7 +65,7 @@ def _deps_mtime() -> float:
 
 
 def _compile(src: str, force: bool, dep_m: float, bench: bool) -> str:
-    obj = os.path.join(OBJ_DIR, src.replace(".hip", "_bench.o" if bench else ".o"))
+    obj = os.path.join(OBJ_DIR, os.path.splitext(src)[0] + ("_bench.o" if bench else ".o"))
     s = os.path.join(CSRC, src)
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= max(os.path.getmtime(s), dep_m):
         return obj

@@ -10,6 +10,7 @@
 #include <mutex>
 #include <vector>
 
+#include "cpu_kernels.h"
 #include "plan.h"
 #include "status.h"
 
@@ -23,7 +24,7 @@ static __device__ __align__(256) unsigned char scratch[ATEXN_STATIC_SCRATCH_BYTE
 
 namespace {
 
-constexpr int kAbiVersion = 1;
+constexpr int kAbiVersion = 2;
 constexpr int64_t kMaxInt = 2147483647;
 
 bool dtype_ok(int dtype) { return dtype == ATEXN_F32 || dtype == ATEXN_F16 || dtype == ATEXN_BF16; }
@@ -48,6 +49,23 @@ int check_tensor(const atexn_tensor* t, const char* name) {
   for (int i = 0; i < t->rank; ++i)
     ATEXN_REQUIRE(t->dims[i] >= 0, "%s has negative dim %lld", name, (long long)t->dims[i]);
   ATEXN_REQUIRE(num_elements(t) == 0 || t->data != nullptr, "%s has elements but a NULL data pointer", name);
+  return ATEXN_OK;
+}
+
+bool device_ok(const atexn_tensor* t) {
+  return t->device == ATEXN_DEVICE_GPU || t->device == ATEXN_DEVICE_CPU;
+}
+
+// All tensors of a call on the device of the first one.
+template <typename... Ts>
+int check_same_device(const atexn_tensor* first, const Ts*... rest) {
+  ATEXN_REQUIRE(device_ok(first), "bad device %d", first->device);
+  const atexn_tensor* all[] = {rest...};
+  for (const atexn_tensor* t : all) {
+    ATEXN_REQUIRE(t->device == first->device,
+                  "all tensors of an op must be on the same device (got %d and %d)", first->device,
+                  t->device);
+  }
   return ATEXN_OK;
 }
 
@@ -278,6 +296,73 @@ int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x
                 workspace_bytes, st);
 }
 
+/* ------------------------------------------------------------- kernel level, host memory */
+
+int atexn_layer_norm_fwd_cpu(int dtype, const void* x, const float* gamma, const float* beta,
+                             int64_t N, int64_t D, float epsilon, void* y, float* mean,
+                             float* inv_std) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
+  if (N == 0 || D == 0) return ATEXN_OK;
+  ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
+  cpu::layer_norm_fwd(dtype, x, gamma, beta, N, D, epsilon, y, mean, inv_std);
+  return ATEXN_OK;
+}
+
+int atexn_layer_norm_bwd_cpu(int dtype, const void* dy, const void* x, const float* gamma,
+                             const float* mean, const float* inv_std, int64_t N, int64_t D,
+                             void* dx, float* dgamma, float* dbeta) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
+  if (N == 0 || D == 0) {
+    if (D > 0) {
+      ATEXN_REQUIRE(dgamma && dbeta, "NULL pointer argument");
+      std::fill(dgamma, dgamma + D, 0.f);
+      std::fill(dbeta, dbeta + D, 0.f);
+    }
+    return ATEXN_OK;
+  }
+  ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
+  ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
+  cpu::layer_norm_bwd(dtype, dy, x, gamma, mean, inv_std, N, D, dx, dgamma, dbeta);
+  return ATEXN_OK;
+}
+
+int atexn_instance_norm_fwd_cpu(int dtype, int layout, const void* x, const float* gamma,
+                                const float* beta, int64_t N, int64_t C, int64_t D,
+                                float epsilon, void* y, float* mean, float* inv_std) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
+  ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
+  if (N == 0 || C == 0 || D == 0) return ATEXN_OK;
+  ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
+  cpu::instance_norm_fwd(dtype, layout == ATEXN_LAYOUT_NC_, x, gamma, beta, N, C, D, epsilon, y, mean,
+                         inv_std);
+  return ATEXN_OK;
+}
+
+int atexn_instance_norm_bwd_cpu(int dtype, int layout, const void* dy, const void* x,
+                                const float* gamma, const float* mean, const float* inv_std,
+                                int64_t N, int64_t C, int64_t D, void* dx, float* dgamma,
+                                float* dbeta) {
+  ATEXN_REQUIRE(dtype_ok(dtype), "bad dtype %d", dtype);
+  ATEXN_REQUIRE(layout == ATEXN_LAYOUT_NC_ || layout == ATEXN_LAYOUT_N_C, "bad layout %d", layout);
+  ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
+  if (N == 0 || C == 0 || D == 0) {
+    if (C > 0) {
+      ATEXN_REQUIRE(dgamma && dbeta, "NULL pointer argument");
+      std::fill(dgamma, dgamma + C, 0.f);
+      std::fill(dbeta, dbeta + C, 0.f);
+    }
+    return ATEXN_OK;
+  }
+  ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
+  ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
+  cpu::instance_norm_bwd(dtype, layout == ATEXN_LAYOUT_NC_, dy, x, gamma, mean, inv_std, N, C, D, dx,
+                         dgamma, dbeta);
+  return ATEXN_OK;
+}
+
 /* ---------------------------------------------------------------------- op level */
 
 int atexn_layer_norm_resolve_axes(int rank, const int64_t* dims, const int* axis, int n_axis,
@@ -332,6 +417,7 @@ int atexn_instance_norm_resolve_format(int rank, const int64_t* dims, const char
 size_t atexn_fused_layer_norm_workspace_bytes(const atexn_tensor* x, const int* axis, int n_axis) {
   int64_t N, D;
   if (!x || atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D) != ATEXN_OK) return 0;
+  if (x->device == ATEXN_DEVICE_CPU) return 0;
   return atexn_layer_norm_fwd_workspace_bytes(x->dtype, N, D);
 }
 
@@ -346,6 +432,7 @@ int atexn_fused_layer_norm(const atexn_tensor* x, const atexn_tensor* scale,
   ATEXN_TRY(check_tensor(y, "y"));
   ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
   ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_TRY(check_same_device(x, scale, offset, y, reserve_space_1, reserve_space_2));
   ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && offset->dtype == ATEXN_F32 &&
                     reserve_space_1->dtype == ATEXN_F32 && reserve_space_2->dtype == ATEXN_F32,
                 "scale, offset and the reserve spaces must be float32");
@@ -362,6 +449,12 @@ int atexn_fused_layer_norm(const atexn_tensor* x, const atexn_tensor* scale,
   ATEXN_REQUIRE(reserve_space_1->rank == 1 && reserve_space_1->dims[0] == N &&
                     reserve_space_2->rank == 1 && reserve_space_2->dims[0] == N,
                 "reserve spaces must be rank 1 with %lld elements", (long long)N);
+  if (x->device == ATEXN_DEVICE_CPU) {
+    return atexn_layer_norm_fwd_cpu(x->dtype, x->data, static_cast<const float*>(scale->data),
+                                    static_cast<const float*>(offset->data), N, D, epsilon, y->data,
+                                    static_cast<float*>(reserve_space_1->data),
+                                    static_cast<float*>(reserve_space_2->data));
+  }
   return atexn_layer_norm_fwd(x->dtype, x->data, static_cast<const float*>(scale->data),
                               static_cast<const float*>(offset->data), N, D, epsilon, y->data,
                               static_cast<float*>(reserve_space_1->data),
@@ -373,6 +466,7 @@ size_t atexn_fused_layer_norm_grad_workspace_bytes(const atexn_tensor* x, const 
                                                    int n_axis) {
   int64_t N, D;
   if (!x || atexn_layer_norm_resolve_axes(x->rank, x->dims, axis, n_axis, &N, &D) != ATEXN_OK) return 0;
+  if (x->device == ATEXN_DEVICE_CPU) return 0;
   return atexn_layer_norm_bwd_workspace_bytes(x->dtype, N, D);
 }
 
@@ -390,6 +484,8 @@ int atexn_fused_layer_norm_grad(const atexn_tensor* y_backprop, const atexn_tens
   ATEXN_TRY(check_tensor(x_backprop, "x_backprop"));
   ATEXN_TRY(check_tensor(scale_backprop, "scale_backprop"));
   ATEXN_TRY(check_tensor(offset_backprop, "offset_backprop"));
+  ATEXN_TRY(check_same_device(x, y_backprop, scale, reserve_space_1, reserve_space_2, x_backprop,
+                              scale_backprop, offset_backprop));
   ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && reserve_space_1->dtype == ATEXN_F32 &&
                     reserve_space_2->dtype == ATEXN_F32 && scale_backprop->dtype == ATEXN_F32 &&
                     offset_backprop->dtype == ATEXN_F32,
@@ -414,6 +510,14 @@ int atexn_fused_layer_norm_grad(const atexn_tensor* y_backprop, const atexn_tens
                 "x_backprop must have the dtype and shape of x");
   ATEXN_REQUIRE(num_elements(scale_backprop) == D && num_elements(offset_backprop) == D,
                 "scale_backprop / offset_backprop must have %lld elements", (long long)D);
+  if (x->device == ATEXN_DEVICE_CPU) {
+    return atexn_layer_norm_bwd_cpu(x->dtype, y_backprop->data, x->data,
+                                    static_cast<const float*>(scale->data),
+                                    static_cast<const float*>(reserve_space_1->data),
+                                    static_cast<const float*>(reserve_space_2->data), N, D,
+                                    x_backprop->data, static_cast<float*>(scale_backprop->data),
+                                    static_cast<float*>(offset_backprop->data));
+  }
   return atexn_layer_norm_bwd(x->dtype, y_backprop->data, x->data,
                               static_cast<const float*>(scale->data),
                               static_cast<const float*>(reserve_space_1->data),
@@ -427,6 +531,7 @@ size_t atexn_fused_instance_norm_workspace_bytes(const atexn_tensor* x, const ch
   int layout;
   int64_t N, C, D;
   if (!x || atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D) != ATEXN_OK) return 0;
+  if (x->device == ATEXN_DEVICE_CPU) return 0;
   return atexn_instance_norm_fwd_workspace_bytes(x->dtype, layout, N, C, D);
 }
 
@@ -441,6 +546,7 @@ int atexn_fused_instance_norm(const atexn_tensor* x, const atexn_tensor* scale,
   ATEXN_TRY(check_tensor(y, "y"));
   ATEXN_TRY(check_tensor(reserve_space_1, "reserve_space_1"));
   ATEXN_TRY(check_tensor(reserve_space_2, "reserve_space_2"));
+  ATEXN_TRY(check_same_device(x, scale, offset, y, reserve_space_1, reserve_space_2));
   ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && offset->dtype == ATEXN_F32 &&
                     reserve_space_1->dtype == ATEXN_F32 && reserve_space_2->dtype == ATEXN_F32,
                 "scale, offset and the reserve spaces must be float32");
@@ -460,6 +566,12 @@ int atexn_fused_instance_norm(const atexn_tensor* x, const atexn_tensor* scale,
   ATEXN_REQUIRE(reserve_space_1->rank == 2 && reserve_space_1->dims[0] == N && reserve_space_1->dims[1] == C &&
                     reserve_space_2->rank == 2 && reserve_space_2->dims[0] == N && reserve_space_2->dims[1] == C,
                 "reserve spaces must have shape [%lld, %lld]", (long long)N, (long long)C);
+  if (x->device == ATEXN_DEVICE_CPU) {
+    return atexn_instance_norm_fwd_cpu(x->dtype, layout, x->data, static_cast<const float*>(scale->data),
+                                       static_cast<const float*>(offset->data), N, C, D, epsilon,
+                                       y->data, static_cast<float*>(reserve_space_1->data),
+                                       static_cast<float*>(reserve_space_2->data));
+  }
   return atexn_instance_norm_fwd(x->dtype, layout, x->data, static_cast<const float*>(scale->data),
                                  static_cast<const float*>(offset->data), N, C, D, epsilon, y->data,
                                  static_cast<float*>(reserve_space_1->data),
@@ -472,6 +584,7 @@ size_t atexn_fused_instance_norm_grad_workspace_bytes(const atexn_tensor* x,
   int layout;
   int64_t N, C, D;
   if (!x || atexn_instance_norm_resolve_format(x->rank, x->dims, data_format, &layout, &N, &C, &D) != ATEXN_OK) return 0;
+  if (x->device == ATEXN_DEVICE_CPU) return 0;
   return atexn_instance_norm_bwd_workspace_bytes(x->dtype, layout, N, C, D);
 }
 
@@ -491,6 +604,8 @@ int atexn_fused_instance_norm_grad(const atexn_tensor* y_backprop, const atexn_t
   ATEXN_TRY(check_tensor(x_backprop, "x_backprop"));
   ATEXN_TRY(check_tensor(scale_backprop, "scale_backprop"));
   ATEXN_TRY(check_tensor(offset_backprop, "offset_backprop"));
+  ATEXN_TRY(check_same_device(x, y_backprop, scale, reserve_space_1, reserve_space_2, x_backprop,
+                              scale_backprop, offset_backprop));
   ATEXN_REQUIRE(scale->dtype == ATEXN_F32 && reserve_space_1->dtype == ATEXN_F32 &&
                     reserve_space_2->dtype == ATEXN_F32 && scale_backprop->dtype == ATEXN_F32 &&
                     offset_backprop->dtype == ATEXN_F32,
@@ -517,6 +632,14 @@ int atexn_fused_instance_norm_grad(const atexn_tensor* y_backprop, const atexn_t
                 "x_backprop must have the dtype and shape of x");
   ATEXN_REQUIRE(num_elements(scale_backprop) == C && num_elements(offset_backprop) == C,
                 "scale_backprop / offset_backprop must have %lld elements", (long long)C);
+  if (x->device == ATEXN_DEVICE_CPU) {
+    return atexn_instance_norm_bwd_cpu(x->dtype, layout, y_backprop->data, x->data,
+                                       static_cast<const float*>(scale->data),
+                                       static_cast<const float*>(reserve_space_1->data),
+                                       static_cast<const float*>(reserve_space_2->data), N, C, D,
+                                       x_backprop->data, static_cast<float*>(scale_backprop->data),
+                                       static_cast<float*>(offset_backprop->data));
+  }
   return atexn_instance_norm_bwd(x->dtype, layout, y_backprop->data, x->data,
                                  static_cast<const float*>(scale->data),
                                  static_cast<const float*>(reserve_space_1->data),

@@ -1,6 +1,7 @@
 """ctypes binding of libatex_norms_hip.so (the C ABI declared in include/atex_norms.h).
 
-Fails loudly when the library is missing: there is no CPU or framework fallback.
+Fails loudly when the library is missing: nothing outside it computes (its CPU kernels serve
+host tensors; they are no fallback for a GPU call).
 """
 from __future__ import annotations
 
@@ -13,6 +14,7 @@ LIB_PATH = os.path.normpath(os.path.join(_HERE, "..", "lib", "libatex_norms_hip.
 ATEXN_F32, ATEXN_F16, ATEXN_BF16 = 0, 1, 2
 ATEXN_LAYOUT_NC_, ATEXN_LAYOUT_N_C = 0, 1
 ATEXN_OK, ATEXN_INVALID_ARGUMENT, ATEXN_LAUNCH_ERROR = 0, 1, 2
+ATEXN_DEVICE_GPU, ATEXN_DEVICE_CPU = 0, 1
 ATEXN_MAX_RANK = 8
 
 
@@ -22,6 +24,7 @@ class AtexnTensor(ctypes.Structure):
         ("rank", ctypes.c_int),
         ("dims", ctypes.c_int64 * ATEXN_MAX_RANK),
         ("data", ctypes.c_void_p),
+        ("device", ctypes.c_int),
     ]
 
 
@@ -57,6 +60,10 @@ SIGNATURES = {
     "atexn_instance_norm_fwd": (_i, [_i, _i, _vp, _vp, _vp, _i64, _i64, _i64, _f, _vp, _vp, _vp, _vp, _sz, _vp]),
     "atexn_instance_norm_bwd_workspace_bytes": (_sz, [_i, _i, _i64, _i64, _i64]),
     "atexn_instance_norm_bwd": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp, _vp, _sz, _vp]),
+    "atexn_layer_norm_fwd_cpu": (_i, [_i, _vp, _vp, _vp, _i64, _i64, _f, _vp, _vp, _vp]),
+    "atexn_layer_norm_bwd_cpu": (_i, [_i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _vp, _vp, _vp]),
+    "atexn_instance_norm_fwd_cpu": (_i, [_i, _i, _vp, _vp, _vp, _i64, _i64, _i64, _f, _vp, _vp, _vp]),
+    "atexn_instance_norm_bwd_cpu": (_i, [_i, _i, _vp, _vp, _vp, _vp, _vp, _i64, _i64, _i64, _vp, _vp, _vp]),
     "atexn_layer_norm_resolve_axes": (_i, [_i, _i64p, _ip, _i, _i64p, _i64p]),
     "atexn_instance_norm_resolve_format": (_i, [_i, _i64p, ctypes.c_char_p, _ip, _i64p, _i64p, _i64p]),
     "atexn_fused_layer_norm_workspace_bytes": (_sz, [_tp, _ip, _i]),
@@ -100,9 +107,10 @@ def check(status: int) -> None:
     raise AtexnError(status, f"{name}: {msg}")
 
 
-def make_tensor(dtype_code: int, shape, ptr: int) -> AtexnTensor:
+def make_tensor(dtype_code: int, shape, ptr: int, device: int = ATEXN_DEVICE_GPU) -> AtexnTensor:
     t = AtexnTensor()
     t.dtype = dtype_code
+    t.device = device
     t.rank = len(shape)
     if len(shape) > ATEXN_MAX_RANK:
         raise InvalidArgumentError(ATEXN_INVALID_ARGUMENT, f"rank {len(shape)} > {ATEXN_MAX_RANK}")

@@ -11,11 +11,14 @@ atex/nv_norms/cc/ops/norm_ops.cc:148-202):
     fused_instance_norm_grad_op(y_backprop, x, scale, reserve_space_1, reserve_space_2,
                                 data_format="N...C", epsilon=0.001)
 
-TensorFlow is not part of this stack; tensors are torch tensors on a ROCm device, used
-purely as owners of device memory and of the HIP stream.  Output allocation (the
-OpKernel's allocate_output / allocate_temp) happens here; validation, axis packing and
-flattening happen in the C ABI (atexn_fused_*), which raises InvalidArgumentError like
-the reference's OP_REQUIRES checks.  There is no CPU path.
+TensorFlow is not part of this stack; tensors are torch tensors, used purely as owners of
+memory and of the HIP stream.  Output allocation (the OpKernel's allocate_output /
+allocate_temp) happens here; validation, axis packing and flattening happen in the C ABI
+(atexn_fused_*), which raises InvalidArgumentError like the reference's OP_REQUIRES checks.
+Tensors on a ROCm device run the HIP kernels; tensors in host memory run the library's CPU
+kernels (the reference registers both, fused_layer_norm_op.cc:465-484), chosen by the device
+of the tensors like a framework's kernel registry does.  Either way the arithmetic is the
+library's: nothing here computes.
 """
 from __future__ import annotations
 
@@ -43,11 +46,32 @@ def _code(t: torch.Tensor, name: str) -> int:
 
 
 def _desc(t: torch.Tensor, name: str) -> _capi.AtexnTensor:
-    if not t.is_cuda:
-        raise RuntimeError(f"{name} must live on the GPU: the fused norm ops have no CPU kernel here")
     if not t.is_contiguous():
         raise InvalidArgumentError(_capi.ATEXN_INVALID_ARGUMENT, f"{name} must be contiguous (row-major)")
-    return _capi.make_tensor(_code(t, name), tuple(t.shape), t.data_ptr() if t.numel() else 0)
+    if t.is_cuda:
+        device = _capi.ATEXN_DEVICE_GPU
+    elif t.device.type == "cpu":
+        device = _capi.ATEXN_DEVICE_CPU
+    else:
+        raise InvalidArgumentError(_capi.ATEXN_INVALID_ARGUMENT, f"{name}: unsupported device {t.device}")
+    return _capi.make_tensor(_code(t, name), tuple(t.shape), t.data_ptr() if t.numel() else 0, device)
+
+
+class _on_device:
+    """Makes a GPU tensor's device current for the allocations and the call (the library plans
+    for the current device); nothing to do for host tensors."""
+
+    def __init__(self, t: torch.Tensor):
+        self._ctx = torch.cuda.device(t.device) if t.is_cuda else None
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            return self._ctx.__exit__(*exc)
+        return False
 
 
 def _axis_array(axis) -> tuple:
@@ -65,6 +89,8 @@ def _workspace(nbytes: int, device) -> tuple:
 
 
 def _stream(device) -> int:
+    if device.type != "cuda":
+        return 0
     return torch.cuda.current_stream(device).cuda_stream
 
 
@@ -82,7 +108,7 @@ def fused_layer_norm_op(x: torch.Tensor, scale: torch.Tensor, offset: torch.Tens
     xd, sd, od = _desc(x, "x"), _desc(scale, "scale"), _desc(offset, "offset")
     n, d = ctypes.c_int64(), ctypes.c_int64()
     _capi.check(L.atexn_layer_norm_resolve_axes(xd.rank, xd.dims, ax, n_ax, ctypes.byref(n), ctypes.byref(d)))
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         y = torch.empty_like(x)
         mean = torch.empty(n.value, dtype=torch.float32, device=x.device)
         inv_std = torch.empty(n.value, dtype=torch.float32, device=x.device)
@@ -103,7 +129,7 @@ def fused_layer_norm_grad_op(y_backprop: torch.Tensor, x: torch.Tensor, scale: t
     ax, n_ax = _axis_array(axis)
     dyd, xd, sd = _desc(y_backprop, "y_backprop"), _desc(x, "x"), _desc(scale, "scale")
     md, rd = _desc(reserve_space_1, "reserve_space_1"), _desc(reserve_space_2, "reserve_space_2")
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         dx = torch.empty_like(x)
         # shaped like scale as passed in (fused_layer_norm_op.cc:451-457)
         dgamma = torch.empty(tuple(scale.shape), dtype=torch.float32, device=x.device)
@@ -132,7 +158,7 @@ def fused_instance_norm_op(x: torch.Tensor, scale: torch.Tensor, offset: torch.T
     n, c, d = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
     _capi.check(L.atexn_instance_norm_resolve_format(xd.rank, xd.dims, fmt, ctypes.byref(layout),
                                                      ctypes.byref(n), ctypes.byref(c), ctypes.byref(d)))
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         y = torch.empty_like(x)
         mean = torch.empty((n.value, c.value), dtype=torch.float32, device=x.device)
         inv_std = torch.empty((n.value, c.value), dtype=torch.float32, device=x.device)
@@ -153,7 +179,7 @@ def fused_instance_norm_grad_op(y_backprop: torch.Tensor, x: torch.Tensor, scale
     fmt = _fmt(data_format)
     dyd, xd, sd = _desc(y_backprop, "y_backprop"), _desc(x, "x"), _desc(scale, "scale")
     md, rd = _desc(reserve_space_1, "reserve_space_1"), _desc(reserve_space_2, "reserve_space_2")
-    with torch.cuda.device(x.device):
+    with _on_device(x):
         dx = torch.empty_like(x)
         dgamma = torch.empty(tuple(scale.shape), dtype=torch.float32, device=x.device)
         dbeta = torch.empty(tuple(scale.shape), dtype=torch.float32, device=x.device)

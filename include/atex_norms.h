@@ -3,6 +3,10 @@
  * and backward on AMD MI355X (gfx950), the drop-in for the device side of NVIDIA/atex's
  * nv_norms custom ops.
  *
+ * The same ops also have host (CPU) kernels, as the reference registers CPU kernels beside its
+ * GPU ones: atexn_*_cpu at the kernel level, and the op level picks them when the tensor
+ * descriptors say ATEXN_DEVICE_CPU.
+ *
  * Two levels:
  *   1. kernel level (atexn_layer_norm_fwd ...): flat [N, D] / [N, C, D] / [N, D, C] views,
  *      raw device pointers, caller-owned workspace, a HIP stream.  These replace the
@@ -58,6 +62,9 @@ enum { ATEXN_F32 = 0, ATEXN_F16 = 1, ATEXN_BF16 = 2 };
 enum { ATEXN_LAYOUT_NC_ = 0, ATEXN_LAYOUT_N_C = 1 };
 
 enum { ATEXN_OK = 0, ATEXN_INVALID_ARGUMENT = 1, ATEXN_LAUNCH_ERROR = 2 };
+
+/* Where a tensor's memory lives (op level).  The zero value is the GPU. */
+enum { ATEXN_DEVICE_GPU = 0, ATEXN_DEVICE_CPU = 1 };
 
 #define ATEXN_MAX_RANK 8
 
@@ -135,14 +142,43 @@ int atexn_instance_norm_bwd(int dtype, int layout, const void* dy, const void* x
                             float* dbeta, void* workspace, size_t workspace_bytes,
                             void* stream);
 
+/* ------------------------------------------------------------- kernel level, host memory */
+
+/* The CPU kernels of the four ops: counterparts of functor::FusedLayerNorm<CPUDevice,T,U>,
+ * FusedLayerNormGrad<CPUDevice,T,U> (cc/kernels/fused_layer_norm_op.cc:27-223, registered
+ * :465-478) and FusedInstanceNorm[Grad]<CPUDevice,T,U> (cc/kernels/fused_instance_norm_op.cc:
+ * 39-284, registered :541-554).  Every pointer is a HOST pointer; the calls are synchronous,
+ * need no workspace and no GPU, and use up to ATEXN_CPU_THREADS (environment; default: all)
+ * host threads.  Same arguments, aliasing rules, return codes and empty-input behaviour as
+ * the GPU entry points (an empty backward zero-fills dgamma / dbeta, fused_layer_norm_op.cc:
+ * 96-103).  Results do not depend on the number of threads. */
+int atexn_layer_norm_fwd_cpu(int dtype, const void* x, const float* gamma, const float* beta,
+                             int64_t N, int64_t D, float epsilon, void* y, float* mean,
+                             float* inv_std);
+int atexn_layer_norm_bwd_cpu(int dtype, const void* dy, const void* x, const float* gamma,
+                             const float* mean, const float* inv_std, int64_t N, int64_t D,
+                             void* dx, float* dgamma, float* dbeta);
+int atexn_instance_norm_fwd_cpu(int dtype, int layout, const void* x, const float* gamma,
+                                const float* beta, int64_t N, int64_t C, int64_t D,
+                                float epsilon, void* y, float* mean, float* inv_std);
+int atexn_instance_norm_bwd_cpu(int dtype, int layout, const void* dy, const void* x,
+                                const float* gamma, const float* mean, const float* inv_std,
+                                int64_t N, int64_t C, int64_t D, void* dx, float* dgamma,
+                                float* dbeta);
+
 /* ---------------------------------------------------------------------- op level */
 
-/* A dense row-major tensor as the op sees it. `dtype` is ATEXN_F32/F16/BF16. */
+/* A dense row-major tensor as the op sees it. `dtype` is ATEXN_F32/F16/BF16, `device` is
+ * ATEXN_DEVICE_GPU (data is a device pointer) or ATEXN_DEVICE_CPU (data is a host pointer).
+ * All tensors of one call must be on the same device: the op then runs the GPU kernels on
+ * `stream`, or the CPU kernels synchronously (workspace and stream are ignored, the workspace
+ * queries return 0), the way a framework picks a registered kernel by device placement. */
 typedef struct atexn_tensor {
   int dtype;
   int rank;
   int64_t dims[ATEXN_MAX_RANK];
-  void* data; /* device pointer; may be NULL only if the tensor has no elements */
+  void* data; /* may be NULL only if the tensor has no elements */
+  int device;
 } atexn_tensor;
 
 /* Axis handling of FusedLayerNorm (cc/ops/norm_ops.cc:18-52,

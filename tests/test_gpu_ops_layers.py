@@ -88,7 +88,7 @@ def test_layer_norm_op_errors():
         nv_norms.fused_layer_norm_op(x.double(), g, g, axis=[1, 2])
     with pytest.raises(InvalidArgumentError, match="contiguous"):
         nv_norms.fused_layer_norm_op(x.transpose(0, 1), g, g, axis=[1, 2])
-    with pytest.raises(RuntimeError, match="must live on the GPU"):
+    with pytest.raises(InvalidArgumentError, match="same device"):
         nv_norms.fused_layer_norm_op(x.cpu(), g, g, axis=[1, 2])
     y, m, r = nv_norms.fused_layer_norm_op(x, g, g, axis=[1, 2])
     with pytest.raises(InvalidArgumentError, match="x and y_backprop must have same shape"):
@@ -113,7 +113,7 @@ def test_instance_norm_op_errors():
         nv_norms.fused_instance_norm_op(x, g, g, data_format="NC...")
     with pytest.raises(InvalidArgumentError, match="scale must be 1-dimensional"):
         nv_norms.fused_instance_norm_op(x, g.reshape(4, 8), g)
-    with pytest.raises(RuntimeError, match="must live on the GPU"):
+    with pytest.raises(InvalidArgumentError, match="same device"):
         nv_norms.fused_instance_norm_op(x.cpu(), g, g)
 
 

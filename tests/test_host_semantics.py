@@ -51,7 +51,7 @@ def test_every_declared_symbol_is_exported(L):
         out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
         exported = {line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("atexn_")}
         assert exported == set(names), (path, exported ^ set(names))
-    assert L.atexn_abi_version() == 1
+    assert L.atexn_abi_version() == 2
     assert L.atexn_status_string(0) == b"OK"
     assert L.atexn_status_string(1) == b"INVALID_ARGUMENT"
     assert L.atexn_status_string(2) == b"LAUNCH_ERROR"
@@ -248,7 +248,7 @@ def test_workspace_queries_without_gpu(L):
 
 def test_python_layer_semantics_on_cpu():
     """The wrappers' own checks (reference: nv_norm_ops.py:86-93, :152-158) run before any
-    device work; valid calls on CPU tensors fail loudly, there is no CPU kernel."""
+    device work; valid calls on host tensors run the library's CPU kernels."""
     import torch
 
     from atex_amd import nv_norms
@@ -269,13 +269,11 @@ def test_python_layer_semantics_on_cpu():
     ln.build((2, 3, 4))
     assert tuple(ln.gamma.shape) == (3, 4) and ln.gamma.dtype == torch.float32
     assert [tuple(w.shape) for w in ln.get_weights()] == [(3, 4), (3, 4)]
-    with pytest.raises(RuntimeError, match="must live on the GPU"):
-        ln(x)
+    assert tuple(ln(x).shape) == (2, 3, 4)
     inn = nv_norms.InstanceNormalization(axis=1)
     inn.build((2, 7, 4, 5))
     assert tuple(inn.gamma.shape) == (7,) and inn.beta.dtype == torch.float32
-    with pytest.raises(RuntimeError, match="must live on the GPU"):
-        inn(torch.zeros(2, 7, 4, 5, dtype=torch.float16))
+    assert inn(torch.zeros(2, 7, 4, 5, dtype=torch.float16)).dtype == torch.float16
     assert set(n for n in dir(nv_norms) if not n.startswith("__")) >= {
         "LayerNormalization", "InstanceNormalization", "fused_layer_norm_op", "fused_layer_norm_grad_op",
         "fused_instance_norm_op", "fused_instance_norm_grad_op", "_layer_norm_grad", "_instance_norm_grad"}
