@@ -332,10 +332,11 @@ __device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], cons
 // of the block's instance and channel tile into sm_b (sum dy * xh) and sm_a (sum dy), and
 // produces the block's share of dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C])
 // is the sum of one column of all N * S partial rows (fixed order, no atomics); block w of the
-// grid takes outputs w, w + #blocks, ...  Ends with a block-wide barrier.
+// grid takes outputs w, w + #blocks, ...  Ends with a block-wide barrier.  fold_lds: 256 floats.
 __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g, int64_t N, int S,
                                              int C, int cap, float* sm_a, float* sm_b,
-                                             float (*red_buf)[16], float* __restrict__ dgamma,
+                                             float (*red_buf)[16], float* fold_lds,
+                                             float* __restrict__ dgamma,
                                              float* __restrict__ dbeta) {
   const FoldMap fm = fold_map(cap);
   const int c_base = g.ct * cap;
@@ -379,26 +380,56 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
   }
   const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
   const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+  const int64_t rows = N * S;
+  const int64_t W2 = 2 * static_cast<int64_t>(C);  // a partial row: [dgamma terms | dbeta terms]
+  // Outputs are dealt to the blocks in chunks of cw adjacent columns, cw the largest of 64, 16,
+  // 4 that still gives every block a chunk: the threads of a chunk read cw adjacent floats of a
+  // partial row at a time.  With more blocks than that, one column per block-wide sum.
+  int cw = 64;
+  while (cw > 1 && (W2 + cw - 1) / cw < n_blocks) cw >>= 2;
+  if (cw > 1) {
+    const int cx = static_cast<int>(threadIdx.x) % cw;
+    const int cy = static_cast<int>(threadIdx.x) / cw;
+    const int rp = kClThreads / cw;  // partial rows in flight
+    const int64_t n_chunks = (W2 + cw - 1) / cw;
+    for (int64_t chunk = w; chunk < n_chunks; chunk += n_blocks) {
+      const int64_t col = chunk * cw + cx;
+      float t[1] = {0.f};
+      if (col < W2) {
+        const float* pc = part + col;
+        batched_for<4>(
+            cy, rows, rp,
+            [&](int64_t r, int64_t step) {
+              float v[4];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) v[u] = pc[(r + u * step) * W2];
+#pragma unroll
+              for (int u = 0; u < 4; ++u) t[0] += v[u];
+            },
+            [&](int64_t r) { t[0] += pc[r * W2]; });
+      }
+      cl_block_sum<1>(t, fold_lds, cw);
+      if (cy == 0 && col < W2) (col < C ? dgamma : dbeta)[col < C ? col : col - C] = t[0];
+      __syncthreads();
+    }
+  }
   int red_it = 0;
-  for (int64_t o = w; o < 2 * static_cast<int64_t>(C); o += n_blocks) {
-    const int which = o < C ? 0 : 1;
-    const int c = static_cast<int>(o < C ? o : o - C);
-    const int64_t rows = N * S;
+  for (int64_t o = w; cw == 1 && o < W2; o += n_blocks) {
     float t = 0.f;
-    const float* pc = part + static_cast<int64_t>(which) * C + c;
+    const float* pc = part + o;
     batched_for<4>(
         threadIdx.x, rows, kClThreads,
         [&](int64_t r, int64_t step) {
           float v[4];
 #pragma unroll
-          for (int u = 0; u < 4; ++u) v[u] = pc[((r + u * step) * 2) * C];
+          for (int u = 0; u < 4; ++u) v[u] = pc[(r + u * step) * W2];
 #pragma unroll
           for (int u = 0; u < 4; ++u) t += v[u];
         },
-        [&](int64_t r) { t += pc[(r * 2) * C]; });
+        [&](int64_t r) { t += pc[r * W2]; });
     t = block_sum1(t, red_buf[red_it & 1]);
     ++red_it;
-    if (threadIdx.x == 0) (which == 0 ? dgamma : dbeta)[c] = t;
+    if (threadIdx.x == 0) (o < C ? dgamma : dbeta)[o < C ? o : o - C] = t;
   }
   __syncthreads();
 }
@@ -702,6 +733,7 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   __shared__ float sm_a[kClMaxTileChannels];  // sum dy
   __shared__ float sm_b[kClMaxTileChannels];  // sum dy * xh
   __shared__ float red_buf[2][16];
+  __shared__ float fold_lds[kClThreads];
   const int CV = (C + V - 1) / V;
   const int cap = (1 << tpp_shift) * V;
   const float inv_d = 1.0f / static_cast<float>(D);
@@ -713,7 +745,7 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, rx, okp);
     cl_load_slab<T, V, U, true>(dy + (g.n * D) * C, g, CV, C, rd, okp);
   }
-  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, dgamma, dbeta);
+  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, fold_lds, dgamma, dbeta);
   if (g.ch_ok) {
     ClBwdCoef<V, RG> k;
     k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);
@@ -855,7 +887,8 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
     forget_derived<T, V>(rx[u]);
     forget_derived<T, V>(rd[u]);
   }
-  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, dgamma, dbeta);
+  __syncthreads();  // lds is free again
+  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, lds, dgamma, dbeta);
   if (g.ch_ok) {
     ClBwdCoef<V, false> k;
     k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);

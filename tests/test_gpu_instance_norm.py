@@ -256,3 +256,11 @@ def test_channels_last_cooperative_launch_matches_two_stage(coracle, N, C, S, dt
     assert_close(util.to_host(ref[1]), m_ref, tol["stat"], "mean")
     assert_close(util.to_host(ref[2]), r_ref, tol["stat"], "inv_std")
     assert_close(util.to_host(ref[0]), y_ref, tol["y"], "y")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(2, 2048, 64), (1, 4096, 40), (3, 520, 300), (2, 96, 5000)])
+def test_channels_last_wide_channel_counts(capi, coracle, N, C, S, dtype):
+    """Few workgroups and thousands of channels: the dgamma / dbeta fold of the second backward
+    stage deals its outputs out in chunks of adjacent columns."""
+    run_case(capi, coracle, N, C, S, dtype, False, 29)
