@@ -177,12 +177,6 @@ __device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, i
   }
 }
 
-// Count of pixels of slab s when an instance of D pixels is cut into slabs of slab_len.
-__device__ __forceinline__ float cl_slab_count(int s, int64_t D, int64_t slab_len) {
-  const int64_t beg = static_cast<int64_t>(s) * slab_len;
-  return static_cast<float>(beg + slab_len <= D ? slab_len : D - beg);
-}
-
 // ------------------------------------------------------- building blocks of the stages
 // Statistics of a register-resident slab: an exact two-pass over the registers (block-wide
 // sum -> slab mean, block-wide sum of squared deviations from it).  lds: V * 256 floats.
@@ -215,12 +209,16 @@ __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], co
   cl_block_sum<V>(m2, lds, TPP);
 }
 
-// Chan-merge of the S slab statistics pstat[(n * S + s)][2][C] of every channel of the
-// block's tile into sm_mean / sm_rstd (and, from the block of slab 0, into the op's outputs).
-// Each of the fm.P lanes of a channel takes every P-th slab in order, then the lanes merge
-// pairwise; the merge is bitwise symmetric, so every workgroup of the instance gets the same
-// bits.  The counts follow from cnt_len (the slab length; after cl_merge_stats S == 1 and
-// cnt_len == D).  The caller synchronises the block before it reads sm_mean / sm_rstd.
+// Combination of the S slab statistics pstat[(n * S + s)][2][C] of every channel of the block's
+// tile into sm_mean / sm_rstd (and, from the block of slab 0, into the op's outputs), in two
+// sweeps over the partials (a few KiB, cache-resident):
+//     mean = sum_s n_s mean_s / D,      m2 = sum_s [ m2_s + n_s (mean_s - mean)^2 ]
+// which is Chan's merge (norm_util.h:190-210) of all slabs at once: every term of m2 is
+// non-negative, nothing cancels, and there is no division or dependent chain per slab.  Each of
+// the fm.P lanes of a channel takes every P-th slab in order, then the lanes add pairwise
+// (commutative, so every workgroup of the instance gets the same bits).  The counts follow from
+// cnt_len (the slab length; after cl_merge_stats S == 1 and cnt_len == D).  The caller
+// synchronises the block before it reads sm_mean / sm_rstd.
 __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& g, int S,
                                               int64_t cnt_len, int64_t D, int C, int cap,
                                               float eps, float* sm_mean, float* sm_rstd,
@@ -228,16 +226,33 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
                                               float* __restrict__ rstd_out) {
   const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
+  const float n_full = static_cast<float>(cnt_len);
+  const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * cnt_len);
   const int c_base = g.ct * cap;
   for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
     const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
     const int sub = static_cast<int>(threadIdx.x) % fm.P;
     const int c = c_base + cl;
     const bool in = cl < cap && c < C;
-    Wf w{0.f, 0.f, 0.f};
+    const float* q = pstat + ((g.n * S) * 2) * C + (in ? c : 0);
+    constexpr int B = 8;
+    float s1 = 0.f;
     if (in) {
-      const float* q = pstat + ((g.n * S) * 2) * C + c;
-      constexpr int B = 8;
+      batched_for<B>(
+          sub, S, fm.P,
+          [&](int64_t sl, int64_t step) {
+            float tm[B];
+#pragma unroll
+            for (int u = 0; u < B; ++u) tm[u] = q[((sl + u * step) * 2) * C];
+#pragma unroll
+            for (int u = 0; u < B; ++u) s1 += tm[u] * (sl + u * step == S - 1 ? n_last : n_full);
+          },
+          [&](int64_t sl) { s1 += q[(sl * 2) * C] * (sl == S - 1 ? n_last : n_full); });
+    }
+    for (int m = 1; m < fm.P; m <<= 1) s1 += lane_xor(s1, m);
+    const float mean = s1 * inv_d;
+    float m2 = 0.f;
+    if (in) {
       batched_for<B>(
           sub, S, fm.P,
           [&](int64_t sl, int64_t step) {
@@ -249,27 +264,22 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
             }
 #pragma unroll
             for (int u = 0; u < B; ++u) {
-              w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, cnt_len)});
+              const float d = tm[u] - mean;
+              m2 += tq[u] + (sl + u * step == S - 1 ? n_last : n_full) * (d * d);
             }
           },
           [&](int64_t sl) {
-            w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
-                               cl_slab_count(static_cast<int>(sl), D, cnt_len)});
+            const float d = q[(sl * 2) * C] - mean;
+            m2 += q[(sl * 2 + 1) * C] + (sl == S - 1 ? n_last : n_full) * (d * d);
           });
     }
-    for (int m = 1; m < fm.P; m <<= 1) {
-      Wf o;
-      o.mean = lane_xor(w.mean, m);
-      o.m2 = lane_xor(w.m2, m);
-      o.n = lane_xor(w.n, m);
-      w = wf_merge(w, o);
-    }
+    for (int m = 1; m < fm.P; m <<= 1) m2 += lane_xor(m2, m);
     if (sub == 0 && in) {
-      const float rs = rsqrtf(w.m2 * inv_d + eps);
-      sm_mean[cl] = w.mean;
+      const float rs = rsqrtf(m2 * inv_d + eps);
+      sm_mean[cl] = mean;
       sm_rstd[cl] = rs;
       if (g.s == 0) {
-        mean_out[g.n * C + c] = w.mean;
+        mean_out[g.n * C + c] = mean;
         rstd_out[g.n * C + c] = rs;
       }
     }
@@ -541,24 +551,51 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
   }
 }
 
-// Between the stages, only when an instance has more than kClFoldAbove slabs: merges the S slab
-// statistics of every (instance, channel) once, in a fixed order, into folded[N][2][C] = (mean,
-// m2 of the whole instance), so that the stage-2 workgroups need not each do it.  Block =
-// kClMergeChannels channels x (256 / kClMergeChannels) slab phases; grid = (channel groups, N).
+// Between the stages, only when an instance has more than kClFoldAbove slabs: combines the S slab
+// statistics of every (instance, channel) once, in a fixed order and by the same two sweeps as
+// cl_fold_stats, into folded[N][2][C] = (mean, m2 of the whole instance), so that the stage-2
+// workgroups need not each do it.  Block = kClMergeChannels channels x (256 / kClMergeChannels)
+// slab phases; grid = (channel groups, N).
 constexpr int kClMergeChannels = 16;
 __global__ void __launch_bounds__(kClThreads)
 cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int64_t D, int C, int S,
                int64_t slab_len) {
   constexpr int PH = kClThreads / kClMergeChannels;
-  __shared__ Wf buf[PH][kClMergeChannels];
+  __shared__ float buf[PH][kClMergeChannels];
   const int cx = threadIdx.x % kClMergeChannels;
   const int ph = threadIdx.x / kClMergeChannels;
   const int c = blockIdx.x * kClMergeChannels + cx;
   const int64_t n = blockIdx.y;
-  Wf w{0.f, 0.f, 0.f};
-  if (c < C) {
-    const float* q = pstat + ((n * S) * 2) * C + c;
-    constexpr int B = 8;
+  const bool in = c < C;
+  const float n_full = static_cast<float>(slab_len);
+  const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * slab_len);
+  const float* q = pstat + ((n * S) * 2) * C + (in ? c : 0);
+  constexpr int B = 8;
+  // the phases' partial sums of a channel, added in phase order
+  auto across_phases = [&](float v) {
+    buf[ph][cx] = v;
+    __syncthreads();
+    float r = buf[0][cx];
+    for (int k = 1; k < PH; ++k) r += buf[k][cx];
+    __syncthreads();
+    return r;
+  };
+  float s1 = 0.f;
+  if (in) {
+    batched_for<B>(
+        ph, S, PH,
+        [&](int64_t sl, int64_t step) {
+          float tm[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) tm[u] = q[((sl + u * step) * 2) * C];
+#pragma unroll
+          for (int u = 0; u < B; ++u) s1 += tm[u] * (sl + u * step == S - 1 ? n_last : n_full);
+        },
+        [&](int64_t sl) { s1 += q[(sl * 2) * C] * (sl == S - 1 ? n_last : n_full); });
+  }
+  const float mean = across_phases(s1) / static_cast<float>(D);
+  float m2 = 0.f;
+  if (in) {
     batched_for<B>(
         ph, S, PH,
         [&](int64_t sl, int64_t step) {
@@ -570,21 +607,19 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
           }
 #pragma unroll
           for (int u = 0; u < B; ++u) {
-            w = wf_merge(w, Wf{tm[u], tq[u], cl_slab_count(static_cast<int>(sl + u * step), D, slab_len)});
+            const float d = tm[u] - mean;
+            m2 += tq[u] + (sl + u * step == S - 1 ? n_last : n_full) * (d * d);
           }
         },
         [&](int64_t sl) {
-          w = wf_merge(w, Wf{q[(sl * 2) * C], q[(sl * 2 + 1) * C],
-                             cl_slab_count(static_cast<int>(sl), D, slab_len)});
+          const float d = q[(sl * 2) * C] - mean;
+          m2 += q[(sl * 2 + 1) * C] + (sl == S - 1 ? n_last : n_full) * (d * d);
         });
   }
-  buf[ph][cx] = w;
-  __syncthreads();
-  if (ph == 0 && c < C) {
-    Wf r = buf[0][cx];
-    for (int k = 1; k < PH; ++k) r = wf_merge(r, buf[k][cx]);
-    folded[(n * 2) * C + c] = r.mean;
-    folded[(n * 2 + 1) * C + c] = r.m2;
+  m2 = across_phases(m2);
+  if (ph == 0 && in) {
+    folded[(n * 2) * C + c] = mean;
+    folded[(n * 2 + 1) * C + c] = m2;
   }
 }
 

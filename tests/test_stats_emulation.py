@@ -10,7 +10,8 @@ zero-padded border of an image whose interior has a large mean.
 * `batch_welford`: what cl_fwd_stats (streaming variant) and chunk_wf do: every thread takes
   batches of B register-resident values, exact two-pass per batch, Chan update of its running
   (mean, m2, n) (the reference's Welford push, norm_util.h:182-211, is the B = 1 case); the
-  workgroup combines its threads around the slab mean; slabs merge with Chan's formula.
+  workgroup combines its threads around the slab mean, and the slabs combine the same way
+  around the instance mean (Chan's merge of all parts at once).
   It must stay within 1e-5 whatever the outliers.
 
 The GPU tests of the same inputs are in test_gpu_conditioning.py.
@@ -39,21 +40,11 @@ def pivot_sums(x, K, threads):
     return float(mean), float(var)
 
 
-def _wf_merge(a, b):
-    """Chan's pairwise merge in float32 on (mean, m2, n) triples (arrays or scalars)."""
-    n = (a[2] + b[2]).astype(F)
-    inv = np.where(n > 0, F(1) / np.maximum(n, F(1)), F(0)).astype(F)
-    d = (b[0] - a[0]).astype(F)
-    mean = ((a[0] * a[2] + b[0] * b[2]) * inv).astype(F)
-    m2 = ((a[1] + b[1]) + (d * d) * ((a[2] * b[2]) * inv)).astype(F)
-    return mean, m2, n
-
-
 def batch_welford(x, threads, batch, slab_len):
     """x: (D,) float32; slabs of slab_len elements, inside a slab thread t owns
     slab[t::threads] and takes it `batch` values at a time."""
     D = x.size
-    total = (np.zeros((), F), np.zeros((), F), np.zeros((), F))
+    slabs = []
     for beg in range(0, D, slab_len):
         slab = x[beg:beg + slab_len]
         per_thread = slab.size // threads
@@ -75,8 +66,17 @@ def batch_welford(x, threads, batch, slab_len):
         slab_mean = F(_seq_sum((mean * n).astype(F), 0) / F(slab.size))
         dd = (mean - slab_mean).astype(F)
         slab_m2 = _seq_sum((m2 + n * (dd * dd)).astype(F), 0)
-        total = _wf_merge(total, (slab_mean, slab_m2, np.asarray(slab.size, F)))
-    return float(total[0]), float(total[1] / F(D))
+        slabs.append((slab_mean, slab_m2, F(slab.size)))
+    # the slabs combine in two sweeps: mean = sum n_s mean_s / D, m2 = sum m2_s + n_s (mean_s - mean)^2
+    s1 = F(0)
+    for m, _, n in slabs:
+        s1 = F(s1 + m * n)
+    mean = F(s1 / F(D))
+    m2 = F(0)
+    for m, q, n in slabs:
+        d = F(m - mean)
+        m2 = F(m2 + F(q + n * F(d * d)))
+    return float(mean), float(m2 / F(D))
 
 
 def _rel_err_inv_std(var, x):
