@@ -250,7 +250,7 @@ void layer_norm_bwd_t(const T* dy, const T* x, const float* gamma, const float* 
   const int64_t rows_per_block = (N + blocks - 1) / blocks;
   std::vector<double> part(static_cast<size_t>(blocks) * 2 * D, 0.0);
   double* pp = part.data();
-  parallel_ranges(blocks, 1, [=](int64_t b0, int64_t b1) {
+  parallel_ranges(blocks, rows_per_thread_floor(rows_per_block * D), [=](int64_t b0, int64_t b1) {
     for (int64_t b = b0; b < b1; ++b) {
       double* ag = pp + b * 2 * D;
       double* ab = ag + D;
