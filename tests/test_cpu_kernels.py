@@ -282,3 +282,39 @@ def test_op_level_and_layers_on_host_tensors():
                                   ctypes.byref(t_gpu), ctypes.byref(s), ctypes.byref(s), None, 0, None)
     assert st == 1 and b"same device" in L.atexn_last_error()
     assert L.atexn_fused_layer_norm_workspace_bytes(ctypes.byref(t_cpu), ax, 1) == 0
+
+
+def test_cpu_kernels_random_shapes(cpu):
+    """Seeded random shapes (rows of 1 .. 5000 elements, 1 .. 40 rows / instances, both layouts,
+    every dtype) against the numpy float64 closed forms."""
+    rng = np.random.Generator(np.random.PCG64(77))
+    for case in range(120):
+        dtype = ("f32", "f16", "bf16")[case % 3]
+        tol = TOL[dtype]
+        if case % 2 == 0:
+            N, D = int(rng.integers(1, 40)), int(rng.integers(1, 5000))
+            x, gamma, beta, dy = util.ln_inputs("row_mean", N, D, dtype, 1000 + case)
+            xv, dyv = O.from_storage(x, dtype), O.from_storage(dy, dtype)
+            y_ref, m_ref, r_ref = O.ln_fwd_np(xv, gamma, beta, EPS)
+            y, m, r = cpu.ln_fwd(x, gamma, beta, EPS, dtype)
+            m32, r32 = m_ref.astype(np.float32), r_ref.astype(np.float32)
+            dx_ref, dg_ref, db_ref = O.ln_bwd_np(dyv, xv, gamma, m32, r32)
+            dx, dg, db = cpu.ln_bwd(dy, x, gamma, m32, r32, dtype)
+        else:
+            N, C, S = int(rng.integers(1, 6)), int(rng.integers(1, 70)), int(rng.integers(1, 900))
+            cf = bool(rng.integers(0, 2))
+            x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, cf, 1000 + case)
+            xv, dyv = O.from_storage(x, dtype), O.from_storage(dy, dtype)
+            y_ref, m_ref, r_ref = O.in_fwd_np(xv, gamma, beta, EPS, cf)
+            y, m, r = cpu.in_fwd(x, gamma, beta, EPS, dtype, cf)
+            m32, r32 = m_ref.astype(np.float32), r_ref.astype(np.float32)
+            dx_ref, dg_ref, db_ref = O.in_bwd_np(dyv, xv, gamma, m32, r32, cf)
+            dx, dg, db = cpu.in_bwd(dy, x, gamma, m32, r32, dtype, cf)
+        what = f"case {case} {dtype} x{x.shape}"
+        assert_close(m, m_ref, 1e-5, what + " mean")
+        assert_close(r, r_ref, 1e-5, what + " inv_std")
+        assert_close(_vals(y, dtype), y_ref, tol["y"], what + " y")
+        scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), r32, dtype)
+        assert_close(_vals(dx, dtype), dx_ref, tol["dx"], what + " dx", scale=scale)
+        assert_close(dg, dg_ref, 1e-5, what + " dgamma")
+        assert_close(db, db_ref, 1e-5, what + " dbeta")

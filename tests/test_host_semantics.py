@@ -301,3 +301,74 @@ def test_header_is_plain_c_and_links_from_c(tmp_path):
     out = subprocess.run([exe], capture_output=True, text=True, timeout=60)
     assert out.returncode == 0, out.stderr + out.stdout
     assert "capi host check ok" in out.stdout
+
+
+# ------------------------------------------------------------------ property tests
+def _axes_model(dims, axis):
+    """Python restatement of GetBatchAndFeatureSizes (cc/ops/norm_ops.cc:18-52): wrap negative
+    axes, reject out-of-range ones, sort, drop duplicates, require the set to be packed up to
+    the last dim.  Returns (N, D) or an error word."""
+    rank = len(dims)
+    wrapped = []
+    for a in axis:
+        w = a + rank if a < 0 else a
+        if w < 0 or w >= rank:
+            return "invalid"
+        wrapped.append(w)
+    uniq = sorted(set(wrapped))
+    if uniq[0] != rank - len(uniq):
+        return "packed"
+    n = d = 1
+    for i, v in enumerate(dims):
+        if i >= uniq[0]:
+            d *= v
+        else:
+            n *= v
+    return n, d
+
+
+def test_axis_resolution_property(L):
+    from hypothesis import given, settings
+    from hypothesis import strategies as st
+
+    @settings(max_examples=400, deadline=None)
+    @given(st.lists(st.integers(0, 9), min_size=1, max_size=6).flatmap(
+        lambda dims: st.tuples(st.just(dims),
+                               st.lists(st.integers(-len(dims) - 2, len(dims) + 1), min_size=1, max_size=7))))
+    def check(case):
+        dims, axis = case
+        want = _axes_model(dims, axis)
+        st_, n, d, msg = resolve_axes(L, dims, axis)
+        if want == "invalid":
+            assert st_ == 1 and "axis contains invalid value" in msg
+        elif want == "packed":
+            assert st_ == 1 and "axis is not packed from last dim." in msg
+        else:
+            assert st_ == 0 and (n, d) == want
+
+    check()
+
+
+def test_data_format_property(L):
+    """fused_instance_norm_op.cc:25-34: accepted iff len > 2, [0] == 'N' and ([1] == 'C' or
+    [-1] == 'C'); a 'C' in position 1 wins."""
+    from hypothesis import given, settings
+    from hypothesis import strategies as st
+
+    @settings(max_examples=400, deadline=None)
+    @given(st.text(alphabet="NCHWD.x", min_size=0, max_size=7), st.lists(st.integers(0, 6), min_size=4, max_size=6))
+    def check(fmt, dims):
+        ok = len(fmt) > 2 and fmt[0] == "N" and (fmt[1] == "C" or fmt[-1] == "C")
+        st_, layout, n, c, d, msg = resolve_format(L, dims, fmt.encode())
+        if not ok:
+            assert st_ == 1 and "We only accept" in msg
+            return
+        cf = fmt[1] == "C"
+        spatial = dims[2:] if cf else dims[1:-1]
+        prod = 1
+        for v in spatial:
+            prod *= v
+        assert st_ == 0 and layout == (0 if cf else 1)
+        assert (n, c, d) == (dims[0], dims[1] if cf else dims[-1], prod)
+
+    check()
