@@ -1,9 +1,13 @@
 """Timing protocol shared by the two benchmark scripts: the reference's train step
 (benchmark_layer_norm.py:16-51): forward through the layer, loss = sum(y), gradients with
 respect to x, gamma and beta; 10 warm-up steps, 20 timed steps, one host synchronisation at
-the end; result in milliseconds per step, eager dispatch overhead included."""
+the end; result in milliseconds per step, eager dispatch overhead included.  Python's cyclic
+garbage collector is off during the timed steps, as in the standard library's timeit: a full
+collection of a process with torch loaded takes tens of milliseconds and would land on
+whichever row of a table happens to cross its threshold."""
 from __future__ import annotations
 
+import gc
 import time
 
 import torch
@@ -23,11 +27,19 @@ def time_train_step(x, fn, params, warmup=WARMUP, repeat=REPEAT) -> float:
     for _ in range(warmup):
         g = train_step(x, fn, params)
     _ = float(g[0].float().sum())  # the reference synchronises through reduce_sum(dx).numpy()
-    start = time.perf_counter()
-    for _ in range(repeat):
-        g = train_step(x, fn, params)
-    _ = float(g[0].float().sum())
-    return 1000.0 * (time.perf_counter() - start) / repeat
+    gc.collect()
+    gc_was_on = gc.isenabled()
+    gc.disable()
+    try:
+        start = time.perf_counter()
+        for _ in range(repeat):
+            g = train_step(x, fn, params)
+        _ = float(g[0].float().sum())
+        elapsed = time.perf_counter() - start
+    finally:
+        if gc_was_on:
+            gc.enable()
+    return 1000.0 * elapsed / repeat
 
 
 def fmt(v):

@@ -77,6 +77,8 @@ CASES = {
     "in_1x32x128x128x128_cl": ("in", "f16", (1, 32, 128 ** 3, False)),
     "inref_8x64x64_cl": ("in", "f16", (8, 64, 64 ** 3, False)),
     "inref_8x64x64_cf": ("in", "f16", (8, 64, 64 ** 3, True)),
+    "inref_8x128x64_cl": ("in", "f16", (8, 128, 64 ** 3, False)),
+    "inref_8x128x64_cf": ("in", "f16", (8, 128, 64 ** 3, True)),
     "inref_4x256x32_cl": ("in", "f16", (4, 256, 32 ** 3, False)),
     "inref_4x256x32_cf": ("in", "f16", (4, 256, 32 ** 3, True)),
 }
