@@ -42,6 +42,7 @@ struct ClGeom {
   int ppb;         // pixel slots per block
   bool ch_ok;      // channel vector inside C
   int64_t p0, p1;  // pixel range of the slab
+  int slab_n;      // p1 - p0 (resident slabs only: they have at most 16 * 256 pixels)
 };
 
 template <bool RG>
@@ -66,6 +67,7 @@ __device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, i
   }
   g.p0 = static_cast<int64_t>(g.s) * slab_len;
   g.p1 = g.p0 + slab_len < D ? g.p0 + slab_len : D;
+  g.slab_n = static_cast<int>(g.p1 - g.p0 < (1 << 20) ? g.p1 - g.p0 : (1 << 20));
   return g;
 }
 
@@ -139,6 +141,16 @@ __device__ __forceinline__ void cl_block_sum(float (&v)[K], float* lds, int TPP)
 // How the threads of a block split the fold over S partial rows for the channels of a
 // tile of `cap` channels (cap = TPP * V, a power of two): P adjacent lanes per channel
 // when the tile has at most 256 channels, else one lane per channel and several sweeps.
+// Slab partials per lane up to which a fold keeps all of them in registers.
+constexpr int kClFoldRegs = 16;
+
+// base[at], or 0 when the position is not the lane's (the load itself is unconditional and
+// `at` then names valid memory).
+__device__ __forceinline__ float q_or_zero(const float* base, unsigned at, bool mine) {
+  const float v = base[at];
+  return mine ? v : 0.f;
+}
+
 struct FoldMap {
   int P;       // lanes per channel (power of two, <= 64)
   int sweeps;  // passes over the tile when it has more channels than threads
@@ -164,15 +176,22 @@ __device__ __forceinline__ void cl_for_pixels(const ClGeom& g, Full&& full, Tail
 // are unconditional so that they are all in flight at once: a lane whose pixel or channel
 // vector lies outside the slab reads the slab's first pixel / the last channel vector
 // instead (always valid memory) and is masked out of the arithmetic.
+// Positions inside a slab are 32-bit element offsets from the slab's first pixel (`slab`, the
+// same address for the whole workgroup): a resident slab has at most 4096 pixels and the
+// planner keeps 4096 * C * sizeof(T) below 2^31, so no thread carries 64-bit addresses for its
+// U pixels through the kernel.
+__device__ __forceinline__ unsigned cl_slab_offset(const ClGeom& g, int C, int u) {
+  return static_cast<unsigned>(g.slot + u * g.ppb) * static_cast<unsigned>(C) + static_cast<unsigned>(g.coff);
+}
+
 template <typename T, int V, int U, bool LAST = false>
-__device__ __forceinline__ void cl_load_slab(const T* base_n, const ClGeom& g, int CV, int C,
+__device__ __forceinline__ void cl_load_slab(const T* slab, const ClGeom& g, int C,
                                              Pack<T, V> (&raw)[U], bool (&ok)[U]) {
-  const T* b = base_n + g.coff;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    const int64_t p = g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb;
-    ok[u] = g.ch_ok && p < g.p1;
-    const T* src = b + (p < g.p1 ? p : g.p0) * C;
+    ok[u] = g.ch_ok && g.slot + u * g.ppb < g.slab_n;
+    const bool inside = g.slot + u * g.ppb < g.slab_n;
+    const T* src = slab + (inside ? cl_slab_offset(g, C, u) : static_cast<unsigned>(g.coff));
     raw[u] = LAST ? load_pack_last<T, V>(src) : load_pack<T, V>(src);
   }
 }
@@ -210,18 +229,23 @@ __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], co
 }
 
 // Combination of the S slab statistics pstat[(n * S + s)][2][C] of every channel of the block's
-// tile into sm_mean / sm_rstd (and, from the block of slab 0, into the op's outputs), in two
+// tile (and, from the block of slab 0, into the op's outputs), in two
 // sweeps over the partials (a few KiB, cache-resident):
 //     mean = sum_s n_s mean_s / D,      m2 = sum_s [ m2_s + n_s (mean_s - mean)^2 ]
 // which is Chan's merge (norm_util.h:190-210) of all slabs at once: every term of m2 is
 // non-negative, nothing cancels, and there is no division or dependent chain per slab.  Each of
 // the fm.P lanes of a channel takes every P-th slab in order, then the lanes add pairwise
 // (commutative, so every workgroup of the instance gets the same bits).  The counts follow from
-// cnt_len (the slab length; after cl_merge_stats S == 1 and cnt_len == D).  The caller
-// synchronises the block before it reads sm_mean / sm_rstd.
+// cnt_len (the slab length; after cl_merge_stats S == 1 and cnt_len == D).  The lane that ends
+// up with a channel's statistics also fetched its gamma / beta (issued with the partials, one
+// round trip) and leaves the constants of y = (x - sm_mean) * sm_sc + sm_bt in LDS, so that no
+// thread of the apply phase loads anything but x.  The caller synchronises the block before it
+// reads them.
 __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& g, int S,
                                               int64_t cnt_len, int64_t D, int C, int cap,
-                                              float eps, float* sm_mean, float* sm_rstd,
+                                              float eps, const float* __restrict__ gamma,
+                                              const float* __restrict__ beta, float* sm_mean,
+                                              float* sm_sc, float* sm_bt,
                                               float* __restrict__ mean_out,
                                               float* __restrict__ rstd_out) {
   const FoldMap fm = fold_map(cap);
@@ -229,55 +253,89 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
   const float n_full = static_cast<float>(cnt_len);
   const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * cnt_len);
   const int c_base = g.ct * cap;
+  // The partials of the instance: one address for the whole workgroup; positions inside are
+  // 32-bit (the planner keeps 2 * S * C below 2^32).
+  const float* q = pstat + ((g.n * S) * 2) * C;
+  const unsigned uC = static_cast<unsigned>(C), uS = static_cast<unsigned>(S);
+  const unsigned P = static_cast<unsigned>(fm.P);
   for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
     const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;  // channel in tile
-    const int sub = static_cast<int>(threadIdx.x) % fm.P;
+    const unsigned sub = static_cast<unsigned>(threadIdx.x) % P;
     const int c = c_base + cl;
     const bool in = cl < cap && c < C;
-    const float* q = pstat + ((g.n * S) * 2) * C + (in ? c : 0);
-    constexpr int B = 8;
-    float s1 = 0.f;
-    if (in) {
-      batched_for<B>(
-          sub, S, fm.P,
-          [&](int64_t sl, int64_t step) {
-            float tm[B];
-#pragma unroll
-            for (int u = 0; u < B; ++u) tm[u] = q[((sl + u * step) * 2) * C];
-#pragma unroll
-            for (int u = 0; u < B; ++u) s1 += tm[u] * (sl + u * step == S - 1 ? n_last : n_full);
-          },
-          [&](int64_t sl) { s1 += q[(sl * 2) * C] * (sl == S - 1 ? n_last : n_full); });
+    const unsigned cc = in ? static_cast<unsigned>(c) : 0u;
+    float gm = 0.f, bt = 0.f;
+    if (sub == 0 && in) {
+      gm = gamma[c];
+      bt = beta[c];
     }
-    for (int m = 1; m < fm.P; m <<= 1) s1 += lane_xor(s1, m);
-    const float mean = s1 * inv_d;
-    float m2 = 0.f;
-    if (in) {
-      batched_for<B>(
-          sub, S, fm.P,
-          [&](int64_t sl, int64_t step) {
-            float tm[B], tq[B];
+    constexpr int B = 8;
+    constexpr int R = kClFoldRegs;
+    float s1 = 0.f, m2 = 0.f, mean;
+    if (uS <= R * P) {
+      // few slabs per lane: all of a lane's (mean, m2) pairs are loaded at once, one memory
+      // round trip for both sweeps (a lane without a slab in a position reads slab 0 and
+      // weighs it 0); same order of additions as the general path below
+      float tm[R], tq[R], tn[R];
 #pragma unroll
-            for (int u = 0; u < B; ++u) {
-              tm[u] = q[((sl + u * step) * 2) * C];
-              tq[u] = q[((sl + u * step) * 2 + 1) * C];
-            }
+      for (int u = 0; u < R; ++u) {
+        const unsigned sl = sub + u * P;
+        const bool ok = in && sl < uS;
+        const unsigned at = ok ? sl : 0u;
+        tm[u] = q[(at * 2) * uC + cc];
+        tq[u] = q[(at * 2 + 1) * uC + cc];
+        tn[u] = !ok ? 0.f : (sl == uS - 1 ? n_last : n_full);
+      }
 #pragma unroll
-            for (int u = 0; u < B; ++u) {
-              const float d = tm[u] - mean;
-              m2 += tq[u] + (sl + u * step == S - 1 ? n_last : n_full) * (d * d);
-            }
-          },
-          [&](int64_t sl) {
-            const float d = q[(sl * 2) * C] - mean;
-            m2 += q[(sl * 2 + 1) * C] + (sl == S - 1 ? n_last : n_full) * (d * d);
-          });
+      for (int u = 0; u < R; ++u) s1 += tm[u] * tn[u];
+      for (int m = 1; m < fm.P; m <<= 1) s1 += lane_xor(s1, m);
+      mean = s1 * inv_d;
+#pragma unroll
+      for (int u = 0; u < R; ++u) {
+        const float d = tm[u] - mean;
+        m2 += tn[u] == 0.f ? 0.f : tq[u] + tn[u] * (d * d);
+      }
+    } else {
+      if (in) {
+        for (unsigned sl = sub; sl < uS; sl += B * P) {
+          float tm[B], tn[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            const unsigned k = sl + u * P;
+            tm[u] = q[((k < uS ? k : 0u) * 2) * uC + cc];
+            tn[u] = k >= uS ? 0.f : (k == uS - 1 ? n_last : n_full);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) s1 += tm[u] * tn[u];
+        }
+      }
+      for (int m = 1; m < fm.P; m <<= 1) s1 += lane_xor(s1, m);
+      mean = s1 * inv_d;
+      if (in) {
+        for (unsigned sl = sub; sl < uS; sl += B * P) {
+          float tm[B], tq[B], tn[B];
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            const unsigned k = sl + u * P;
+            const unsigned at = k < uS ? k : 0u;
+            tm[u] = q[(at * 2) * uC + cc];
+            tq[u] = q[(at * 2 + 1) * uC + cc];
+            tn[u] = k >= uS ? 0.f : (k == uS - 1 ? n_last : n_full);
+          }
+#pragma unroll
+          for (int u = 0; u < B; ++u) {
+            const float d = tm[u] - mean;
+            m2 += tn[u] == 0.f ? 0.f : tq[u] + tn[u] * (d * d);
+          }
+        }
+      }
     }
     for (int m = 1; m < fm.P; m <<= 1) m2 += lane_xor(m2, m);
     if (sub == 0 && in) {
       const float rs = rsqrtf(m2 * inv_d + eps);
       sm_mean[cl] = mean;
-      sm_rstd[cl] = rs;
+      sm_sc[cl] = gm * rs;
+      sm_bt[cl] = bt;
       if (g.s == 0) {
         mean_out[g.n * C + c] = mean;
         rstd_out[g.n * C + c] = rs;
@@ -286,22 +344,21 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
   }
 }
 
-// Per-thread constants of the forward apply: mean and gamma * rstd of the thread's channels.
+// Per-thread constants of the forward apply, read from what cl_fold_stats left in LDS.
 template <int V, bool RG>
 struct ClFwdCoef {
   float mean[V], sc[V], bt[V];
-  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, const float* gamma,
-                                       const float* beta, const float* sm_mean,
-                                       const float* sm_rstd) {
+  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, const float* sm_mean,
+                                       const float* sm_sc, const float* sm_bt) {
     // channel of element i inside the tile; elements the thread does not own may fall before
     // the tile (their results are never stored)
     const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
-    load_f32<V>(gamma + g.coff, sc);
-    load_f32<V>(beta + g.coff, bt);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      mean[i] = sm_mean[RG && cl0 + i < 0 ? 0 : cl0 + i];
-      sc[i] *= sm_rstd[RG && cl0 + i < 0 ? 0 : cl0 + i];
+      const int at = RG && cl0 + i < 0 ? 0 : cl0 + i;
+      mean[i] = sm_mean[at];
+      sc[i] = sm_sc[at];
+      bt[i] = sm_bt[at];
     }
   }
   template <typename T>
@@ -339,55 +396,24 @@ __device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], cons
 }
 
 // Backward counterpart of cl_fold_stats: adds up the S slab partials part[(n * S + s)][2][C]
-// of the block's instance and channel tile into sm_b (sum dy * xh) and sm_a (sum dy), and
+// of the block's instance and channel tile into B = sum dy * xh and A = sum dy, leaves the
+// constants of dx = sm_sc * dy + (sm_ca * (x - sm_mu) + sm_cb) in LDS (sc = gamma * r,
+// ca = -sc * r * B / D, cb = -sc * A / D; norm_util.h:599-615 in s1 / s2 form; gamma, mean and
+// inverse std of a channel are fetched by the lane that folds it, with the partials), and
 // produces the block's share of dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C])
 // is the sum of one column of all N * S partial rows (fixed order, no atomics); block w of the
 // grid takes outputs w, w + #blocks, ...  Ends with a block-wide barrier.  fold_lds: 256 floats.
 __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g, int64_t N, int S,
-                                             int C, int cap, float* sm_a, float* sm_b,
+                                             int C, int cap, float inv_d,
+                                             const float* __restrict__ gamma,
+                                             const float* __restrict__ mean_in,
+                                             const float* __restrict__ rstd_in, float* sm_mu,
+                                             float* sm_sc, float* sm_ca, float* sm_cb,
                                              float (*red_buf)[16], float* fold_lds,
                                              float* __restrict__ dgamma,
                                              float* __restrict__ dbeta) {
   const FoldMap fm = fold_map(cap);
   const int c_base = g.ct * cap;
-  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
-    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;
-    const int sub = static_cast<int>(threadIdx.x) % fm.P;
-    const int c = c_base + cl;
-    const bool in = cl < cap && c < C;
-    float a = 0.f, b = 0.f;
-    if (in) {
-      const float* pr = part + ((g.n * S) * 2) * C + c;
-      constexpr int B = 16;
-      batched_for<B>(
-          sub, S, fm.P,
-          [&](int64_t sl, int64_t step) {
-            float tb[B], ta[B];
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              tb[u] = pr[((sl + u * step) * 2) * C];
-              ta[u] = pr[((sl + u * step) * 2 + 1) * C];
-            }
-#pragma unroll
-            for (int u = 0; u < B; ++u) {
-              b += tb[u];
-              a += ta[u];
-            }
-          },
-          [&](int64_t sl) {
-            b += pr[(sl * 2) * C];
-            a += pr[(sl * 2 + 1) * C];
-          });
-    }
-    for (int m = 1; m < fm.P; m <<= 1) {
-      a += lane_xor(a, m);
-      b += lane_xor(b, m);
-    }
-    if (sub == 0 && in) {
-      sm_a[cl] = a;
-      sm_b[cl] = b;
-    }
-  }
   const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
   const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
   const int64_t rows = N * S;
@@ -397,6 +423,76 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
   // partial row at a time.  With more blocks than that, one column per block-wide sum.
   int cw = 64;
   while (cw > 1 && (W2 + cw - 1) / cw < n_blocks) cw >>= 2;
+  // At most one output per block and at most kEarly partial rows per thread: the column's loads
+  // are issued here, ahead of the slab fold's, so that both share one memory round trip.
+  constexpr int kEarly = 4;
+  const bool early = cw == 1 && W2 <= n_blocks && rows <= kEarly * kClThreads;
+  float ev[kEarly];
+  if (early) {
+#pragma unroll
+    for (int u = 0; u < kEarly; ++u) {
+      const int64_t r = static_cast<int64_t>(threadIdx.x) + u * kClThreads;
+      ev[u] = (w < W2 && r < rows) ? part[r * W2 + w] : 0.f;
+    }
+  }
+  // the partials of the instance: one address for the whole workgroup, 32-bit positions inside
+  const float* pr = part + ((g.n * S) * 2) * C;
+  const unsigned uC = static_cast<unsigned>(C), uS = static_cast<unsigned>(S);
+  const unsigned P = static_cast<unsigned>(fm.P);
+  for (int sweep = 0; sweep < fm.sweeps; ++sweep) {
+    const int cl = sweep * kClThreads + static_cast<int>(threadIdx.x) / fm.P;
+    const unsigned sub = static_cast<unsigned>(threadIdx.x) % P;
+    const int c = c_base + cl;
+    const bool in = cl < cap && c < C;
+    const unsigned cc = in ? static_cast<unsigned>(c) : 0u;
+    float gm = 0.f, mu = 0.f, rs = 0.f;
+    if (sub == 0 && in) {
+      gm = gamma[c];
+      mu = mean_in[g.n * C + c];
+      rs = rstd_in[g.n * C + c];
+    }
+    float a = 0.f, b = 0.f;
+    if (in) {
+      constexpr int B = kClFoldRegs;
+      for (unsigned sl = sub; sl < uS; sl += B * P) {
+        float tb[B], ta[B];
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+          const unsigned k = sl + u * P;
+          const unsigned at = k < uS ? k : 0u;
+          tb[u] = q_or_zero(pr, (at * 2) * uC + cc, k < uS);
+          ta[u] = q_or_zero(pr, (at * 2 + 1) * uC + cc, k < uS);
+        }
+#pragma unroll
+        for (int u = 0; u < B; ++u) {
+          b += tb[u];
+          a += ta[u];
+        }
+      }
+    }
+    for (int m = 1; m < fm.P; m <<= 1) {
+      a += lane_xor(a, m);
+      b += lane_xor(b, m);
+    }
+    if (sub == 0 && in) {
+      const float sc = gm * rs;
+      sm_mu[cl] = mu;
+      sm_sc[cl] = sc;
+      sm_ca[cl] = -(sc * rs) * (b * inv_d);
+      sm_cb[cl] = -sc * (a * inv_d);
+    }
+  }
+  if (early) {
+    if (w < W2) {  // uniform over the block
+      float t = 0.f;
+#pragma unroll
+      for (int u = 0; u < kEarly; ++u) t += ev[u];
+      t = block_sum1(t, red_buf[0]);
+      if (threadIdx.x == 0) (w < C ? dgamma : dbeta)[w < C ? w : w - C] = t;
+    }
+    __syncthreads();
+    return;
+  }
   if (cw > 1) {
     const int cx = static_cast<int>(threadIdx.x) % cw;
     const int cy = static_cast<int>(threadIdx.x) / cw;
@@ -444,25 +540,21 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
   __syncthreads();
 }
 
-// Per-thread constants of the backward apply:
-// dx = r * gamma * (dy - (A + xh * B) / D) with A = sum dy, B = sum dy * xh over the whole
-// (n, c) instance (norm_util.h:599-615 in s1 / s2 form) = sc * dy + (ca * xh + cb).
+// Per-thread constants of the backward apply, read from what cl_fold_sums left in LDS.
 template <int V, bool RG>
 struct ClBwdCoef {
-  float mu[V], rs[V], sc[V], ca[V], cb[V];
-  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, int C, float inv_d,
-                                       const float* gamma, const float* mean_in,
-                                       const float* rstd_in, const float* sm_a,
-                                       const float* sm_b) {
+  float mu[V], sc[V], ca[V], cb[V];
+  __device__ __forceinline__ void load(const ClGeom& g, int tpp_shift, const float* sm_mu,
+                                       const float* sm_sc, const float* sm_ca,
+                                       const float* sm_cb) {
     const int cl0 = g.coff - ((g.ct << tpp_shift) * V);
-    load_f32<V>(mean_in + g.n * C + g.coff, mu);
-    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
-    load_f32<V>(gamma + g.coff, sc);
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      sc[i] *= rs[i];
-      ca[i] = -sc[i] * (sm_b[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
-      cb[i] = -sc[i] * (sm_a[RG && cl0 + i < 0 ? 0 : cl0 + i] * inv_d);
+      const int at = RG && cl0 + i < 0 ? 0 : cl0 + i;
+      mu[i] = sm_mu[at];
+      sc[i] = sm_sc[at];
+      ca[i] = sm_ca[at];
+      cb[i] = sm_cb[at];
     }
   }
   template <typename T>
@@ -470,8 +562,7 @@ struct ClBwdCoef {
     Pack<T, V> o;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      const float xh = (to_f32(px.v[i]) - mu[i]) * rs[i];
-      o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * xh + cb[i]));
+      o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * (to_f32(px.v[i]) - mu[i]) + cb[i]));
     }
     return o;
   }
@@ -502,7 +593,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
   if constexpr (U > 0) {
     Pack<T, V> raw[U];
     bool ok[U];
-    cl_load_slab<T, V, U>(xn, g, CV, C, raw, ok);
+    cl_load_slab<T, V, U>(xn + g.p0 * C, g, C, raw, ok);
     cl_resident_stats<T, V, U>(raw, ok, inv_n, TPP, lds, mean, m2);
   } else {
     WfLanes<V> run;
@@ -627,25 +718,27 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
 template <typename T, int V, int U, bool RG>
-__global__ void __launch_bounds__(kClThreads)
+__global__ void __launch_bounds__(kClThreads, 2)  // two workgroups per CU: a grid of 2 x CUs slabs runs in one round
 cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restrict__ gamma,
              const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
              float* __restrict__ rstd_out, int64_t D, int C, int S, int64_t cnt_len,
              int tpp_shift, int64_t slab_len, float eps, int rev) {
   __shared__ float sm_mean[kClMaxTileChannels];
-  __shared__ float sm_rstd[kClMaxTileChannels];
+  __shared__ float sm_sc[kClMaxTileChannels];
+  __shared__ float sm_bt[kClMaxTileChannels];
   const int CV = (C + V - 1) / V;
   const int cap = (1 << tpp_shift) * V;
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, slab_len);
   // resident slab: its loads are issued first and fly while the partials are merged
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
-  if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, raw, ok);
-  cl_fold_stats(pstat, g, S, cnt_len, D, C, cap, eps, sm_mean, sm_rstd, mean_out, rstd_out);
+  if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
+  cl_fold_stats(pstat, g, S, cnt_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
+                rstd_out);
   __syncthreads();
   if (g.ch_ok) {
     ClFwdCoef<V, RG> k;
-    k.load(g, tpp_shift, gamma, beta, sm_mean, sm_rstd);
+    k.load(g, tpp_shift, sm_mean, sm_sc, sm_bt);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& pk, int64_t p) {
       store_pack_from<T, V>(y + boff + p * C, k.template apply<T>(pk), RG ? g.lo : 0);
@@ -653,7 +746,10 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
     if constexpr (U > 0) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (ok[u]) apply(raw[u], g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb);
+        if (ok[u]) {
+          store_pack_from<T, V>(y + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
+                                k.template apply<T>(raw[u]), RG ? g.lo : 0);
+        }
       }
     } else {
       constexpr int B = 8;
@@ -696,8 +792,8 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) {
-    cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
-    cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+    cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+    cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   }
   float mu[V], rs[V];
 #pragma unroll
@@ -759,14 +855,16 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 // produces its share of dgamma / dbeta (cl_fold_sums), which spares a third launch, then
 // writes dx for its slab.
 template <typename T, int V, int U, bool RG>
-__global__ void __launch_bounds__(kClThreads)
+__global__ void __launch_bounds__(kClThreads, 2)  // two workgroups per CU: a grid of 2 x CUs slabs runs in one round
 cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
              const float* __restrict__ part, T* dx, float* __restrict__ dgamma,
              float* __restrict__ dbeta, int64_t N, int64_t D, int C, int S, int tpp_shift,
              int64_t slab_len, int rev) {
-  __shared__ float sm_a[kClMaxTileChannels];  // sum dy
-  __shared__ float sm_b[kClMaxTileChannels];  // sum dy * xh
+  __shared__ float sm_mu[kClMaxTileChannels];
+  __shared__ float sm_sc[kClMaxTileChannels];
+  __shared__ float sm_ca[kClMaxTileChannels];
+  __shared__ float sm_cb[kClMaxTileChannels];
   __shared__ float red_buf[2][16];
   __shared__ float fold_lds[kClThreads];
   const int CV = (C + V - 1) / V;
@@ -777,13 +875,14 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool okp[U > 0 ? U : 1];
   if constexpr (U > 0) {
-    cl_load_slab<T, V, U, true>(x + (g.n * D) * C, g, CV, C, rx, okp);
-    cl_load_slab<T, V, U, true>(dy + (g.n * D) * C, g, CV, C, rd, okp);
+    cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, rx, okp);
+    cl_load_slab<T, V, U, true>(dy + (g.n * D + g.p0) * C, g, C, rd, okp);
   }
-  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, fold_lds, dgamma, dbeta);
+  cl_fold_sums(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
+               red_buf, fold_lds, dgamma, dbeta);
   if (g.ch_ok) {
     ClBwdCoef<V, RG> k;
-    k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);
+    k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t p) {
       store_pack_from<T, V>(dx + boff + p * C, k.template apply<T>(px, pd), RG ? g.lo : 0);
@@ -791,7 +890,10 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     if constexpr (U > 0) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
-        if (okp[u]) apply(rx[u], rd[u], g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb);
+        if (okp[u]) {
+          store_pack_from<T, V>(dx + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
+                                k.template apply<T>(rx[u], rd[u]), RG ? g.lo : 0);
+        }
       }
     } else {
       constexpr int B = 4;
@@ -841,14 +943,15 @@ cl_fwd_coop(const T* x, float* pstat, const float* __restrict__ gamma,
             int64_t slab_len, float eps) {
   __shared__ float lds[V * kClThreads];
   __shared__ float sm_mean[kClMaxTileChannels];
-  __shared__ float sm_rstd[kClMaxTileChannels];
+  __shared__ float sm_sc[kClMaxTileChannels];
+  __shared__ float sm_bt[kClMaxTileChannels];
   const int CV = C / V;
   const int TPP = 1 << tpp_shift;
   const int cap = TPP * V;
   const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
   Pack<T, V> raw[U];
   bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
   float mean[V], m2[V];
   cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(g.p1 - g.p0), TPP, lds, mean, m2);
   if (g.ch_ok && g.slot == 0) {
@@ -859,16 +962,16 @@ cl_fwd_coop(const T* x, float* pstat, const float* __restrict__ gamma,
   cooperative_groups::this_grid().sync();
 #pragma unroll
   for (int u = 0; u < U; ++u) forget_derived<T, V>(raw[u]);
-  cl_fold_stats(pstat, g, S, slab_len, D, C, cap, eps, sm_mean, sm_rstd, mean_out, rstd_out);
+  cl_fold_stats(pstat, g, S, slab_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
+                rstd_out);
   __syncthreads();
   if (g.ch_ok) {
     ClFwdCoef<V, false> k;
-    k.load(g, tpp_shift, gamma, beta, sm_mean, sm_rstd);
-    const int64_t boff = (g.n * D) * C + g.coff;
+    k.load(g, tpp_shift, sm_mean, sm_sc, sm_bt);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (ok[u]) {
-        store_pack<T, V>(y + boff + (g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb) * C,
+        store_pack<T, V>(y + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
                          k.template apply<T>(raw[u]));
       }
     }
@@ -882,8 +985,10 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
             T* dx, float* __restrict__ dgamma, float* __restrict__ dbeta, int64_t N, int64_t D,
             int C, int S, int tpp_shift, int64_t slab_len) {
   __shared__ float lds[2 * V * kClThreads];
-  __shared__ float sm_a[kClMaxTileChannels];
-  __shared__ float sm_b[kClMaxTileChannels];
+  __shared__ float sm_mu[kClMaxTileChannels];
+  __shared__ float sm_sc[kClMaxTileChannels];
+  __shared__ float sm_ca[kClMaxTileChannels];
+  __shared__ float sm_cb[kClMaxTileChannels];
   __shared__ float red_buf[2][16];
   const int CV = C / V;
   const int TPP = 1 << tpp_shift;
@@ -892,8 +997,8 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
   const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
   Pack<T, V> rx[U], rd[U];
   bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
-  cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+  cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   {
     float mu[V], rs[V];
 #pragma unroll
@@ -923,15 +1028,15 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
     forget_derived<T, V>(rd[u]);
   }
   __syncthreads();  // lds is free again
-  cl_fold_sums(part, g, N, S, C, cap, sm_a, sm_b, red_buf, lds, dgamma, dbeta);
+  cl_fold_sums(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
+               red_buf, lds, dgamma, dbeta);
   if (g.ch_ok) {
     ClBwdCoef<V, false> k;
-    k.load(g, tpp_shift, C, inv_d, gamma, mean_in, rstd_in, sm_a, sm_b);
-    const int64_t boff = (g.n * D) * C + g.coff;
+    k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       if (ok[u]) {
-        store_pack<T, V>(dx + boff + (g.p0 + g.slot + static_cast<int64_t>(u) * g.ppb) * C,
+        store_pack<T, V>(dx + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
                          k.template apply<T>(rx[u], rd[u]));
       }
     }
@@ -958,7 +1063,7 @@ cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restric
   const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
   Pack<T, V> raw[U];
   bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, raw, ok);
+  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
   float gm[V], bt[V];
   load_f32<V>(gamma + g.coff, gm);
   load_f32<V>(beta + g.coff, bt);
@@ -993,14 +1098,13 @@ cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restric
     rs[i] = rsqrtf(q[i] * inv_d + eps);
     gm[i] *= rs[i];
   }
-  const int64_t boff = (g.n * D) * C + g.coff;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (ok[u]) {
       Pack<T, V> o;
 #pragma unroll
       for (int i = 0; i < V; ++i) o.v[i] = from_f32<T>((to_f32(raw[u].v[i]) - mean[i]) * gm[i] + bt[i]);
-      store_pack<T, V>(y + boff + (g.slot + static_cast<int64_t>(u) * g.ppb) * C, o);
+      store_pack<T, V>(y + (g.n * D) * C + cl_slab_offset(g, C, u), o);
     }
   }
   if (g.ch_ok && g.slot == 0) {
@@ -1026,8 +1130,8 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
   Pack<T, V> rx[U], rd[U];
   bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D) * C, g, CV, C, rx, ok);
-  cl_load_slab<T, V, U>(dy + (g.n * D) * C, g, CV, C, rd, ok);
+  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+  cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   float mu[V], rs[V], sc[V];
   load_f32<V>(mean_in + g.n * C + g.coff, mu);
   load_f32<V>(rstd_in + g.n * C + g.coff, rs);
@@ -1053,7 +1157,6 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     ca[i] = -sc[i] * (acc[i] * inv_d);
     cb[i] = -sc[i] * (acc[V + i] * inv_d);
   }
-  const int64_t boff = (g.n * D) * C + g.coff;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
     if (ok[u]) {
@@ -1063,7 +1166,7 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
         const float h = (to_f32(rx[u].v[i]) - mu[i]) * rs[i];
         o.v[i] = from_f32<T>(sc[i] * to_f32(rd[u].v[i]) + (ca[i] * h + cb[i]));
       }
-      store_pack<T, V>(dx + boff + (g.slot + static_cast<int64_t>(u) * g.ppb) * C, o);
+      store_pack<T, V>(dx + (g.n * D) * C + cl_slab_offset(g, C, u), o);
     }
   }
   if (g.ch_ok && g.slot == 0) {

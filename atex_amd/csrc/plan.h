@@ -348,7 +348,9 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   const int ppb = 256 / p.TPP;
   const int64_t want = div_up(int64_t(cus) * t.cl_items_per_cu, std::max<int64_t>(N * p.CT, 1));
   const int64_t max_s = std::max<int64_t>(1, D / (int64_t(ppb) * 4));
-  const int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), 4096));
+  // the kernels index the slab partials of an instance ([S][2][C] floats) with 32 bits
+  const int64_t s_cap = std::min<int64_t>(4096, std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / std::max<int64_t>(C, 1)));
+  const int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), s_cap));
   p.slab_len = round_up(div_up(D, S), ppb);
   p.S = static_cast<int>(div_up(D, p.slab_len));
   p.n_work = N * p.S * p.CT;
@@ -357,7 +359,9 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   // registers between its load and its use
   const int64_t per_thread = p.slab_len / ppb;
   const int max_u = bwd ? 8 : 16;
-  for (int u = 4; u <= max_u; u *= 2) {
+  // ... and the elements of a resident slab with 32-bit offsets from its first pixel
+  const bool slab32 = (int64_t(16) * ppb + 1) * C < (int64_t(1) << 32);
+  for (int u = 4; slab32 && u <= max_u; u *= 2) {
     if (per_thread <= u) {
       p.U = u;
       break;
@@ -370,7 +374,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.off_fold = 2 * sect;
   p.fold = p.S > kClFoldAbove && N <= 65535;
   // (the backward holds x and dy: 16 pixels per thread of both measured no better than two stages)
-  if (t.cl_fused && V > 1 && C % V == 0 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
+  if (t.cl_fused && slab32 && V > 1 && C % V == 0 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
     p.fused = true;
     p.fused_u = std::max(1, pow2_ceil(per_thread));
   }
