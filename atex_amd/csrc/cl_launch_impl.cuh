@@ -41,6 +41,9 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   // one workgroup column per instance: the launch's x extent N * 256 must stay below 2^32
   ATEXN_REQUIRE(N < (int64_t(1) << 24), "batch size %lld too large (channels-last limit 2^24 - 1)",
                 (long long)N);
+  // channel tiles of 2048 channels are the launch's z extent
+  ATEXN_REQUIRE(p.CT <= 65535, "channel count %lld too large (channels-last limit 65535 * 2048)",
+                (long long)C);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_FWD(U_, RG_)                                                                  \
   do {                                                                                        \
@@ -117,6 +120,9 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   // one workgroup column per instance: the launch's x extent N * 256 must stay below 2^32
   ATEXN_REQUIRE(N < (int64_t(1) << 24), "batch size %lld too large (channels-last limit 2^24 - 1)",
                 (long long)N);
+  // channel tiles of 2048 channels are the launch's z extent
+  ATEXN_REQUIRE(p.CT <= 65535, "channel count %lld too large (channels-last limit 65535 * 2048)",
+                (long long)C);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
 #define ATEXN_CL_BWD(U_, RG_)                                                                  \
   do {                                                                                        \

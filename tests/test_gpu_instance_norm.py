@@ -259,7 +259,8 @@ def test_channels_last_cooperative_launch_matches_two_stage(coracle, N, C, S, dt
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
-@pytest.mark.parametrize("N,C,S", [(2, 2048, 64), (1, 4096, 40), (3, 520, 300), (2, 96, 5000)])
+@pytest.mark.parametrize("N,C,S", [(2, 2048, 64), (1, 4096, 40), (3, 520, 300), (2, 96, 5000), (1, 1048584, 3),
+                                   (2, 300000, 5)])
 def test_channels_last_wide_channel_counts(capi, coracle, N, C, S, dtype):
     """Few workgroups and thousands of channels: the dgamma / dbeta fold of the second backward
     stage deals its outputs out in chunks of adjacent columns."""
