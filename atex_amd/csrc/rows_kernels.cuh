@@ -77,7 +77,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   constexpr int NE = V * VPT;
   static_assert(!(RAGGED && (EXACT || V == 1)), "ragged rows use the non-exact vector variants");
   // gamma / beta live in registers across rows unless that would exhaust the budget
-  constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 4);
+  constexpr bool GB_REGS = !ROW_AFFINE && (VPT <= 8);
   static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float red_buf[2][2][16];
 

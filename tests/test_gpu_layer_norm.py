@@ -100,7 +100,7 @@ def test_in_place(capi, coracle, N, D, dtype):
 
 @pytest.mark.parametrize("dtype", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("N,D", [(64, 1024), (37, 1000), (5, 8192), (3, 40000), (7, 40003), (2, 300001), (1000, 10),
-                                 (500, 100)])
+                                 (500, 100), (300, 20000), (259, 24577), (11, 32761)])
 def test_unaligned_pointers(capi, coracle, N, D, dtype):
     """Every array starts one element past an aligned address (a slice of a larger tensor):
     the 16-byte accesses of the kernels must not depend on pointer alignment."""
