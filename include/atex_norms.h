@@ -123,7 +123,8 @@ int atexn_layer_norm_bwd_static(int dtype, const void* dy, const void* x, const 
 
 /* Replaces functor::FusedInstanceNorm<GPUDevice,T,U>::operator()
  * (cc/kernels/fused_instance_norm_op.cu:1458-1517). mean / inv_std are [N, C] in both
- * layouts. y may alias x. */
+ * layouts. y may alias x.  Size limits (ATEXN_INVALID_ARGUMENT beyond them): N and C below 2^31;
+ * channels-last also N below 2^24 and C at most 65535 * 2048. */
 size_t atexn_instance_norm_fwd_workspace_bytes(int dtype, int layout, int64_t N, int64_t C,
                                                int64_t D);
 int atexn_instance_norm_fwd(int dtype, int layout, const void* x, const float* gamma,
