@@ -265,3 +265,13 @@ def test_channels_last_wide_channel_counts(capi, coracle, N, C, S, dtype):
     """Few workgroups and thousands of channels: the dgamma / dbeta fold of the second backward
     stage deals its outputs out in chunks of adjacent columns."""
     run_case(capi, coracle, N, C, S, dtype, False, 29)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(16, 256, 8192), (9, 512, 4096), (20, 1024, 3000), (8, 8, 40000), (30, 16, 20000),
+                                   (12, 64, 16 * 1024 + 5)])
+def test_channels_last_slab_fold_paths(capi, coracle, N, C, S, dtype):
+    """The second stage folds the slab partials of its instance with all of a lane's partials in
+    registers (at most 16 per lane) or in batches (more): shapes with one lane per channel and
+    17 .. 64 slabs, with 32 lanes per channel, and with a short last slab."""
+    run_case(capi, coracle, N, C, S, dtype, False, 31)
