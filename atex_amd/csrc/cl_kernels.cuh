@@ -38,6 +38,14 @@ struct ClGeom {
                    //   vector of a C that is not a multiple of V starts at C - V (it overlaps
                    //   its neighbour) and owns only its elements lo .. V-1
   int lo;
+  int lo_out;      // first element of the vector that the thread writes to y / dx: the elements
+                   //   lo_out .. lo - 1 of an overlapping last vector belong to the neighbour,
+                   //   which computes the same bits for them from the same inputs and constants,
+                   //   so both may store the full vector (lo_out = 0); only where the vector
+                   //   reaches into the previous channel tile, whose constants this workgroup
+                   //   does not have, or where the neighbour sits in another wave (in-place
+                   //   calls: that wave may already have overwritten x), the thread keeps to
+                   //   its own elements (lo_out = lo)
   int slot;        // pixel slot inside the block
   int ppb;         // pixel slots per block
   bool ch_ok;      // channel vector inside C
@@ -61,9 +69,11 @@ __device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, i
   if constexpr (RG) {  // C is not a multiple of V (and C >= V)
     g.coff = nominal + V <= C ? nominal : C - V;
     g.lo = g.ch_ok ? nominal - g.coff : 0;
+    g.lo_out = g.coff >= (g.ct << tpp_shift) * V && (t & (kWave - 1)) != 0 ? 0 : g.lo;
   } else {
     g.coff = nominal;
     g.lo = 0;
+    g.lo_out = 0;
   }
   g.p0 = static_cast<int64_t>(g.s) * slab_len;
   g.p1 = g.p0 + slab_len < D ? g.p0 + slab_len : D;
@@ -607,6 +617,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
             Pack<T, V> pk[B];
 #pragma unroll
             for (int u = 0; u < B; ++u) pk[u] = load_pack<T, V>(base + (p + u * step) * C);
+            batch_loaded<T, V, B>(pk);
             float f[B][V];
 #pragma unroll
             for (int u = 0; u < B; ++u) {
@@ -741,14 +752,14 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
     k.load(g, tpp_shift, sm_mean, sm_sc, sm_bt);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& pk, int64_t p) {
-      store_pack_from<T, V>(y + boff + p * C, k.template apply<T>(pk), RG ? g.lo : 0);
+      store_pack_from<T, V>(y + boff + p * C, k.template apply<T>(pk), RG ? g.lo_out : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (ok[u]) {
           store_pack_from<T, V>(y + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
-                                k.template apply<T>(raw[u]), RG ? g.lo : 0);
+                                k.template apply<T>(raw[u]), RG ? g.lo_out : 0);
         }
       }
     } else {
@@ -765,6 +776,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
               q[u] = rev ? flip - (p + u * step) : p + u * step;
               pk[u] = load_pack_last<T, V>(x + boff + q[u] * C);
             }
+            batch_loaded<T, V, B>(pk);
 #pragma unroll
             for (int u = 0; u < B; ++u) apply(pk[u], q[u]);
           },
@@ -828,6 +840,7 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
               px[u] = load_pack<T, V>(x + boff + (p + u * step) * C);
               pd[u] = load_pack<T, V>(dy + boff + (p + u * step) * C);
             }
+            batch_loaded<T, V, B>(px, pd);
 #pragma unroll
             for (int u = 0; u < B; ++u) add(px[u], pd[u]);
           },
@@ -885,14 +898,14 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
     const int64_t boff = (g.n * D) * C + g.coff;
     auto apply = [&](const Pack<T, V>& px, const Pack<T, V>& pd, int64_t p) {
-      store_pack_from<T, V>(dx + boff + p * C, k.template apply<T>(px, pd), RG ? g.lo : 0);
+      store_pack_from<T, V>(dx + boff + p * C, k.template apply<T>(px, pd), RG ? g.lo_out : 0);
     };
     if constexpr (U > 0) {
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         if (okp[u]) {
           store_pack_from<T, V>(dx + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
-                                k.template apply<T>(rx[u], rd[u]), RG ? g.lo : 0);
+                                k.template apply<T>(rx[u], rd[u]), RG ? g.lo_out : 0);
         }
       }
     } else {
@@ -909,6 +922,7 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
               px[u] = load_pack_last<T, V>(x + boff + q[u] * C);
               pd[u] = load_pack_last<T, V>(dy + boff + q[u] * C);
             }
+            batch_loaded<T, V, B>(px, pd);
 #pragma unroll
             for (int u = 0; u < B; ++u) apply(px[u], pd[u], q[u]);
           },
@@ -1051,16 +1065,16 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
 // instance in registers instead of shared memory and an exact two-pass over them (mean, then
 // centred squares) instead of Welford merges.  Grid = (N, 1, channel tiles).
 // y may alias x: a workgroup loads all of its elements before it stores any.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta, T* y,
              float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t D, int C,
              int tpp_shift, float eps) {
   __shared__ float lds[V * kClThreads];
-  const int CV = C / V;
+  const int CV = (C + V - 1) / V;
   const int TPP = 1 << tpp_shift;
   const float inv_d = 1.0f / static_cast<float>(D);
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, D);
   Pack<T, V> raw[U];
   bool ok[U];
   cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
@@ -1104,12 +1118,12 @@ cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restric
       Pack<T, V> o;
 #pragma unroll
       for (int i = 0; i < V; ++i) o.v[i] = from_f32<T>((to_f32(raw[u].v[i]) - mean[i]) * gm[i] + bt[i]);
-      store_pack<T, V>(y + (g.n * D) * C + cl_slab_offset(g, C, u), o);
+      store_pack_from<T, V>(y + (g.n * D) * C + cl_slab_offset(g, C, u), o, RG ? g.lo_out : 0);
     }
   }
   if (g.ch_ok && g.slot == 0) {
-    store_f32<V>(mean_out + g.n * C + g.coff, mean);
-    store_f32<V>(rstd_out + g.n * C + g.coff, rs);
+    store_f32_from<V>(mean_out + g.n * C + g.coff, mean, RG ? g.lo : 0);
+    store_f32_from<V>(rstd_out + g.n * C + g.coff, rs, RG ? g.lo : 0);
   }
 }
 
@@ -1117,17 +1131,17 @@ cl_fwd_fused(const T* x, const float* __restrict__ gamma, const float* __restric
 // sums go to part[n][0][c] = sum dy * xh, part[n][1][c] = sum dy for the column reduction over
 // n that follows; with a single instance they are dgamma / dbeta themselves (out0 / out1 then
 // point at dgamma / dbeta and `stride` is 0).  dx may alias dy.
-template <typename T, int V, int U>
+template <typename T, int V, int U, bool RG>
 __global__ void __launch_bounds__(kClThreads)
 cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in, T* dx,
              float* __restrict__ out0, float* __restrict__ out1, int64_t stride, int64_t D, int C,
              int tpp_shift) {
   __shared__ float lds[2 * V * kClThreads];
-  const int CV = C / V;
+  const int CV = (C + V - 1) / V;
   const int TPP = 1 << tpp_shift;
   const float inv_d = 1.0f / static_cast<float>(D);
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, D);
+  const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, D);
   Pack<T, V> rx[U], rd[U];
   bool ok[U];
   cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
@@ -1166,7 +1180,7 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
         const float h = (to_f32(rx[u].v[i]) - mu[i]) * rs[i];
         o.v[i] = from_f32<T>(sc[i] * to_f32(rd[u].v[i]) + (ca[i] * h + cb[i]));
       }
-      store_pack<T, V>(dx + (g.n * D) * C + cl_slab_offset(g, C, u), o);
+      store_pack_from<T, V>(dx + (g.n * D) * C + cl_slab_offset(g, C, u), o, RG ? g.lo_out : 0);
     }
   }
   if (g.ch_ok && g.slot == 0) {
@@ -1176,8 +1190,8 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
       t0[i] = acc[i];
       t1[i] = acc[V + i];
     }
-    store_f32<V>(out0 + g.n * stride + g.coff, t0);
-    store_f32<V>(out1 + g.n * stride + g.coff, t1);
+    store_f32_from<V>(out0 + g.n * stride + g.coff, t0, RG ? g.lo : 0);
+    store_f32_from<V>(out1 + g.n * stride + g.coff, t1, RG ? g.lo : 0);
   }
 }
 

@@ -68,8 +68,16 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
     if (p.fused) {
       const dim3 fgrid(static_cast<unsigned>(N), 1, p.CT);
 #define ATEXN_CL_FWD_FUSED(U_)                                                                 \
-  cl_fwd_fused<T, V, U_><<<fgrid, kClThreads, 0, st>>>(x, gamma, beta, y, mean, rstd, D, Ci,   \
-                                                        p.tpp_shift, eps)
+  do {                                                                                        \
+    if (C % V != 0)                                                                           \
+      cl_fwd_fused<T, V, U_, true><<<fgrid, kClThreads, 0, st>>>(x, gamma, beta, y, mean,     \
+                                                                  rstd, D, Ci, p.tpp_shift,   \
+                                                                  eps);                       \
+    else                                                                                      \
+      cl_fwd_fused<T, V, U_, false><<<fgrid, kClThreads, 0, st>>>(x, gamma, beta, y, mean,    \
+                                                                   rstd, D, Ci, p.tpp_shift,  \
+                                                                   eps);                      \
+  } while (0)
       switch (p.fused_u) {
         case 1: ATEXN_CL_FWD_FUSED(1); break;
         case 2: ATEXN_CL_FWD_FUSED(2); break;
@@ -95,9 +103,15 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       if (launch_cooperative(fn, grid, kClThreads, args, st)) return ATEXN_OK;
       // refused (the grid cannot be co-resident here): the two-stage kernels below
     }
-    // a channel count that is not a multiple of V: streaming kernels with an overlapping
-    // last channel vector
-    if (C % V != 0) { ATEXN_CL_FWD(0, true); return ATEXN_OK; }
+    // a channel count that is not a multiple of V: the last channel vector of a pixel overlaps
+    // its neighbour and owns only its last C % V elements
+    if (C % V != 0) {
+      if (p.U == 4) { ATEXN_CL_FWD(4, true); return ATEXN_OK; }
+      if (p.U == 8) { ATEXN_CL_FWD(8, true); return ATEXN_OK; }
+      if (p.U == 16) { ATEXN_CL_FWD(16, true); return ATEXN_OK; }
+      ATEXN_CL_FWD(0, true);
+      return ATEXN_OK;
+    }
     if (p.U == 4) { ATEXN_CL_FWD(4, false); return ATEXN_OK; }
     if (p.U == 8) { ATEXN_CL_FWD(8, false); return ATEXN_OK; }
     if (p.U == 16) { ATEXN_CL_FWD(16, false); return ATEXN_OK; }
@@ -150,8 +164,16 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       float* o1 = N == 1 ? dbeta : part + C;
       const int64_t stride = N == 1 ? 0 : 2 * C;
 #define ATEXN_CL_BWD_FUSED(U_)                                                                 \
-  cl_bwd_fused<T, V, U_><<<fgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, dx, o0, o1,   \
-                                                        stride, D, Ci, p.tpp_shift)
+  do {                                                                                        \
+    if (C % V != 0)                                                                           \
+      cl_bwd_fused<T, V, U_, true><<<fgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd,    \
+                                                                  dx, o0, o1, stride, D, Ci,  \
+                                                                  p.tpp_shift);               \
+    else                                                                                      \
+      cl_bwd_fused<T, V, U_, false><<<fgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd,   \
+                                                                   dx, o0, o1, stride, D, Ci, \
+                                                                   p.tpp_shift);              \
+  } while (0)
       switch (p.fused_u) {
         case 1: ATEXN_CL_BWD_FUSED(1); break;
         case 2: ATEXN_CL_BWD_FUSED(2); break;
@@ -175,7 +197,12 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
                                 : reinterpret_cast<const void*>(cl_bwd_coop<T, V, 8>);
       if (launch_cooperative(fn, grid, kClThreads, args, st)) return ATEXN_OK;
     }
-    if (C % V != 0) { ATEXN_CL_BWD(0, true); return ATEXN_OK; }
+    if (C % V != 0) {
+      if (p.U == 4) { ATEXN_CL_BWD(4, true); return ATEXN_OK; }
+      if (p.U == 8) { ATEXN_CL_BWD(8, true); return ATEXN_OK; }
+      ATEXN_CL_BWD(0, true);
+      return ATEXN_OK;
+    }
     if (p.U == 4) { ATEXN_CL_BWD(4, false); return ATEXN_OK; }
     if (p.U == 8) { ATEXN_CL_BWD(8, false); return ATEXN_OK; }
   }

@@ -103,6 +103,53 @@ __device__ __forceinline__ void forget_derived(Pack<T, V>& v) {
   }
 }
 
+// Between the loads of a batch (up to two arrays of N <= 4 vectors, or one of N <= 8) and their
+// first use: one empty asm statement takes every vector of the batch as an operand, so the
+// compiler must have issued all the loads before it and cannot sink a load down to its use
+// (left alone it sometimes emits load, wait, use, load, wait, use, ... and a batch then pays
+// one memory latency per load instead of one per batch).
+template <typename T, int V, int N>
+__device__ __forceinline__ void batch_loaded(Pack<T, V> (&a)[N]) {
+  static_assert(N <= 8, "at most 8 vectors per statement");
+  if constexpr (sizeof(T) * V == 16) {
+    u32x4 b[8];
+#pragma unroll
+    for (int i = 0; i < N; ++i) __builtin_memcpy(&b[i], &a[i], 16);
+#pragma unroll
+    for (int i = N; i < 8; ++i) b[i] = b[0];
+    if constexpr (N <= 1) asm volatile("" : "+v"(b[0]));
+    else if constexpr (N <= 2) asm volatile("" : "+v"(b[0]), "+v"(b[1]));
+    else if constexpr (N <= 4) asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]));
+    else asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7]));
+#pragma unroll
+    for (int i = 0; i < N; ++i) __builtin_memcpy(&a[i], &b[i], 16);
+  }
+}
+template <typename T, int V, int N>
+__device__ __forceinline__ void batch_loaded(Pack<T, V> (&a)[N], Pack<T, V> (&c)[N]) {
+  static_assert(N <= 4, "at most 8 vectors per statement");
+  if constexpr (sizeof(T) * V == 16) {
+    u32x4 b[8];
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      __builtin_memcpy(&b[i], &a[i], 16);
+      __builtin_memcpy(&b[4 + i], &c[i], 16);
+    }
+#pragma unroll
+    for (int i = N; i < 4; ++i) {
+      b[i] = b[0];
+      b[4 + i] = b[4];
+    }
+    if constexpr (N <= 2) asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[4]), "+v"(b[5]));
+    else asm volatile("" : "+v"(b[0]), "+v"(b[1]), "+v"(b[2]), "+v"(b[3]), "+v"(b[4]), "+v"(b[5]), "+v"(b[6]), "+v"(b[7]));
+#pragma unroll
+    for (int i = 0; i < N; ++i) {
+      __builtin_memcpy(&a[i], &b[i], 16);
+      __builtin_memcpy(&c[i], &b[4 + i], 16);
+    }
+  }
+}
+
 // The first cnt (0 <= cnt <= V) elements of a vector; the rest read as zero / are not written.
 // cnt == V takes the single wide access.
 template <typename T, int V>

@@ -374,7 +374,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.off_fold = 2 * sect;
   p.fold = p.S > kClFoldAbove && N <= 65535;
   // (the backward holds x and dy: 16 pixels per thread of both measured no better than two stages)
-  if (t.cl_fused && slab32 && V > 1 && C % V == 0 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
+  if (t.cl_fused && slab32 && V > 1 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
     p.fused = true;
     p.fused_u = std::max(1, pow2_ceil(per_thread));
   }

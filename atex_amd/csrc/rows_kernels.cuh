@@ -129,27 +129,45 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   const int64_t stride = static_cast<int64_t>(gridDim.x) * rpb * RB;
   int64_t row0 = static_cast<int64_t>(blockIdx.x) * rpb * RB;
 
-  auto load_batch = [&](int64_t base, Pack<T, V>(&raw)[RB][VPT]) {
+  // ROW_AFFINE: gamma / beta of a row's channel travel with the row's vectors (fetched at their
+  // point of use, after the two reductions, they would cost a trip to L2 per row)
+  struct RowAffine {
+    float g[ROW_AFFINE ? RB : 1], b[ROW_AFFINE ? RB : 1];
+  };
+  auto load_batch = [&](int64_t base, Pack<T, V>(&raw)[RB][VPT], RowAffine& ra) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
-      const int64_t row = base + r * rpb + slot;
-      const T* xr = x + ((EXACT || row < n_rows) ? row : n_rows - 1) * D;
+      const int64_t row_q = base + r * rpb + slot;
+      const int64_t row = (EXACT || row_q < n_rows) ? row_q : n_rows - 1;
+      const T* xr = x + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) raw[r][k] = load_pack<T, V>(xr + col[k]);
+      if constexpr (ROW_AFFINE) {
+        const int c = static_cast<int>(row % C);
+        ra.g[r] = gamma[c];
+        ra.b[r] = beta[c];
+      }
     }
   };
 
   // prefetching doubles the raw-vector registers; long rows do without it
   constexpr bool PREFETCH = VPT * RB <= 4;
   Pack<T, V> cur[RB][VPT];
-  if (PREFETCH && row0 < n_rows) load_batch(row0, cur);
+  RowAffine cur_ra;
+  if (PREFETCH && row0 < n_rows) load_batch(row0, cur, cur_ra);
   for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
     Pack<T, V> nxt[PREFETCH ? RB : 1][VPT];
+    RowAffine nxt_ra;
     const bool more = PREFETCH && row0 + stride < n_rows;
     if constexpr (PREFETCH) {
-      if (more) load_batch(row0 + stride, nxt);
+      if (more) load_batch(row0 + stride, nxt, nxt_ra);
     } else {
-      load_batch(row0, cur);
+      load_batch(row0, cur, cur_ra);
+      if constexpr (ROW_AFFINE) {
+        // they are needed where the row's vectors are: not to be moved down to their use
+#pragma unroll
+        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur_ra.g[r]), "+v"(cur_ra.b[r]));
+      }
     }
 
     bool row_ok[RB];
@@ -211,11 +229,8 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       const int64_t row = row0 + r * rpb + slot;
       float gs = 1.f, bs = 0.f;
       if constexpr (ROW_AFFINE) {
-        if (row_ok[r]) {
-          const int c = static_cast<int>(row % C);
-          gs = gamma[c] * rstd[r];
-          bs = beta[c];
-        }
+        gs = cur_ra.g[r] * rstd[r];
+        bs = cur_ra.b[r];
       }
       T* yr = y + row * D;
 #pragma unroll
@@ -259,6 +274,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 #pragma unroll
           for (int k = 0; k < VPT; ++k) cur[r][k] = nxt[r][k];
         }
+        cur_ra = nxt_ra;
       }
     }
   }
@@ -344,6 +360,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   struct Batch {
     Pack<T, V> px[RB][VPT], pd[RB][VPT];
     float mean[RB], rstd[RB];
+    float gm[ROW_AFFINE ? RB : 1];  // ROW_AFFINE: gamma of the row's channel, fetched with the row
   };
   auto load_batch = [&](int64_t base, Batch& t) {
 #pragma unroll
@@ -354,6 +371,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       const T* dyr = dy + row * D;
       t.mean[r] = mean_in[row];
       t.rstd[r] = rstd_in[row];
+      if constexpr (ROW_AFFINE) t.gm[r] = gamma[static_cast<int>(row % C)];
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
         t.px[r][k] = load_pack<T, V>(xr + col[k]);
@@ -372,6 +390,11 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       if (more) load_batch(row0 + stride, nxt);
     } else {
       load_batch(row0, cur);
+      if constexpr (ROW_AFFINE) {
+        // needed where the row's vectors are: not to be moved down to its use
+#pragma unroll
+        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur.gm[r]));
+      }
     }
 
     bool row_ok[RB];
@@ -431,7 +454,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       const int64_t row = row0 + r * rpb + slot;
       float scale = cur.rstd[r];
       if constexpr (ROW_AFFINE) {
-        if (row_ok[r]) scale *= gamma[static_cast<int>(row % C)];
+        scale *= cur.gm[r];
         if (row_ok[r] && lane_r == 0) {
           const int64_t n = row / C;
           const int c = static_cast<int>(row % C);
@@ -679,6 +702,7 @@ __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
         Pack<T, V> pk[kSplitBatch];
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u) pk[u] = load_pack<T, V>(p + (v + u * step) * V);
+        batch_loaded<T, V, kSplitBatch>(pk);
         float f[kSplitBatch * V];
 #pragma unroll
         for (int u = 0; u < kSplitBatch; ++u) {
@@ -790,6 +814,7 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
             i[u] = split_pos(v + u * step, n_vec, rev) * V;
             pk[u] = load_pack_last<T, V>(xp + i[u]);
           }
+          batch_loaded<T, V, B>(pk);
 #pragma unroll
           for (int u = 0; u < B; ++u) one(pk[u], i[u]);
         },
@@ -864,6 +889,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
             px[u] = load_pack<T, V>(xp + (v + u * step) * V);
             pd[u] = load_pack<T, V>(dp + (v + u * step) * V);
           }
+          batch_loaded<T, V, B>(px, pd);
 #pragma unroll
           for (int u = 0; u < B; ++u) one(px[u], pd[u], (v + u * step) * V);
         },
@@ -957,6 +983,7 @@ __global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
             px[u] = load_pack_last<T, V>(xp + i[u]);
             pd[u] = load_pack_last<T, V>(dp + i[u]);
           }
+          batch_loaded<T, V, B>(px, pd);
 #pragma unroll
           for (int u = 0; u < B; ++u) one(px[u], pd[u], i[u]);
         },

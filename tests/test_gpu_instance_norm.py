@@ -189,6 +189,12 @@ def test_deterministic(capi):
     (40, 128, 250),    # 16 forward, two stages backward
     (3, 4096, 4),      # two channel tiles
     (5, 520, 31),      # channel vectors not a power of two
+    (600, 12, 20),     # channel counts that are not a multiple of the vector width: the last
+    (64, 100, 64),     #   vector of a pixel overlaps its neighbour
+    (2, 20, 216),
+    (300, 36, 50),
+    (1, 9, 1000),
+    (3, 2051, 7),      # ... with two channel tiles
 ])
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
@@ -269,7 +275,8 @@ def test_channels_last_wide_channel_counts(capi, coracle, N, C, S, dtype):
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("N,C,S", [(16, 256, 8192), (9, 512, 4096), (20, 1024, 3000), (8, 8, 40000), (30, 16, 20000),
-                                   (12, 64, 16 * 1024 + 5)])
+                                   (12, 64, 16 * 1024 + 5), (8, 100, 16384), (64, 100, 4096), (16, 20, 9000),
+                                   (7, 13, 33333)])
 def test_channels_last_slab_fold_paths(capi, coracle, N, C, S, dtype):
     """The second stage folds the slab partials of its instance with all of a lane's partials in
     registers (at most 16 per lane) or in batches (more): shapes with one lane per channel and
