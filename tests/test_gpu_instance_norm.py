@@ -94,6 +94,14 @@ def test_channel_counts(capi, coracle, C, dtype, channel_first):
 def test_in_place(capi, coracle, dtype, channel_first):
     run_case(capi, coracle, 2, 32, 4096, dtype, channel_first, 23, in_place=True)
     run_case(capi, coracle, 1, 8, 300000, dtype, channel_first, 23, in_place=True)
+    # channel counts whose last vector overlaps its neighbour: the neighbour in the same wave
+    # (268 = 33.5 vectors on 64 lanes), in the previous wave (516 = 64.5 vectors on 128 lanes),
+    # streamed and register-resident slabs, single pass
+    run_case(capi, coracle, 3, 268, 500, dtype, channel_first, 23, in_place=True)
+    run_case(capi, coracle, 2, 516, 300, dtype, channel_first, 23, in_place=True)
+    run_case(capi, coracle, 4, 100, 4096, dtype, channel_first, 23, in_place=True)
+    run_case(capi, coracle, 40, 100, 60, dtype, channel_first, 23, in_place=True)
+    run_case(capi, coracle, 2, 516, 40000, dtype, channel_first, 23, in_place=True)
 
 
 @pytest.mark.parametrize("channel_first", [False, True])
