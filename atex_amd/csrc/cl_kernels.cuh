@@ -231,7 +231,7 @@ __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], co
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
-      m2[i] += d * d;
+      m2[i] = __builtin_fmaf(d, d, m2[i]);
     }
   }
   __syncthreads();  // the first sum's LDS reads are done
@@ -258,6 +258,9 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
                                               float* sm_sc, float* sm_bt,
                                               float* __restrict__ mean_out,
                                               float* __restrict__ rstd_out) {
+  // (the kernels that share this fold must produce the same bits from the same partials:
+  // which multiply-adds get fused is not left to the compiler's choice per kernel)
+#pragma clang fp contract(off)
   const FoldMap fm = fold_map(cap);
   const float inv_d = 1.0f / static_cast<float>(D);
   const float n_full = static_cast<float>(cnt_len);
@@ -342,7 +345,7 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
     }
     for (int m = 1; m < fm.P; m <<= 1) m2 += lane_xor(m2, m);
     if (sub == 0 && in) {
-      const float rs = rsqrtf(m2 * inv_d + eps);
+      const float rs = rsqrtf(__builtin_fmaf(m2, inv_d, eps));
       sm_mean[cl] = mean;
       sm_sc[cl] = gm * rs;
       sm_bt[cl] = bt;
@@ -376,8 +379,9 @@ struct ClFwdCoef {
     Pack<T, V> o;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      // subtract the mean first: x * scale - mean * scale would cancel badly when |mean| >> std
-      o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean[i]) * sc[i] + bt[i]);
+      // subtract the mean first: x * scale - mean * scale would cancel badly when |mean| >> std.
+      // (explicit fused multiply-adds: every kernel that applies these constants rounds alike)
+      o.v[i] = from_f32<T>(__builtin_fmaf(to_f32(pk.v[i]) - mean[i], sc[i], bt[i]));
     }
     return o;
   }
@@ -398,7 +402,7 @@ __device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], cons
     for (int i = 0; i < V; ++i) {
       const float d = ok[u] ? to_f32(rd[u].v[i]) : 0.f;
       const float xh = ok[u] ? (to_f32(rx[u].v[i]) - mu[i]) * rs[i] : 0.f;
-      acc[i] += d * xh;
+      acc[i] = __builtin_fmaf(d, xh, acc[i]);
       acc[V + i] += d;
     }
   }
@@ -422,6 +426,7 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
                                              float (*red_buf)[16], float* fold_lds,
                                              float* __restrict__ dgamma,
                                              float* __restrict__ dbeta) {
+#pragma clang fp contract(off)
   const FoldMap fm = fold_map(cap);
   const int c_base = g.ct * cap;
   const int64_t n_blocks = static_cast<int64_t>(gridDim.x) * gridDim.y * gridDim.z;
@@ -497,7 +502,7 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
       float t = 0.f;
 #pragma unroll
       for (int u = 0; u < kEarly; ++u) t += ev[u];
-      t = block_sum1(t, red_buf[0]);
+      t = block_sum1(t, red_buf[0], kClThreads / kWave);
       if (threadIdx.x == 0) (w < C ? dgamma : dbeta)[w < C ? w : w - C] = t;
     }
     __syncthreads();
@@ -543,7 +548,7 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
           for (int u = 0; u < 4; ++u) t += v[u];
         },
         [&](int64_t r) { t += pc[r * W2]; });
-    t = block_sum1(t, red_buf[red_it & 1]);
+    t = block_sum1(t, red_buf[red_it & 1], kClThreads / kWave);
     ++red_it;
     if (threadIdx.x == 0) (o < C ? dgamma : dbeta)[o < C ? o : o - C] = t;
   }
@@ -572,7 +577,7 @@ struct ClBwdCoef {
     Pack<T, V> o;
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      o.v[i] = from_f32<T>(sc[i] * to_f32(pd.v[i]) + (ca[i] * (to_f32(px.v[i]) - mu[i]) + cb[i]));
+      o.v[i] = from_f32<T>(__builtin_fmaf(sc[i], to_f32(pd.v[i]), __builtin_fmaf(ca[i], to_f32(px.v[i]) - mu[i], cb[i])));
     }
     return o;
   }

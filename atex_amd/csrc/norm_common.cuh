@@ -46,9 +46,20 @@ struct F32x4 {
   float v[4];
 };
 
+// (16 bytes are loaded as ONE vector value and then viewed as elements: loaded as a struct of
+// elements, the optimiser may cut the access into per-element pieces when the value travels
+// through a loop-carried copy, and reassemble them into 2- and 4-byte loads.)
 template <typename T, int V>
 __device__ __forceinline__ Pack<T, V> load_pack(const T* p) {
-  return *reinterpret_cast<const Pack<T, V>*>(p);
+  if constexpr (sizeof(T) * V == 16) {
+    using u32x4_u = typename Bits16<sizeof(T)>::type;
+    const u32x4 bits = *reinterpret_cast<const u32x4_u*>(p);
+    Pack<T, V> r;
+    __builtin_memcpy(&r, &bits, 16);
+    return r;
+  } else {
+    return *reinterpret_cast<const Pack<T, V>*>(p);
+  }
 }
 // The last read of an input by the second stage of a two-stage kernel: the non-temporal hint
 // keeps these lines from displacing what is still to be read (measured: 0-3 % off the
@@ -366,12 +377,21 @@ __device__ __forceinline__ Wf group_wf(Wf w) {
   return w;
 }
 
-// Block-wide Welford all-reduce for blocks that are a whole number of waves.  `buf`
-// must hold 16 Wf entries and be private to this call until the block has passed
+// blockDim.x, read once and made opaque to the compiler.  Kernels call it at their start and
+// hand the value (or the wave count) to the helpers below: left to itself the compiler may
+// re-read the block size from the dispatch packet inside a loop, a memory load whose wait also
+// waits for every prefetch issued before it.
+__device__ __forceinline__ int block_threads() {
+  int n = static_cast<int>(blockDim.x);
+  asm volatile("" : "+s"(n));
+  return n;
+}
+
+// Block-wide Welford all-reduce for blocks that are a whole number of waves (nw of them).
+// `buf` must hold 16 Wf entries and be private to this call until the block has passed
 // another barrier (callers alternate between two buffers).
-__device__ __forceinline__ Wf block_wf(Wf w, Wf* buf) {
+__device__ __forceinline__ Wf block_wf(Wf w, Wf* buf, int nw) {
   w = group_wf<kWave>(w);
-  const int nw = blockDim.x / kWave;
   if (nw == 1) return w;
   const int wave = threadIdx.x / kWave;
   if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = w;
@@ -382,10 +402,9 @@ __device__ __forceinline__ Wf block_wf(Wf w, Wf* buf) {
 }
 
 // Block-wide all-reduce of two sums, same contract as block_wf (`buf` holds 16 float2).
-__device__ __forceinline__ float2 block_sum2(float a, float b, float2* buf) {
+__device__ __forceinline__ float2 block_sum2(float a, float b, float2* buf, int nw) {
   a = group_sum<kWave>(a);
   b = group_sum<kWave>(b);
-  const int nw = blockDim.x / kWave;
   if (nw == 1) return make_float2(a, b);
   const int wave = threadIdx.x / kWave;
   if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = make_float2(a, b);
@@ -419,9 +438,8 @@ __device__ __forceinline__ float2 wavegroup_sum2(float a, float b, float2* buf) 
 }
 
 // Block-wide all-reduce of one sum, same contract (`buf` holds 16 floats).
-__device__ __forceinline__ float block_sum1(float a, float* buf) {
+__device__ __forceinline__ float block_sum1(float a, float* buf, int nw) {
   a = group_sum<kWave>(a);
-  const int nw = blockDim.x / kWave;
   if (nw == 1) return a;
   const int wave = threadIdx.x / kWave;
   if ((threadIdx.x & (kWave - 1)) == 0) buf[wave] = a;

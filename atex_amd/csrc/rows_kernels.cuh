@@ -24,8 +24,9 @@ namespace atexn {
 // by 2 or 4 consecutive waves.  TPR == 0: the whole block owns one row.
 template <int TPR>
 struct RowMap {
-  __device__ __forceinline__ static int tpr() { return TPR ? TPR : static_cast<int>(blockDim.x); }
-  __device__ __forceinline__ static int rows_per_block() { return TPR ? static_cast<int>(blockDim.x) / TPR : 1; }
+  // bdim: the block size (block_threads())
+  __device__ __forceinline__ static int tpr(int bdim) { return TPR ? TPR : bdim; }
+  __device__ __forceinline__ static int rows_per_block(int bdim) { return TPR ? bdim / TPR : 1; }
   __device__ __forceinline__ static int lane_in_row() {
     return TPR ? static_cast<int>(threadIdx.x) % TPR : static_cast<int>(threadIdx.x);
   }
@@ -81,8 +82,10 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   static_assert(TPR != 0 || RB == 1, "row batching is for rows that fit one wave");
   __shared__ float red_buf[2][2][16];
 
-  const int tpr = M::tpr();
-  const int rpb = M::rows_per_block();
+  const int bdim = block_threads();
+  const int n_waves = bdim / kWave;
+  const int tpr = M::tpr(bdim);
+  const int rpb = M::rows_per_block(bdim);
   const int lane_r = M::lane_in_row();
   const int slot = M::slot();
   const int64_t D = d_elems;
@@ -152,24 +155,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 
   // prefetching doubles the raw-vector registers; long rows do without it
   constexpr bool PREFETCH = VPT * RB <= 4;
-  Pack<T, V> cur[RB][VPT];
-  RowAffine cur_ra;
-  if (PREFETCH && row0 < n_rows) load_batch(row0, cur, cur_ra);
-  for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
-    Pack<T, V> nxt[PREFETCH ? RB : 1][VPT];
-    RowAffine nxt_ra;
-    const bool more = PREFETCH && row0 + stride < n_rows;
-    if constexpr (PREFETCH) {
-      if (more) load_batch(row0 + stride, nxt, nxt_ra);
-    } else {
-      load_batch(row0, cur, cur_ra);
-      if constexpr (ROW_AFFINE) {
-        // they are needed where the row's vectors are: not to be moved down to their use
-#pragma unroll
-        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur_ra.g[r]), "+v"(cur_ra.b[r]));
-      }
-    }
-
+  auto process = [&](Pack<T, V>(&cur)[RB][VPT], const RowAffine& cur_ra, int64_t row0, int it) {
     bool row_ok[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
@@ -195,7 +181,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       if constexpr (TPR != 0) {
         mean[r] = group_sum<(TPR ? TPR : 1)>(mean[r]) * inv_d;
       } else {
-        mean[r] = block_sum1(mean[r], red_buf[it & 1][0]) * inv_d;
+        mean[r] = block_sum1(mean[r], red_buf[it & 1][0], n_waves) * inv_d;
       }
     }
     // stage 2: centre (exact second pass over registers), sum of squares
@@ -219,7 +205,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       if constexpr (TPR != 0) {
         q = group_sum<(TPR ? TPR : 1)>(rstd[r]);
       } else {
-        q = block_sum1(rstd[r], red_buf[it & 1][1]);
+        q = block_sum1(rstd[r], red_buf[it & 1][1], n_waves);
       }
       rstd[r] = rsqrtf(q * inv_d + eps);
     }
@@ -267,7 +253,44 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
         rstd_out[row] = rstd[r];
       }
     }
-    if constexpr (PREFETCH) {
+  };
+  // Two shapes of the prefetching loop.  PEELED: a loop that always requests the next batch and
+  // the last batch after it; otherwise the request sits under a condition inside one loop, and
+  // the waits behind it, which must assume that it was not made, also wait for the next batch
+  // before the current one is finished.  Which is faster is a matter of measurement per
+  // variant (rows on lane groups: peeled, [262144, 128] forward 25.8 -> 21.6 us; a workgroup per
+  // row: not peeled, [16384, 4096] forward 43.8 against 62.5 us peeled).
+  constexpr bool PEELED = TPR != 0;
+  if constexpr (PREFETCH && PEELED) {
+    if (row0 < n_rows) {
+      Pack<T, V> cur[RB][VPT];
+      RowAffine cur_ra;
+      load_batch(row0, cur, cur_ra);
+      int it = 0;
+      for (; row0 + stride < n_rows; row0 += stride, ++it) {
+        Pack<T, V> nxt[RB][VPT];
+        RowAffine nxt_ra;
+        load_batch(row0 + stride, nxt, nxt_ra);
+        process(cur, cur_ra, row0, it);
+#pragma unroll
+        for (int r = 0; r < RB; ++r) {
+#pragma unroll
+          for (int k = 0; k < VPT; ++k) cur[r][k] = nxt[r][k];
+        }
+        cur_ra = nxt_ra;
+      }
+      process(cur, cur_ra, row0, it);
+    }
+  } else if constexpr (PREFETCH) {
+    Pack<T, V> cur[RB][VPT];
+    RowAffine cur_ra;
+    if (row0 < n_rows) load_batch(row0, cur, cur_ra);
+    for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+      Pack<T, V> nxt[RB][VPT];
+      RowAffine nxt_ra;
+      const bool more = row0 + stride < n_rows;
+      if (more) load_batch(row0 + stride, nxt, nxt_ra);
+      process(cur, cur_ra, row0, it);
       if (more) {
 #pragma unroll
         for (int r = 0; r < RB; ++r) {
@@ -276,6 +299,18 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
         }
         cur_ra = nxt_ra;
       }
+    }
+  } else {
+    for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+      Pack<T, V> cur[RB][VPT];
+      RowAffine cur_ra;
+      load_batch(row0, cur, cur_ra);
+      if constexpr (ROW_AFFINE) {
+        // they are needed where the row's vectors are: not to be moved down to their use
+#pragma unroll
+        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur_ra.g[r]), "+v"(cur_ra.b[r]));
+      }
+      process(cur, cur_ra, row0, it);
     }
   }
 }
@@ -314,8 +349,10 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   // LayerNorm only: min(waves / 2, kFoldWaves) * 2 * NE * 64 floats
   extern __shared__ float fold_buf[];
 
-  const int tpr = M::tpr();
-  const int rpb = M::rows_per_block();
+  const int bdim = block_threads();
+  const int n_waves = bdim / kWave;
+  const int tpr = M::tpr(bdim);
+  const int rpb = M::rows_per_block(bdim);
   const int lane_r = M::lane_in_row();
   const int slot = M::slot();
   const int64_t D = d_elems;
@@ -381,22 +418,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   };
 
   constexpr bool PREFETCH = VPT * RB <= 2;
-  Batch cur;
-  if (PREFETCH && row0 < n_rows) load_batch(row0, cur);
-  for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
-    Batch nxt;
-    const bool more = PREFETCH && row0 + stride < n_rows;
-    if constexpr (PREFETCH) {
-      if (more) load_batch(row0 + stride, nxt);
-    } else {
-      load_batch(row0, cur);
-      if constexpr (ROW_AFFINE) {
-        // needed where the row's vectors are: not to be moved down to its use
-#pragma unroll
-        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur.gm[r]));
-      }
-    }
-
+  auto process = [&](Batch& cur, int64_t row0, int it) {
     bool row_ok[RB];
 #pragma unroll
     for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
@@ -443,7 +465,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
         s1[r] = group_sum<(TPR && TPR <= kWave ? TPR : 1)>(s1[r]);
         s2[r] = group_sum<(TPR && TPR <= kWave ? TPR : 1)>(s2[r]);
       } else {
-        const float2 t = block_sum2(s1[r], s2[r], sum_buf[it & 1]);
+        const float2 t = block_sum2(s1[r], s2[r], sum_buf[it & 1], n_waves);
         s1[r] = t.x;
         s2[r] = t.y;
       }
@@ -481,8 +503,44 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
         }
       }
     }
-    if constexpr (PREFETCH) {
+  };
+  // (the two shapes of the prefetching loop: see the forward kernel.  Here a workgroup per row
+  // and rows on several waves are faster peeled, [16384, 4096] 81.9 -> 76.6 us, [8192, 2048]
+  // 26.6 -> 22.7 us; rows on lane groups are not, [262144, 128] 42.5 against 45.3 us.)
+  constexpr bool PEELED = TPR == 0 || TPR > kWave;
+  if constexpr (PREFETCH && PEELED) {
+    if (row0 < n_rows) {
+      Batch cur;
+      load_batch(row0, cur);
+      int it = 0;
+      for (; row0 + stride < n_rows; row0 += stride, ++it) {
+        Batch nxt;
+        load_batch(row0 + stride, nxt);
+        process(cur, row0, it);
+        cur = nxt;
+      }
+      process(cur, row0, it);
+    }
+  } else if constexpr (PREFETCH) {
+    Batch cur;
+    if (row0 < n_rows) load_batch(row0, cur);
+    for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+      Batch nxt;
+      const bool more = row0 + stride < n_rows;
+      if (more) load_batch(row0 + stride, nxt);
+      process(cur, row0, it);
       if (more) cur = nxt;
+    }
+  } else {
+    for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
+      Batch cur;
+      load_batch(row0, cur);
+      if constexpr (ROW_AFFINE) {
+        // needed where the row's vectors are: not to be moved down to its use
+#pragma unroll
+        for (int r = 0; r < RB; ++r) asm volatile("" : "+v"(cur.gm[r]));
+      }
+      process(cur, row0, it);
     }
   }
 
@@ -523,7 +581,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       // 2) fold waves pairwise through LDS: upper half writes, lower half adds
       const int lane = threadIdx.x & (kWave - 1);
       const int wave = threadIdx.x / kWave;
-      const int nw = blockDim.x / kWave;
+      const int nw = n_waves;
       // (at most kFoldWaves waves' worth of LDS is used per step); waves w and w + half own
       // the same columns as long as half is a multiple of the waves per row
       constexpr int WPG = TPR > kWave ? TPR / kWave : 1;
@@ -678,6 +736,7 @@ col_reduce(const float* __restrict__ part, float* __restrict__ out0, float* __re
 // tail is what the memory-side cache still holds when stage 2 starts.
 
 constexpr int kSplitBatch = 4;
+constexpr int kSplitThreads = 256;  // block size of every split_* launch
 
 // Vector index of virtual position p of a chunk of n_vec vectors.
 __device__ __forceinline__ int64_t split_pos(int64_t p, int64_t n_vec, bool rev) {
@@ -694,10 +753,10 @@ __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
   const int64_t n_vec = len / V;
   const int rem = static_cast<int>(len % V);  // only the last chunk of a ragged row
   const int64_t tid = threadIdx.x;
-  const bool has_tail = rem != 0 && n_vec % blockDim.x == tid;
+  const bool has_tail = rem != 0 && n_vec % kSplitThreads == tid;
   Wf w{0.f, 0.f, 0.f};
   batched_for<kSplitBatch>(
-      tid, n_vec, blockDim.x,
+      tid, n_vec, kSplitThreads,
       [&](int64_t v, int64_t step) {
         Pack<T, V> pk[kSplitBatch];
 #pragma unroll
@@ -726,7 +785,7 @@ __device__ __forceinline__ Wf chunk_wf(const T* p, int64_t len) {
 
 // stage 1 forward: stats[w] = (mean, m2) of chunk w; the count follows from geometry.
 template <typename T, int V>
-__global__ void split_fwd_stats(const T* __restrict__ x, float2* __restrict__ stats,
+__global__ void __launch_bounds__(kSplitThreads) split_fwd_stats(const T* __restrict__ x, float2* __restrict__ stats,
                                 int64_t n_rows, int64_t D, int S, int64_t chunk) {
   __shared__ Wf wf_buf[2][16];
   const int64_t n_work = n_rows * S;
@@ -737,7 +796,7 @@ __global__ void split_fwd_stats(const T* __restrict__ x, float2* __restrict__ st
     const int64_t beg = static_cast<int64_t>(s) * chunk;
     const int64_t len = (beg + chunk <= D ? chunk : D - beg);
     Wf r = chunk_wf<T, V>(x + row * D + beg, len);
-    r = block_wf(r, wf_buf[it & 1]);
+    r = block_wf(r, wf_buf[it & 1], kSplitThreads / kWave);
     if (threadIdx.x == 0) stats[w] = make_float2(r.mean, r.m2);
   }
 }
@@ -757,7 +816,7 @@ __device__ __forceinline__ Wf merge_chunks(const float2* stats, int S, int64_t D
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads its vectors of a batch before it writes the same vectors.
 template <typename T, int V, bool ROW_AFFINE>
-__global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
+__global__ void __launch_bounds__(kSplitThreads) split_fwd_apply(const T* x, const float2* __restrict__ stats,
                                 const float* __restrict__ gamma, const float* __restrict__ beta,
                                 T* y, float* __restrict__ mean_out,
                                 float* __restrict__ rstd_out, int64_t n_rows, int64_t D, int S,
@@ -805,7 +864,7 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
       store_pack<T, V>(yp + i, o);
     };
     batched_for<B>(
-        threadIdx.x, n_vec, blockDim.x,
+        threadIdx.x, n_vec, kSplitThreads,
         [&](int64_t v, int64_t step) {
           Pack<T, V> pk[B];
           int64_t i[B];
@@ -824,7 +883,7 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
         });
     // ragged row end (last chunk only): the elements after the last full vector
     const int rem = static_cast<int>(len % V);
-    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+    if (rem != 0 && n_vec % kSplitThreads == threadIdx.x) {
       const int64_t i = n_vec * V;
       Pack<T, V> o;
       const Pack<T, V> pk = load_pack_n<T, V>(xp + i, rem);
@@ -846,7 +905,7 @@ __global__ void split_fwd_apply(const T* x, const float2* __restrict__ stats,
 // stage 1 backward: sums[w] = (sum g, sum g * xh) over chunk w, g = dy * gamma
 // (ROW_AFFINE: (sum dy, sum dy * xh), gamma applied in stage 2).
 template <typename T, int V, bool ROW_AFFINE>
-__global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
+__global__ void __launch_bounds__(kSplitThreads) split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
                                const float* __restrict__ gamma,
                                const float* __restrict__ mean_in,
                                const float* __restrict__ rstd_in, float2* __restrict__ sums,
@@ -881,7 +940,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
       }
     };
     batched_for<B>(
-        threadIdx.x, n_vec, blockDim.x,
+        threadIdx.x, n_vec, kSplitThreads,
         [&](int64_t v, int64_t step) {
           Pack<T, V> px[B], pd[B];
 #pragma unroll
@@ -895,7 +954,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
         },
         [&](int64_t v) { one(load_pack<T, V>(xp + v * V), load_pack<T, V>(dp + v * V), v * V); });
     const int rem = static_cast<int>(len % V);
-    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+    if (rem != 0 && n_vec % kSplitThreads == threadIdx.x) {
       // zero-filled dy beyond the row end adds nothing
       const int64_t i = n_vec * V;
       const Pack<T, V> px = load_pack_n<T, V>(xp + i, rem);
@@ -911,7 +970,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
         s2 += gv * xc;
       }
     }
-    const float2 r = block_sum2(s1, s2 * rstd, sum_buf[it & 1]);
+    const float2 r = block_sum2(s1, s2 * rstd, sum_buf[it & 1], kSplitThreads / kWave);
     if (threadIdx.x == 0) sums[w] = r;
   }
 }
@@ -919,7 +978,7 @@ __global__ void split_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x
 // stage 2 backward: merge the row's chunk sums, write dx for the chunk.  ROW_AFFINE also
 // writes the per-(n, c) sums into `part` (layout as in rows_bwd_resident).
 template <typename T, int V, bool ROW_AFFINE>
-__global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
+__global__ void __launch_bounds__(kSplitThreads) split_bwd_apply(const T* dy, const T* __restrict__ x,
                                 const float* __restrict__ gamma,
                                 const float* __restrict__ mean_in,
                                 const float* __restrict__ rstd_in,
@@ -973,7 +1032,7 @@ __global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
       store_pack<T, V>(op + i, o);
     };
     batched_for<B>(
-        threadIdx.x, n_vec, blockDim.x,
+        threadIdx.x, n_vec, kSplitThreads,
         [&](int64_t v, int64_t step) {
           Pack<T, V> px[B], pd[B];
           int64_t i[B];
@@ -992,7 +1051,7 @@ __global__ void split_bwd_apply(const T* dy, const T* __restrict__ x,
           one(load_pack_last<T, V>(xp + i), load_pack_last<T, V>(dp + i), i);
         });
     const int rem = static_cast<int>(len % V);
-    if (rem != 0 && n_vec % blockDim.x == threadIdx.x) {
+    if (rem != 0 && n_vec % kSplitThreads == threadIdx.x) {
       const int64_t i = n_vec * V;
       const Pack<T, V> px = load_pack_n<T, V>(xp + i, rem);
       const Pack<T, V> pd = load_pack_n<T, V>(dp + i, rem);

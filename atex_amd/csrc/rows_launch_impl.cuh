@@ -130,9 +130,9 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   }
   if constexpr (AFF && V > 1) {
     float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
-    split_fwd_stats<T, V><<<p.split_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
+    split_fwd_stats<T, V><<<p.split_grid, kSplitThreads, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
     ATEXN_CHECK_LAUNCH("split_fwd_stats");
-    split_fwd_apply<T, V, true><<<p.split_grid, 256, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
+    split_fwd_apply<T, V, true><<<p.split_grid, kSplitThreads, 0, st>>>(x, stats, gamma, beta, y, mean, rstd,
                                                              n_rows, D, p.S, p.chunk, C, eps,
                                                              tuning().reverse_second_pass);
     ATEXN_CHECK_LAUNCH("split_fwd_apply");
@@ -192,7 +192,7 @@ int tiles_fwd(const T* x, const float* gamma, const float* beta, int64_t n_rows,
   ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
-  split_fwd_stats<T, V><<<p.stats_grid, 256, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
+  split_fwd_stats<T, V><<<p.stats_grid, kSplitThreads, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
   ATEXN_CHECK_LAUNCH("split_fwd_stats");
   merge_row_stats<4><<<static_cast<unsigned>(div_up(n_rows, 4)), 256, 0, st>>>(stats, mean, rstd, n_rows,
                                                                         D, p.S, p.chunk, eps);
@@ -261,10 +261,10 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   }
   if constexpr (AFF && V > 1) {
     float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
-    split_bwd_sums<T, V, true><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
+    split_bwd_sums<T, V, true><<<p.split_grid, kSplitThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
                                                             D, p.S, p.chunk);
     ATEXN_CHECK_LAUNCH("split_bwd_sums");
-    split_bwd_apply<T, V, true><<<p.split_grid, 256, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
+    split_bwd_apply<T, V, true><<<p.split_grid, kSplitThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, dx,
                                                              part, n_rows, D, p.S, p.chunk, C,
                                                              tuning().reverse_second_pass);
     ATEXN_CHECK_LAUNCH("split_bwd_apply");
