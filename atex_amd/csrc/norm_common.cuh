@@ -377,15 +377,13 @@ __device__ __forceinline__ Wf group_wf(Wf w) {
   return w;
 }
 
-// blockDim.x, read once and made opaque to the compiler.  Kernels call it at their start and
-// hand the value (or the wave count) to the helpers below: left to itself the compiler may
-// re-read the block size from the dispatch packet inside a loop, a memory load whose wait also
-// waits for every prefetch issued before it.
-__device__ __forceinline__ int block_threads() {
-  int n = static_cast<int>(blockDim.x);
-  asm volatile("" : "+s"(n));
-  return n;
-}
+// blockDim.x.  Kernels read it once at their start and hand the value (or the wave count) to the
+// helpers below, so that no helper called inside a loop reads the block size itself: such a read
+// can end up as a load from the dispatch packet in the loop, whose wait also waits for every
+// prefetch issued before it.  (Hiding the value from the optimiser behind an empty asm
+// statement, to rule that out entirely, cost the block-per-row forward 10-20 %: the compiler
+// uses what it knows about the block size.)
+__device__ __forceinline__ int block_threads() { return static_cast<int>(blockDim.x); }
 
 // Block-wide Welford all-reduce for blocks that are a whole number of waves (nw of them).
 // `buf` must hold 16 Wf entries and be private to this call until the block has passed
