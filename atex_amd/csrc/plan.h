@@ -32,7 +32,7 @@ struct Tuning {
   TuneInt cl_items_per_cu{2};        // channels-last: (n, slab, tile) work items per CU
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
-  TuneInt bwd_rows_batch{1};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
+  TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
   TuneInt reverse_second_pass{1};
@@ -189,7 +189,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     } else {
       p.threads = 256;
       if (V > 1 && (!p.ragged || p.vpt == 1)) {
-        p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch : t.bwd_rows_batch;
+        // backward: two rows per batch pay for rows of one vector per lane (D <= 512 halves:
+        // 85 -> 89 % of the streaming rate); with more vectors per lane they cost registers
+        // and measured slower
+        p.rb = kind == RowsKind::kFwd ? t.fwd_rows_batch.load() : (p.vpt == 1 ? t.bwd_rows_batch.load() : 1);
       }
       if (kind == RowsKind::kBwdCols) {
         // bigger blocks -> fewer partial rows for the column reduction

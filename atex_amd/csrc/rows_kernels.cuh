@@ -417,7 +417,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
     }
   };
 
-  constexpr bool PREFETCH = VPT * RB <= 2;
+  constexpr bool PREFETCH = VPT * RB <= (TPR == 0 ? 2 : 4);
   auto process = [&](Batch& cur, int64_t row0, int it) {
     bool row_ok[RB];
 #pragma unroll
