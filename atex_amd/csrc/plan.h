@@ -109,6 +109,9 @@ struct RowsRoute {
   bool tiles = false;
   bool small = false;
 };
+// LDS of the LayerNorm backward's fold: same constants as rows_kernels.cuh
+constexpr int kPlanFoldLdsBytes = 64 * 1024;
+constexpr int kPlanFoldMaxWaves = 8;
 constexpr int kPlanSmallMaxVec = 4;
 constexpr int64_t kPlanSmallMinRows = 4096;
 inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, int64_t D) {
@@ -217,7 +220,15 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.part_rows = p.grid;
       p.off_part = 0;
       p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
-      if (p.tpr != 0) p.fold_lds = size_t(std::min(waves / 2, 4)) * 2 * size_t(V * p.vpt) * 64 * sizeof(float);
+      if (p.tpr != 0) {
+        // the fold of the waves' dgamma / dbeta sums (rows_bwd_resident): waves x groups per
+        // pass x lanes with sums x floats per group
+        const int w = V % 4 == 0 ? 4 : 1;
+        const int lr = std::min(p.tpr, 64);
+        const int q = 2 * V * p.vpt / w;
+        const int cap = kPlanFoldLdsBytes / (kPlanFoldMaxWaves * lr * w * 4);
+        p.fold_lds = size_t(waves) * size_t(std::min(q, cap)) * lr * w * sizeof(float);
+      }
     } else if (kind == RowsKind::kBwdAffine) {
       p.part_rows = static_cast<int>(n_rows / C);
       p.off_part = 0;

@@ -10,6 +10,9 @@
 
 namespace atexn {
 
+static_assert(kFoldLdsBytes == kPlanFoldLdsBytes && kFoldMaxWaves == kPlanFoldMaxWaves,
+              "the planner sizes the fold's LDS with the kernels' constants");
+
 template <typename T, int V, bool AFF>
 using FwdResidentFn = void (*)(const T*, const float*, const float*, T*, float*, float*, int64_t,
                                int, int, float);

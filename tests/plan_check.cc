@@ -98,9 +98,12 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
       EXPECT(p.ws_bytes >= sizeof(float) * 2 * size_t(D) * size_t(p.grid), "partial rows workspace");
       const int waves = p.threads / 64;
       if (p.tpr != 0) {
-        EXPECT(waves == 4 || waves == 8, "fold expects 4 or 8 waves, got %d", waves);
-        EXPECT(p.fold_lds >= size_t(std::min(waves / 2, 4)) * 2 * size_t(r.V * p.vpt) * 64 * sizeof(float), "fold_lds");
-        EXPECT(p.fold_lds <= 64 * 1024, "fold_lds=%zu", p.fold_lds);
+        EXPECT(waves <= kPlanFoldMaxWaves && waves % std::max(1, p.tpr / 64) == 0, "fold: %d waves, %d lanes per row", waves, p.tpr);
+        const int w = r.V % 4 == 0 ? 4 : 1, lr = std::min(p.tpr, 64), q = 2 * r.V * p.vpt / w;
+        const int per_pass = std::min(q, kPlanFoldLdsBytes / (kPlanFoldMaxWaves * lr * w * 4));
+        EXPECT(per_pass >= 1 && (2 * r.V * p.vpt) % w == 0, "fold groups");
+        EXPECT(p.fold_lds == size_t(waves) * per_pass * lr * w * sizeof(float), "fold_lds=%zu", p.fold_lds);
+        EXPECT(p.fold_lds <= size_t(kPlanFoldLdsBytes), "fold_lds=%zu", p.fold_lds);
       }
     } else if (kind == RowsKind::kBwdAffine) {
       EXPECT(n_rows % C == 0 && p.part_rows == n_rows / C, "affine part rows");
