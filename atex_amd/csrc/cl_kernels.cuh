@@ -18,6 +18,8 @@
 
 #include <hip/hip_cooperative_groups.h>
 
+#include <type_traits>
+
 #include "norm_common.cuh"
 
 namespace atexn {
@@ -151,7 +153,8 @@ __device__ __forceinline__ void cl_block_sum(float (&v)[K], float* lds, int TPP)
 // How the threads of a block split the fold over S partial rows for the channels of a
 // tile of `cap` channels (cap = TPP * V, a power of two): P adjacent lanes per channel
 // when the tile has at most 256 channels, else one lane per channel and several sweeps.
-// Slab partials per lane up to which a fold keeps all of them in registers.
+// Slab partials per lane up to which a fold keeps all of them in registers: kClFoldRegs, or
+// twice that by a second variant of the code.
 constexpr int kClFoldRegs = 16;
 
 // base[at], or 0 when the position is not the lane's (the load itself is unconditional and
@@ -251,6 +254,7 @@ __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], co
 // round trip) and leaves the constants of y = (x - sm_mean) * sm_sc + sm_bt in LDS, so that no
 // thread of the apply phase loads anything but x.  The caller synchronises the block before it
 // reads them.
+template <bool WIDE>
 __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& g, int S,
                                               int64_t cnt_len, int64_t D, int C, int cap,
                                               float eps, const float* __restrict__ gamma,
@@ -282,32 +286,40 @@ __device__ __forceinline__ void cl_fold_stats(const float* pstat, const ClGeom& 
       gm = gamma[c];
       bt = beta[c];
     }
-    constexpr int B = 8;
-    constexpr int R = kClFoldRegs;
+    constexpr int B = 16;
     float s1 = 0.f, m2 = 0.f, mean;
-    if (uS <= R * P) {
-      // few slabs per lane: all of a lane's (mean, m2) pairs are loaded at once, one memory
-      // round trip for both sweeps (a lane without a slab in a position reads slab 0 and
-      // weighs it 0); same order of additions as the general path below
-      float tm[R], tq[R], tn[R];
+    // few slabs per lane (at most R): all of a lane's (mean, m2) pairs are loaded at once, one
+    // memory round trip for both sweeps (a lane without a slab in a position reads slab 0 and
+    // weighs it 0); same order of additions as the general path below
+    auto from_registers = [&](auto rc) {
+      constexpr int R = decltype(rc)::value;
+      float tm[R], tq[R];
+      auto weight = [&](int u) {
+        const unsigned sl = sub + u * P;
+        return !(in && sl < uS) ? 0.f : (sl == uS - 1 ? n_last : n_full);
+      };
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         const unsigned sl = sub + u * P;
-        const bool ok = in && sl < uS;
-        const unsigned at = ok ? sl : 0u;
+        const unsigned at = in && sl < uS ? sl : 0u;
         tm[u] = q[(at * 2) * uC + cc];
         tq[u] = q[(at * 2 + 1) * uC + cc];
-        tn[u] = !ok ? 0.f : (sl == uS - 1 ? n_last : n_full);
       }
 #pragma unroll
-      for (int u = 0; u < R; ++u) s1 += tm[u] * tn[u];
+      for (int u = 0; u < R; ++u) s1 += tm[u] * weight(u);
       for (int m = 1; m < fm.P; m <<= 1) s1 += lane_xor(s1, m);
       mean = s1 * inv_d;
 #pragma unroll
       for (int u = 0; u < R; ++u) {
         const float d = tm[u] - mean;
-        m2 += tn[u] == 0.f ? 0.f : tq[u] + tn[u] * (d * d);
+        const float tn = weight(u);
+        m2 += tn == 0.f ? 0.f : tq[u] + tn * (d * d);
       }
+    };
+    if (uS <= kClFoldRegs * P) {
+      from_registers(std::integral_constant<int, kClFoldRegs>{});
+    } else if (WIDE && uS <= 2 * kClFoldRegs * P) {
+      from_registers(std::integral_constant<int, WIDE ? 2 * kClFoldRegs : 1>{});
     } else {
       if (in) {
         for (unsigned sl = sub; sl < uS; sl += B * P) {
@@ -417,6 +429,7 @@ __device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], cons
 // produces the block's share of dgamma / dbeta: output o (o < C: dgamma[o], else dbeta[o - C])
 // is the sum of one column of all N * S partial rows (fixed order, no atomics); block w of the
 // grid takes outputs w, w + #blocks, ...  Ends with a block-wide barrier.  fold_lds: 256 floats.
+template <bool WIDE>
 __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g, int64_t N, int S,
                                              int C, int cap, float inv_d,
                                              const float* __restrict__ gamma,
@@ -425,7 +438,7 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
                                              float* sm_sc, float* sm_ca, float* sm_cb,
                                              float (*red_buf)[16], float* fold_lds,
                                              float* __restrict__ dgamma,
-                                             float* __restrict__ dbeta) {
+                                             float* __restrict__ dbeta, int cw_shift) {
 #pragma clang fp contract(off)
   const FoldMap fm = fold_map(cap);
   const int c_base = g.ct * cap;
@@ -433,21 +446,26 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
   const int64_t w = (static_cast<int64_t>(blockIdx.z) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
   const int64_t rows = N * S;
   const int64_t W2 = 2 * static_cast<int64_t>(C);  // a partial row: [dgamma terms | dbeta terms]
-  // Outputs are dealt to the blocks in chunks of cw adjacent columns, cw the largest of 64, 16,
-  // 4 that still gives every block a chunk: the threads of a chunk read cw adjacent floats of a
-  // partial row at a time.  With more blocks than that, one column per block-wide sum.
-  int cw = 64;
-  while (cw > 1 && (W2 + cw - 1) / cw < n_blocks) cw >>= 2;
-  // At most one output per block and at most kEarly partial rows per thread: the column's loads
+  // Outputs are dealt to the blocks in chunks of cw = 64, 16, 4 or 1 adjacent columns (the host
+  // picks the width that leaves a block the fewest dependent memory round trips,
+  // cl_dparam_chunk_shift): the 256 / cw thread rows of a chunk each take every (256 / cw)-th
+  // partial row, four at a time.
+  const int cw = 1 << cw_shift;
+  const int rp = kClThreads >> cw_shift;  // partial rows in flight
+  const int cx = static_cast<int>(threadIdx.x) & (cw - 1);
+  const int cy = static_cast<int>(threadIdx.x) >> cw_shift;
+  const int64_t n_chunks = (W2 + cw - 1) >> cw_shift;
+  // At most one chunk per block and at most kEarly partial rows per thread: the chunk's loads
   // are issued here, ahead of the slab fold's, so that both share one memory round trip.
   constexpr int kEarly = 4;
-  const bool early = cw == 1 && W2 <= n_blocks && rows <= kEarly * kClThreads;
+  const bool early = n_chunks <= n_blocks && rows <= static_cast<int64_t>(kEarly) * rp;
   float ev[kEarly];
   if (early) {
+    const int64_t col = w * cw + cx;
 #pragma unroll
     for (int u = 0; u < kEarly; ++u) {
-      const int64_t r = static_cast<int64_t>(threadIdx.x) + u * kClThreads;
-      ev[u] = (w < W2 && r < rows) ? part[r * W2 + w] : 0.f;
+      const int64_t r = cy + u * rp;
+      ev[u] = (col < W2 && r < rows) ? part[r * W2 + col] : 0.f;
     }
   }
   // the partials of the instance: one address for the whole workgroup, 32-bit positions inside
@@ -467,8 +485,10 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
       rs = rstd_in[g.n * C + c];
     }
     float a = 0.f, b = 0.f;
-    if (in) {
-      constexpr int B = kClFoldRegs;
+    // a lane's slabs in batches of 16 or, when that spares a round trip, 32 (the additions are
+    // in slab order either way)
+    auto in_batches = [&](auto bc) {
+      constexpr int B = decltype(bc)::value;
       for (unsigned sl = sub; sl < uS; sl += B * P) {
         float tb[B], ta[B];
 #pragma unroll
@@ -484,6 +504,13 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
           a += ta[u];
         }
       }
+    };
+    if (in) {
+      if (!WIDE || uS <= kClFoldRegs * P) {
+        in_batches(std::integral_constant<int, kClFoldRegs>{});
+      } else {
+        in_batches(std::integral_constant<int, WIDE ? 2 * kClFoldRegs : 1>{});
+      }
     }
     for (int m = 1; m < fm.P; m <<= 1) {
       a += lane_xor(a, m);
@@ -498,21 +525,18 @@ __device__ __forceinline__ void cl_fold_sums(const float* part, const ClGeom& g,
     }
   }
   if (early) {
-    if (w < W2) {  // uniform over the block
-      float t = 0.f;
+    if (w < n_chunks) {  // uniform over the block
+      float t[1] = {0.f};
 #pragma unroll
-      for (int u = 0; u < kEarly; ++u) t += ev[u];
-      t = block_sum1(t, red_buf[0], kClThreads / kWave);
-      if (threadIdx.x == 0) (w < C ? dgamma : dbeta)[w < C ? w : w - C] = t;
+      for (int u = 0; u < kEarly; ++u) t[0] += ev[u];
+      cl_block_sum<1>(t, fold_lds, cw);
+      const int64_t col = w * cw + cx;
+      if (cy == 0 && col < W2) (col < C ? dgamma : dbeta)[col < C ? col : col - C] = t[0];
     }
     __syncthreads();
     return;
   }
   if (cw > 1) {
-    const int cx = static_cast<int>(threadIdx.x) % cw;
-    const int cy = static_cast<int>(threadIdx.x) / cw;
-    const int rp = kClThreads / cw;  // partial rows in flight
-    const int64_t n_chunks = (W2 + cw - 1) / cw;
     for (int64_t chunk = w; chunk < n_chunks; chunk += n_blocks) {
       const int64_t col = chunk * cw + cx;
       float t[1] = {0.f};
@@ -677,7 +701,7 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
   const float n_full = static_cast<float>(slab_len);
   const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * slab_len);
   const float* q = pstat + ((n * S) * 2) * C + (in ? c : 0);
-  constexpr int B = 8;
+  constexpr int B = 16;
   // the phases' partial sums of a channel, added in phase order
   auto across_phases = [&](float v) {
     buf[ph][cx] = v;
@@ -687,41 +711,42 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
     __syncthreads();
     return r;
   };
+  // a phase's slabs ph, ph + PH, ... in batches of B whose loads are all in flight at once; a
+  // position past the last slab reads slab 0 and weighs it 0 (no dependent single loads at the
+  // end of a phase)
+  auto weight = [&](int k) { return k >= S ? 0.f : (k == S - 1 ? n_last : n_full); };
   float s1 = 0.f;
   if (in) {
-    batched_for<B>(
-        ph, S, PH,
-        [&](int64_t sl, int64_t step) {
-          float tm[B];
+    for (int sl = ph; sl < S; sl += B * PH) {
+      float tm[B];
 #pragma unroll
-          for (int u = 0; u < B; ++u) tm[u] = q[((sl + u * step) * 2) * C];
+      for (int u = 0; u < B; ++u) {
+        const int k = sl + u * PH;
+        tm[u] = q[(static_cast<int64_t>(k < S ? k : 0) * 2) * C];
+      }
 #pragma unroll
-          for (int u = 0; u < B; ++u) s1 += tm[u] * (sl + u * step == S - 1 ? n_last : n_full);
-        },
-        [&](int64_t sl) { s1 += q[(sl * 2) * C] * (sl == S - 1 ? n_last : n_full); });
+      for (int u = 0; u < B; ++u) s1 += tm[u] * weight(sl + u * PH);
+    }
   }
   const float mean = across_phases(s1) / static_cast<float>(D);
   float m2 = 0.f;
   if (in) {
-    batched_for<B>(
-        ph, S, PH,
-        [&](int64_t sl, int64_t step) {
-          float tm[B], tq[B];
+    for (int sl = ph; sl < S; sl += B * PH) {
+      float tm[B], tq[B];
 #pragma unroll
-          for (int u = 0; u < B; ++u) {
-            tm[u] = q[((sl + u * step) * 2) * C];
-            tq[u] = q[((sl + u * step) * 2 + 1) * C];
-          }
+      for (int u = 0; u < B; ++u) {
+        const int k = sl + u * PH;
+        const int64_t at = k < S ? k : 0;
+        tm[u] = q[(at * 2) * C];
+        tq[u] = q[(at * 2 + 1) * C];
+      }
 #pragma unroll
-          for (int u = 0; u < B; ++u) {
-            const float d = tm[u] - mean;
-            m2 += tq[u] + (sl + u * step == S - 1 ? n_last : n_full) * (d * d);
-          }
-        },
-        [&](int64_t sl) {
-          const float d = q[(sl * 2) * C] - mean;
-          m2 += q[(sl * 2 + 1) * C] + (sl == S - 1 ? n_last : n_full) * (d * d);
-        });
+      for (int u = 0; u < B; ++u) {
+        const float d = tm[u] - mean;
+        const float tn = weight(sl + u * PH);
+        m2 += tn == 0.f ? 0.f : tq[u] + tn * (d * d);
+      }
+    }
   }
   m2 = across_phases(m2);
   if (ph == 0 && in) {
@@ -749,7 +774,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
-  cl_fold_stats(pstat, g, S, cnt_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
+  cl_fold_stats<(U > 0)>(pstat, g, S, cnt_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
                 rstd_out);
   __syncthreads();
   if (g.ch_ok) {
@@ -878,7 +903,7 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
              const float* __restrict__ part, T* dx, float* __restrict__ dgamma,
              float* __restrict__ dbeta, int64_t N, int64_t D, int C, int S, int tpp_shift,
-             int64_t slab_len, int rev) {
+             int64_t slab_len, int rev, int cw_shift) {
   __shared__ float sm_mu[kClMaxTileChannels];
   __shared__ float sm_sc[kClMaxTileChannels];
   __shared__ float sm_ca[kClMaxTileChannels];
@@ -896,8 +921,8 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, rx, okp);
     cl_load_slab<T, V, U, true>(dy + (g.n * D + g.p0) * C, g, C, rd, okp);
   }
-  cl_fold_sums(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
-               red_buf, fold_lds, dgamma, dbeta);
+  cl_fold_sums<(U > 0)>(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
+               red_buf, fold_lds, dgamma, dbeta, cw_shift);
   if (g.ch_ok) {
     ClBwdCoef<V, RG> k;
     k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
@@ -981,7 +1006,7 @@ cl_fwd_coop(const T* x, float* pstat, const float* __restrict__ gamma,
   cooperative_groups::this_grid().sync();
 #pragma unroll
   for (int u = 0; u < U; ++u) forget_derived<T, V>(raw[u]);
-  cl_fold_stats(pstat, g, S, slab_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
+  cl_fold_stats<true>(pstat, g, S, slab_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
                 rstd_out);
   __syncthreads();
   if (g.ch_ok) {
@@ -1002,7 +1027,7 @@ __global__ void __launch_bounds__(kClThreads, 2)
 cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
             const float* __restrict__ mean_in, const float* __restrict__ rstd_in, float* part,
             T* dx, float* __restrict__ dgamma, float* __restrict__ dbeta, int64_t N, int64_t D,
-            int C, int S, int tpp_shift, int64_t slab_len) {
+            int C, int S, int tpp_shift, int64_t slab_len, int cw_shift) {
   __shared__ float lds[2 * V * kClThreads];
   __shared__ float sm_mu[kClMaxTileChannels];
   __shared__ float sm_sc[kClMaxTileChannels];
@@ -1047,8 +1072,8 @@ cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamm
     forget_derived<T, V>(rd[u]);
   }
   __syncthreads();  // lds is free again
-  cl_fold_sums(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
-               red_buf, lds, dgamma, dbeta);
+  cl_fold_sums<true>(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
+               red_buf, lds, dgamma, dbeta, cw_shift);
   if (g.ch_ok) {
     ClBwdCoef<V, false> k;
     k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);

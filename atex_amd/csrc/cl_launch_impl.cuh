@@ -18,6 +18,8 @@ inline bool stream_is_capturing(hipStream_t st) {
   return status != hipStreamCaptureStatusNone;
 }
 
+static_assert(kPlanClFoldRegs == 2 * kClFoldRegs, "the planner and the kernels must agree on the fold's register limit");
+
 // True if the kernel was enqueued.  False if the runtime refused the launch (typically: more
 // workgroups than the device can hold at once); the error is cleared and the caller falls
 // back to its multi-launch path.
@@ -138,6 +140,9 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   ATEXN_REQUIRE(p.CT <= 65535, "channel count %lld too large (channels-last limit 65535 * 2048)",
                 (long long)C);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
+  // how stage 2 deals the dgamma / dbeta columns to its workgroups (after the fold launch a
+  // partial row per instance is left)
+  const int cw_shift = cl_dparam_chunk_shift(p.fold ? N : N * p.S, 2 * C, N * p.S * p.CT);
 #define ATEXN_CL_BWD(U_, RG_)                                                                  \
   do {                                                                                        \
     cl_bwd_sums<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S, \
@@ -153,7 +158,8 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
                                                        dgamma, dbeta, N, D, Ci,               \
                                                        p.fold ? 1 : p.S,                      \
                                                        p.tpp_shift, p.slab_len,               \
-                                                       tuning().reverse_second_pass);         \
+                                                       tuning().reverse_second_pass,          \
+                                                       cw_shift);                             \
     ATEXN_CHECK_LAUNCH("cl_bwd_apply");                                                       \
   } while (0)
   if constexpr (V > 1) {
@@ -191,8 +197,8 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       float* pa = part;
       T* dxa = dx;
       int64_t Na = N, Da = D, sl = p.slab_len;
-      int Ca = Ci, Sa = p.S, sh = p.tpp_shift;
-      void* args[] = {&dya, &xa, &gamma, &mean, &rstd, &pa, &dxa, &dgamma, &dbeta, &Na, &Da, &Ca, &Sa, &sh, &sl};
+      int Ca = Ci, Sa = p.S, sh = p.tpp_shift, cws = cw_shift;
+      void* args[] = {&dya, &xa, &gamma, &mean, &rstd, &pa, &dxa, &dgamma, &dbeta, &Na, &Da, &Ca, &Sa, &sh, &sl, &cws};
       const void* fn = p.U == 4 ? reinterpret_cast<const void*>(cl_bwd_coop<T, V, 4>)
                                 : reinterpret_cast<const void*>(cl_bwd_coop<T, V, 8>);
       if (launch_cooperative(fn, grid, kClThreads, args, st)) return ATEXN_OK;

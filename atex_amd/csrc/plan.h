@@ -36,6 +36,7 @@ struct Tuning {
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
   TuneInt reverse_second_pass{1};
+  TuneInt cl_fold_cap{1};     // channels-last: no more slabs than a stage-2 fold takes from registers
   TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
   // channels-last: both stages in one cooperative launch when every slab is register-resident
   // and the grid fits the chip at once.  Off: the grid-wide barrier of the cooperative-groups
@@ -350,6 +351,29 @@ struct ClPlan {
   size_t off_a = 0, off_fold = 0, ws_bytes = 0;
 };
 constexpr int kClFoldAbove = 64;
+// slab partials per lane that a stage-2 fold takes in one round trip (cl_kernels.cuh: twice
+// kClFoldRegs)
+constexpr int kPlanClFoldRegs = 32;
+
+// Width (as a shift: 64, 16, 4 or 1 columns) of the chunks of adjacent dgamma / dbeta columns
+// that the channels-last backward's stage 2 deals to its workgroups (cl_fold_sums): `rows`
+// partial rows of W2 columns, n_blocks workgroups of 256 threads; a chunk is summed by 256 / cw
+// thread rows taking four partial rows each per round trip.  The width with the fewest
+// dependent round trips per workgroup wins, the wider one on a tie (longer contiguous reads).
+inline int cl_dparam_chunk_shift(int64_t rows, int64_t W2, int64_t n_blocks) {
+  int best_shift = 0;
+  int64_t best = INT64_MAX;
+  for (int sh = 6; sh >= 0; sh -= 2) {
+    const int64_t cw = int64_t(1) << sh;
+    const int64_t per_block = div_up(div_up(W2, cw), std::max<int64_t>(n_blocks, 1));
+    const int64_t trips = div_up(rows, (256 / cw) * 4);
+    if (per_block * trips < best) {
+      best = per_block * trips;
+      best_shift = sh;
+    }
+  }
+  return best_shift;
+}
 
 inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
   const Tuning& t = tuning();
@@ -364,7 +388,21 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   const int64_t max_s = std::max<int64_t>(1, D / (int64_t(ppb) * 4));
   // the kernels index the slab partials of an instance ([S][2][C] floats) with 32 bits
   const int64_t s_cap = std::min<int64_t>(4096, std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / std::max<int64_t>(C, 1)));
-  const int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), s_cap));
+  int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), s_cap));
+  const int max_u = bwd ? 8 : 16;
+  // the elements of a register-resident slab are addressed with 32-bit offsets from its first
+  // pixel
+  const bool slab32 = (int64_t(16) * ppb + 1) * C < (int64_t(1) << 32);
+  {
+    // A stage-2 workgroup combines the S slab partials of its channels on fold_p lanes per
+    // channel, and in one memory round trip while a lane has at most kPlanClFoldRegs of them.
+    // An instance small enough to be register-resident with that many slabs gets no more:
+    // its launches are bound by dependent round trips, not by the number of workgroups.
+    const int cap = p.TPP * V;
+    const int fold_p = cap >= 256 ? 1 : std::min(64, 256 / cap);
+    const int64_t s_reg = std::min<int64_t>(int64_t(kPlanClFoldRegs) * fold_p, kClFoldAbove);
+    if (t.cl_fold_cap && slab32 && S > s_reg && div_up(round_up(div_up(D, s_reg), ppb), ppb) <= max_u) S = s_reg;
+  }
   p.slab_len = round_up(div_up(D, S), ppb);
   p.S = static_cast<int>(div_up(D, p.slab_len));
   p.n_work = N * p.S * p.CT;
@@ -372,9 +410,6 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   // a slab of at most 16 (backward: 8, it holds x and dy) vectors per thread stays in
   // registers between its load and its use
   const int64_t per_thread = p.slab_len / ppb;
-  const int max_u = bwd ? 8 : 16;
-  // ... and the elements of a resident slab with 32-bit offsets from its first pixel
-  const bool slab32 = (int64_t(16) * ppb + 1) * C < (int64_t(1) << 32);
   for (int u = 4; slab32 && u <= max_u; u *= 2) {
     if (per_thread <= u) {
       p.U = u;

@@ -143,6 +143,11 @@ static void check_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) 
   if (p.fused) EXPECT(p.S == 1 && V > 1 && C >= V, "fused with S=%d", p.S);
   if (p.fold) EXPECT(p.S > kClFoldAbove && N <= 65535, "fold");
   EXPECT(p.n_work == N * p.S * p.CT && p.grid >= 1, "n_work");
+  if (bwd) {
+    // the chunk width of the dgamma / dbeta columns in stage 2: 64, 16, 4 or 1
+    const int sh = cl_dparam_chunk_shift(p.fold ? N : N * p.S, 2 * C, p.n_work);
+    EXPECT(sh == 0 || sh == 2 || sh == 4 || sh == 6, "chunk shift %d", sh);
+  }
   const size_t sect = sizeof(float) * size_t(N) * size_t(p.S) * size_t(C);
   EXPECT(p.off_fold >= 2 * sect && p.ws_bytes >= p.off_fold + sizeof(float) * 2 * size_t(N) * size_t(C), "workspace sections");
 }

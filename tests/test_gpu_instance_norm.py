@@ -295,9 +295,14 @@ def test_channels_last_wide_channel_counts(capi, coracle, N, C, S, dtype):
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("N,C,S", [(16, 256, 8192), (9, 512, 4096), (20, 1024, 3000), (8, 8, 40000), (30, 16, 20000),
                                    (12, 64, 16 * 1024 + 5), (8, 100, 16384), (64, 100, 4096), (16, 20, 9000),
-                                   (7, 13, 33333)])
+                                   (7, 13, 33333), (2, 128, 8000), (2, 320, 512), (2, 512, 2000), (3, 24, 2000),
+                                   (1, 8, 300000)])
 def test_channels_last_slab_fold_paths(capi, coracle, N, C, S, dtype):
     """The second stage folds the slab partials of its instance with all of a lane's partials in
-    registers (at most 16 per lane) or in batches (more): shapes with one lane per channel and
-    17 .. 64 slabs, with 32 lanes per channel, and with a short last slab."""
+    registers (at most 16 per lane, or 32 when the slab itself is register-resident) or in
+    batches (more): shapes with one lane per channel and 17 .. 64 slabs, with 32 lanes per
+    channel, with a short last slab, small instances whose slab count the planner caps at what
+    the registers take (two sweeps of a 512-channel tile among them), and one instance of 235
+    slabs, whose partials a launch of its own folds in batches that end in a partial one.  The
+    backward cases deal the dgamma / dbeta columns out in chunks of 1, 4, 16 and 64."""
     run_case(capi, coracle, N, C, S, dtype, False, 31)
