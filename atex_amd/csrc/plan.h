@@ -37,6 +37,7 @@ struct Tuning {
   // is what the memory-side cache still holds).
   TuneInt reverse_second_pass{1};
   TuneInt cl_fold_cap{1};     // channels-last: no more slabs than a stage-2 fold takes from registers
+  TuneInt cl_fused_split{1};  // channels-last single pass: narrower channel tiles so that an instance fits
   TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
   // channels-last: both stages in one cooperative launch when every slab is register-resident
   // and the grid fits the chip at once.  Off: the grid-wide barrier of the cooperative-groups
@@ -381,6 +382,23 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   p.V = V;
   p.CV = static_cast<int>(div_up(C, V));
   p.TPP = std::min(256, pow2_ceil(p.CV));
+  const int max_u = bwd ? 8 : 16;
+  bool single_pass = false;
+  if (t.cl_fused && t.cl_fused_split && V > 1) {
+    // Single pass: the D pixels of an instance, for a tile of TPP channel vectors, fit the
+    // registers of one workgroup at max_u vectors per thread.  Narrower tiles (down to 8
+    // vectors: 128-byte pieces of a pixel) hold more pixels each, and there are more of them:
+    // the widest tile that fits is split further while the launch has fewer workgroups than CUs.
+    int pick = 0;
+    for (int tp = p.TPP; tp >= std::min(p.TPP, 8); tp >>= 1) {
+      if (div_up(D, 256 / tp) > max_u) continue;
+      if (pick == 0 || N * div_up(p.CV, pick) < cus) pick = tp;
+    }
+    if (pick != 0) {
+      p.TPP = pick;
+      single_pass = true;
+    }
+  }
   while ((1 << p.tpp_shift) < p.TPP) ++p.tpp_shift;
   p.CT = static_cast<int>(div_up(p.CV, p.TPP));
   const int ppb = 256 / p.TPP;
@@ -388,8 +406,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   const int64_t max_s = std::max<int64_t>(1, D / (int64_t(ppb) * 4));
   // the kernels index the slab partials of an instance ([S][2][C] floats) with 32 bits
   const int64_t s_cap = std::min<int64_t>(4096, std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / std::max<int64_t>(C, 1)));
-  int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), s_cap));
-  const int max_u = bwd ? 8 : 16;
+  int64_t S = single_pass ? 1 : std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), s_cap));
   // the elements of a register-resident slab are addressed with 32-bit offsets from its first
   // pixel
   const bool slab32 = (int64_t(16) * ppb + 1) * C < (int64_t(1) << 32);

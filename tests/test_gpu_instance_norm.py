@@ -203,6 +203,12 @@ def test_deterministic(capi):
     (300, 36, 50),
     (1, 9, 1000),
     (3, 2051, 7),      # ... with two channel tiles
+    (2, 320, 216),     # few instances: channel tiles of 8 vectors so that an instance fits and
+    (2, 320, 512),     #   the launch has more workgroups (forward only at 512 pixels)
+    (2, 100, 300),     # ... ragged, the last vector inside the second tile
+    (3, 68, 200),      # ... ragged, the last vector reaching back into the first tile
+    (5, 332, 128),     # ... ragged, six tiles
+    (1, 64, 512),      # one workgroup in all
 ])
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
