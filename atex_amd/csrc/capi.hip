@@ -133,6 +133,7 @@ int atexn_set_tuning(const char* name, int value) {
     t.bwd_ln_threads = value;
   } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_affine_waves_per_cu")) t.bwd_affine_waves_per_cu = value;
+  else if (!strcmp(name, "bwd_min_rows")) t.bwd_min_rows = value;
   else if (!strcmp(name, "split_items_per_cu")) t.split_items_per_cu = value;
   else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
   else if (!strcmp(name, "tile_items_per_cu")) t.tile_items_per_cu = value;

@@ -33,6 +33,7 @@ struct Tuning {
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
+  TuneInt bwd_min_rows{4};           // resident LayerNorm backward: rows per workgroup worth a partial row
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
   TuneInt reverse_second_pass{1};
@@ -219,6 +220,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
                waves);
     p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(groups, int64_t(cus) * per_cu)));
     if (kind == RowsKind::kBwdCols) {
+      // A workgroup leaves one partial row of 2 * D floats however few rows it had: with fewer
+      // than bwd_min_rows (4) rows each, the partial rows are more traffic than the rows.  Few
+      // long rows get fewer workgroups (not below half the CUs).
+      while (p.grid >= cus && p.grid > 1 && div_up(n_rows, p.grid) < t.bwd_min_rows) p.grid = (p.grid + 1) / 2;
       p.part_rows = p.grid;
       p.off_part = 0;
       p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
