@@ -843,15 +843,78 @@ __global__ void __launch_bounds__(kSplitThreads) split_fwd_stats(const T* __rest
   }
 }
 
+// Statistics of a row from those of its S chunks (S <= 1024), the same in every lane of every
+// wave: lane l takes chunks l, l + 64, ... (all its loads in flight at once), and the row is
+//     mean = sum_s n_s mean_s / D,      m2 = sum_s [ m2_s + n_s (mean_s - mean)^2 ]
+// which is Chan's merge (norm_util.h:190-210) of all chunks at once: every term of m2 is
+// non-negative and there is no chain of S dependent merges.  The sums over the lanes are
+// commutative butterflies, so every workgroup of the row gets the same bits.
 __device__ __forceinline__ Wf merge_chunks(const float2* stats, int S, int64_t D, int64_t chunk) {
-  Wf r{0.f, 0.f, 0.f};
-  for (int s = 0; s < S; ++s) {
-    const int64_t beg = static_cast<int64_t>(s) * chunk;
-    const float2 t = stats[s];
-    Wf o{t.x, t.y, static_cast<float>(beg + chunk <= D ? chunk : D - beg)};
-    r = wf_merge(r, o);
+#pragma clang fp contract(off)
+  constexpr int B = 4;
+  const int lane = static_cast<int>(threadIdx.x) & (kWave - 1);
+  const float n_full = static_cast<float>(chunk);
+  const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * chunk);
+  const float inv_d = 1.0f / static_cast<float>(D);
+  auto count = [&](int k) { return k >= S ? 0.f : (k == S - 1 ? n_last : n_full); };
+  float s1 = 0.f, m2 = 0.f, mean;
+  if (S <= B * kWave) {  // one round trip
+    float2 t[B];
+#pragma unroll
+    for (int u = 0; u < B; ++u) {
+      const int k = lane + u * kWave;
+      t[u] = stats[k < S ? k : 0];
+    }
+#pragma unroll
+    for (int u = 0; u < B; ++u) s1 += t[u].x * count(lane + u * kWave);
+    mean = group_sum<kWave>(s1) * inv_d;
+#pragma unroll
+    for (int u = 0; u < B; ++u) {
+      const float n = count(lane + u * kWave);
+      const float d = t[u].x - mean;
+      m2 += n == 0.f ? 0.f : t[u].y + n * (d * d);
+    }
+  } else {
+    for (int k0 = lane; k0 < S; k0 += B * kWave) {
+      float2 t[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) t[u] = stats[k0 + u * kWave < S ? k0 + u * kWave : 0];
+#pragma unroll
+      for (int u = 0; u < B; ++u) s1 += t[u].x * count(k0 + u * kWave);
+    }
+    mean = group_sum<kWave>(s1) * inv_d;
+    for (int k0 = lane; k0 < S; k0 += B * kWave) {
+      float2 t[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) t[u] = stats[k0 + u * kWave < S ? k0 + u * kWave : 0];
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        const float n = count(k0 + u * kWave);
+        const float d = t[u].x - mean;
+        m2 += n == 0.f ? 0.f : t[u].y + n * (d * d);
+      }
+    }
   }
-  return r;
+  m2 = group_sum<kWave>(m2);
+  return Wf{mean, m2, static_cast<float>(D)};
+}
+
+// Sums of a row from those of its S chunks, likewise in every lane of every wave.
+__device__ __forceinline__ float2 sum_chunks(const float2* sums, int S) {
+  constexpr int B = 4;
+  const int lane = static_cast<int>(threadIdx.x) & (kWave - 1);
+  float a = 0.f, b = 0.f;
+  for (int k0 = lane; k0 < S; k0 += B * kWave) {
+    float2 t[B];
+#pragma unroll
+    for (int u = 0; u < B; ++u) t[u] = sums[k0 + u * kWave < S ? k0 + u * kWave : 0];
+#pragma unroll
+    for (int u = 0; u < B; ++u) {
+      a += k0 + u * kWave < S ? t[u].x : 0.f;
+      b += k0 + u * kWave < S ? t[u].y : 0.f;
+    }
+  }
+  return make_float2(group_sum<kWave>(a), group_sum<kWave>(b));
 }
 
 // stage 2 forward: merge the S chunk statistics of the row, normalise the chunk.
@@ -1033,12 +1096,8 @@ __global__ void __launch_bounds__(kSplitThreads) split_bwd_apply(const T* dy, co
   for (int64_t w = blockIdx.x; w < n_work; w += gridDim.x) {
     const int64_t row = w / S;
     const int s = static_cast<int>(w % S);
-    float s1 = 0.f, s2 = 0.f;
-    for (int k = 0; k < S; ++k) {
-      const float2 t = sums[row * S + k];
-      s1 += t.x;
-      s2 += t.y;
-    }
+    const float2 st = sum_chunks(sums + row * S, S);
+    const float s1 = st.x, s2 = st.y;
     const float mean = mean_in[row], rstd = rstd_in[row];
     float gs = 1.f;
     if constexpr (ROW_AFFINE) {
