@@ -81,7 +81,15 @@ CASES = {
     "inref_8x128x64_cf": ("in", "f16", (8, 128, 64 ** 3, True)),
     "inref_4x256x32_cl": ("in", "f16", (4, 256, 32 ** 3, False)),
     "inref_4x256x32_cf": ("in", "f16", (4, 256, 32 ** 3, True)),
+    # few instances, hundreds of channels (the deep levels of a 3-D U-Net), and few long rows
+    "in_2x320x216_cl": ("in", "f16", (2, 320, 6 ** 3, False)),
+    "in_2x320x512_cl": ("in", "f16", (2, 320, 8 ** 3, False)),
+    "in_2x128x4096_cl": ("in", "f16", (2, 128, 16 ** 3, False)),
+    "ln_512x4096_f16": ("ln", "f16", (512, 4096)),
 }
+# cases that `--case all` leaves out (single-purpose sweeps and the reference's benchmark table)
+SWEEP_ONLY_CASES = frozenset(
+    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
 DEFAULT_CASE = "ln_bert"
 # the two shapes the throughput target is stated on, reported on the default run's line
 TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
@@ -558,7 +566,7 @@ def main():
                 sys.exit(f"--tune {item}: {L.atexn_last_error().decode()}")
     if args.case == "all":
         for name in CASES:
-            if "ref_" in name or "in_1x" in name or "x1" in name or "x2" in name or "x7" in name or name.endswith("_f32"):
+            if name in SWEEP_ONLY_CASES:
                 continue
             steps = args.steps if "3d" not in name else max(10, args.steps // 10)
             r = run_case(name, steps, args.warmup, with_cpu=False)
