@@ -33,6 +33,7 @@ struct Tuning {
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
+  TuneInt bwd_lds_rows{1};           // LayerNorm backward: the single-pass kernel with accumulators in LDS
   TuneInt bwd_min_rows{4};           // resident LayerNorm backward: rows per workgroup worth a partial row
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
   // is what the memory-side cache still holds).
@@ -86,6 +87,7 @@ struct RowsPlan {
   bool ragged = false;  // D % V != 0: the last vector of a row is partial
   int grid = 1;
   size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
+  bool acc_lds = false;  // LayerNorm backward with the column accumulators in LDS (rows_bwd_lds)
   // split
   int S = 1;
   int64_t chunk = 0;
@@ -101,6 +103,17 @@ struct RowsPlan {
 // The channel-first InstanceNorm backward has no such accumulators and goes as far as the
 // forward.
 inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kBwdCols ? 2048 : 4096; }
+
+// LayerNorm backward beyond that: one more single-pass kernel keeps the dgamma / dbeta
+// accumulators of a workgroup's columns in LDS (rows_bwd_lds: 8 bytes per column, 8 vectors per
+// thread at up to 512 threads) while they fit the 160 KiB of a gfx950 CU beside the block
+// reductions' buffer.
+constexpr size_t kPlanLdsBytes = 160 * 1024;
+constexpr size_t kPlanBwdLdsReserve = 512;
+inline size_t bwd_lds_bytes(int64_t D) { return size_t(round_up(D, 4)) * 2 * sizeof(float); }
+inline bool bwd_lds_fits(int V, int64_t D) {
+  return V > 1 && tuning().bwd_lds_rows && div_up(D, V) <= 4096 && bwd_lds_bytes(D) + kPlanBwdLdsReserve <= kPlanLdsBytes;
+}
 
 // Which kernels take a contiguous-row problem.  vec = 16 / sizeof(T).
 //   V = vec: rows of at least one vector (a ragged end, D % vec != 0, is handled inside the
@@ -125,7 +138,8 @@ inline RowsRoute route_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_r
     return r;
   }
   if (D >= vec) r.V = vec;  // ragged row ends are handled by every vector kernel
-  r.tiles = layer_norm && div_up(D, r.V) > resident_limit(kind);
+  r.tiles = layer_norm && div_up(D, r.V) > resident_limit(kind) &&
+            !(kind == RowsKind::kBwdCols && bwd_lds_fits(r.V, D));
   return r;
 }
 
@@ -157,6 +171,22 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   const int64_t n_vec = div_up(D, V);
   p.ragged = D % V != 0;
   p.resident = n_vec <= resident_limit(kind);
+  if (!p.resident && kind == RowsKind::kBwdCols && bwd_lds_fits(V, D)) {
+    p.resident = true;
+    p.acc_lds = true;
+    p.tpr = 0;
+    p.vpt = 8;
+    p.threads = static_cast<int>(round_up(div_up(n_vec, p.vpt), 64));
+    p.rpb = 1;
+    p.rb = 1;
+    p.fold_lds = bwd_lds_bytes(D);
+    p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(n_rows, cus)));  // one workgroup per CU (LDS)
+    while (p.grid >= cus && p.grid > 1 && div_up(n_rows, p.grid) < t.bwd_min_rows) p.grid = (p.grid + 1) / 2;
+    p.part_rows = p.grid;
+    p.off_part = 0;
+    p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
+    return p;
+  }
   if (p.resident) {
     // Rows of up to 192 vectors sit on a group of 8..64 lanes with 1, 2 or 3 vectors per lane:
     // the candidate with the fewest slots wins (3 vectors per lane make the 3 * 2^k hidden

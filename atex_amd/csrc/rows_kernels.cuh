@@ -675,6 +675,161 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   }
 }
 
+// ------------------------------------------- backward, resident, accumulators in LDS
+// LayerNorm rows too long for rows_bwd_resident, whose per-lane dgamma / dbeta accumulators
+// cost two registers per element held: the same single pass (a workgroup per row, x and dy
+// read once, one partial row per workgroup for col_reduce), with the accumulators of the
+// workgroup's columns in LDS instead, acc[0][0..D) (dgamma terms) and acc[1][0..D) (dbeta
+// terms): 8 * D bytes, so D <= 20416 on the 160 KiB of a gfx950 CU (one workgroup per CU).
+// A thread owns its columns outright (one row per workgroup), so nobody else touches its
+// LDS words and the accumulation needs no barrier; per row it reads and writes 16 * D
+// bytes of LDS per workgroup, about a sixth of the time the CU's share of the memory
+// bandwidth needs for the row.  xh and g are recomputed from the raw vectors for the dx
+// pass instead of being kept (8 vectors per lane: they would not fit).
+// dx may alias dy, not x.
+constexpr int kBwdLdsThreads = 512;
+constexpr int kBwdLdsVpt = 8;
+
+template <typename T, int V, bool RAGGED>
+__global__ void __launch_bounds__(kBwdLdsThreads)
+rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
+             const float* __restrict__ mean_in, const float* __restrict__ rstd_in, T* dx,
+             float* __restrict__ part, int64_t n_rows, int d_elems) {
+  constexpr int VPT = kBwdLdsVpt;
+  __shared__ float2 sum_buf[2][16];
+  extern __shared__ __attribute__((aligned(16))) float acc[];  // [2][d_elems rounded up to 4]
+  float* const acc_b = acc + (d_elems + 3) / 4 * 4;
+  const int bdim = block_threads();
+  const int n_waves = bdim / kWave;
+  const int64_t D = d_elems;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const int n_full = d_elems / V;
+  const int rem = RAGGED ? d_elems % V : 0;
+  // unpredicated loads from clamped positions, masked arithmetic (as in rows_bwd_resident)
+  bool vec_ok[VPT];
+  int col[VPT];
+  int lo[VPT];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    const int idx = static_cast<int>(threadIdx.x) + k * bdim;
+    const bool full = idx < n_full;
+    const bool tail = RAGGED && idx == n_full;
+    vec_ok[k] = full || tail;
+    col[k] = full ? idx * V : d_elems - V;
+    lo[k] = tail ? V - rem : 0;
+  }
+  float g[VPT][V];
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    load_f32<V>(gamma + col[k], g[k]);
+    if (vec_ok[k]) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        if (!RAGGED || i >= lo[k]) {
+          acc[col[k] + i] = 0.f;
+          acc_b[col[k] + i] = 0.f;
+        }
+      }
+    }
+  }
+  int it = 0;
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x, ++it) {
+    const T* xr = x + row * D;
+    const T* dyr = dy + row * D;
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    Pack<T, V> px[VPT], pd[VPT];
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      px[k] = load_pack<T, V>(xr + col[k]);
+      pd[k] = load_pack<T, V>(dyr + col[k]);
+    }
+    batch_loaded<T, V, VPT>(px);
+    batch_loaded<T, V, VPT>(pd);
+    float a1 = 0.f, a2 = 0.f;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (vec_ok[k]) {
+        float tg[V], tb[V];
+        if (!RAGGED || lo[k] == 0) {
+          load_f32<V>(acc + col[k], tg);
+          load_f32<V>(acc_b + col[k], tb);
+        }
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          const bool ok = !RAGGED || i >= lo[k];
+          const float h = ok ? (to_f32(px[k].v[i]) - mean) * rstd : 0.f;
+          const float d = ok ? to_f32(pd[k].v[i]) : 0.f;
+          const float t = d * g[k][i];
+          a1 += t;
+          a2 += t * h;
+          if (!RAGGED || lo[k] == 0) {
+            tg[i] += d * h;
+            tb[i] += d;
+          } else if (ok) {  // the overlapping last vector: its own elements only
+            acc[col[k] + i] += d * h;
+            acc_b[col[k] + i] += d;
+          }
+        }
+        if (!RAGGED || lo[k] == 0) {
+          store_f32<V>(acc + col[k], tg);
+          store_f32<V>(acc_b + col[k], tb);
+        }
+      }
+      // one vector's accumulators at a time: with the LDS reads of all eight vectors moved to
+      // the front, the kernel does not fit its registers
+      asm volatile("" ::: "memory");
+    }
+    // (only the raw vectors wait through the reduction; xh and g are computed again)
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      forget_derived(px[k]);
+      forget_derived(pd[k]);
+    }
+    const float2 s = block_sum2(a1, a2, sum_buf[it & 1], n_waves);
+    const float ca = -rstd * (s.y * inv_d), cb = -rstd * (s.x * inv_d);
+    T* dxr = dx + row * D;
+#pragma unroll
+    for (int k = 0; k < VPT; ++k) {
+      if (vec_ok[k]) {
+        Pack<T, V> o;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          const float h = (to_f32(px[k].v[i]) - mean) * rstd;
+          const float t = to_f32(pd[k].v[i]) * g[k][i];
+          o.v[i] = from_f32<T>(rstd * t + (ca * h + cb));
+        }
+        if constexpr (RAGGED) {
+          store_pack_from<T, V>(dxr + col[k], o, lo[k]);
+        } else {
+          store_pack<T, V>(dxr + col[k], o);
+        }
+      }
+    }
+  }
+  // the workgroup's partial row: every thread copies the columns it owns
+  float* prow = part + static_cast<int64_t>(blockIdx.x) * 2 * D;
+#pragma unroll
+  for (int k = 0; k < VPT; ++k) {
+    if (vec_ok[k]) {
+      float tg[V], tb[V];
+      if (!RAGGED || lo[k] == 0) {
+        load_f32<V>(acc + col[k], tg);
+        load_f32<V>(acc_b + col[k], tb);
+        store_f32<V>(prow + col[k], tg);
+        store_f32<V>(prow + D + col[k], tb);
+      } else {
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          if (i >= lo[k]) {
+            prow[col[k] + i] = acc[col[k] + i];
+            prow[D + col[k] + i] = acc_b[col[k] + i];
+          }
+        }
+      }
+    }
+  }
+}
+
 // ------------------------------------------------------------- column reduction
 // out0[j] = sum_g part[g][0][j], out1[j] = sum_g part[g][1][j] for j < W, g < G, summed
 // in a fixed order (deterministic; the reference likewise uses no atomics,

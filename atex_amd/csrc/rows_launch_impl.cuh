@@ -250,6 +250,30 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_part);
   const int64_t W = AFF ? C : D;
+  if constexpr (!AFF && V > 1) {
+    if (p.acc_lds) {
+      // more dynamic LDS than the default limit of a launch: raised once per kernel
+      static const hipError_t raised[2] = {
+          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_lds<T, V, false>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve)),
+          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_lds<T, V, true>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve))};
+      ATEXN_REQUIRE(raised[0] == hipSuccess && raised[1] == hipSuccess,
+                    "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      static_assert(kBwdLdsThreads == 512 && kBwdLdsVpt == 8, "plan_rows sizes rows_bwd_lds launches");
+      const int stages = bwd_stage_mask();
+      if (stages & 1) {
+        if (p.ragged) {
+          rows_bwd_lds<T, V, true><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, static_cast<int>(D));
+        } else {
+          rows_bwd_lds<T, V, false><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, static_cast<int>(D));
+        }
+        ATEXN_CHECK_LAUNCH("rows_bwd_lds");
+      }
+      if (!(stages & 2)) return ATEXN_OK;
+      return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+    }
+  }
   if (p.resident) {
     auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact, p.ragged);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);

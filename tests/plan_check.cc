@@ -70,7 +70,15 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
   const RowsPlan p = plan_rows(kind, r.V, n_rows, D, C, cus);
   EXPECT(p.ragged == (D % r.V != 0), "ragged");
   if (p.resident) {
-    EXPECT(n_vec <= resident_limit(kind), "resident beyond the limit");
+    if (p.acc_lds) {
+      // the LayerNorm backward with its column accumulators in LDS
+      EXPECT(kind == RowsKind::kBwdCols && r.V > 1 && n_vec > resident_limit(kind) && n_vec <= 4096, "acc_lds with n_vec=%lld", (long long)n_vec);
+      EXPECT(p.tpr == 0 && p.vpt == 8 && p.threads <= 512 && !p.exact, "acc_lds launch shape");
+      EXPECT(p.fold_lds >= sizeof(float) * 2 * size_t(round_up(D, 4)) && p.fold_lds + 512 <= 160 * 1024, "acc_lds LDS bytes %zu", p.fold_lds);
+      EXPECT(p.grid >= 1 && p.grid <= cus, "acc_lds grid=%d: one workgroup per CU", p.grid);
+    } else {
+      EXPECT(n_vec <= resident_limit(kind), "resident beyond the limit");
+    }
     EXPECT(p.threads >= 64 && p.threads <= 1024 && p.threads % 64 == 0, "threads=%d", p.threads);
     EXPECT(p.vpt >= 1 && p.vpt <= 8, "vpt=%d", p.vpt);
     if (p.tpr == 0) {

@@ -44,8 +44,9 @@ def run_case(capi, coracle, cfg, N, D, dtype, seed_index, in_place=False):
     rstd32 = rstd_ref.astype(np.float32)
     dx_ref, dg_ref, db_ref = coracle.ln_bwd(dy, x, gamma, mean32.astype(np.float64),
                                             rstd32.astype(np.float64), dtype, f64=True)
-    dx, dg, db = capi.ln_bwd(util.to_device(dy, dtype), x_keep, gd, torch.from_numpy(mean32).cuda(),
-                             torch.from_numpy(rstd32).cuda(), dtype)
+    dyd = util.to_device(dy, dtype)
+    dx, dg, db = capi.ln_bwd(dyd, x_keep, gd, torch.from_numpy(mean32).cuda(),
+                             torch.from_numpy(rstd32).cuda(), dtype, dx=dyd if in_place else None)
     torch.cuda.synchronize()
     assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx",
                  scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), rstd32, dtype))
@@ -124,6 +125,19 @@ def test_unaligned_pointers(capi, coracle, N, D, dtype):
                  scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), util.to_host(rstd), dtype))
     assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
     assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,D,in_place", [(600, 18432, False), (300, 20416, False), (1, 20000, False),
+                                          (700, 16388, True), (257, 17001, False), (520, 12288, False),
+                                          (9, 12291, True), (1500, 9000, False), (40, 16383, False)])
+def test_backward_accumulators_in_lds(capi, coracle, N, D, dtype, in_place):
+    """Rows of more than 2048 vectors whose dgamma / dbeta accumulators still fit a CU's LDS
+    (up to 20416 elements: every 16-bit row from 16385 on, every float32 row from 8193 on)
+    take a single-pass backward with the accumulators in LDS; ragged row ends (an overlapping
+    last vector), a row count that is not a multiple of the workgroups, one row, the largest
+    row, and dx written over dy."""
+    run_case(capi, coracle, "plain", N, D, dtype, 19, in_place=in_place)
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
