@@ -124,7 +124,7 @@ int atexn_abi_version(void) { return kAbiVersion; }
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_coop") || !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_coop") || !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -165,6 +165,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "cl_fused_split")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_fused_split must be 0 or 1");
     t.cl_fused_split = value;
+  } else if (!strcmp(name, "cl_narrow_tiles")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "cl_narrow_tiles must be 0 or 1");
+    t.cl_narrow_tiles = value;
   } else if (!strcmp(name, "cl_fold_cap")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_fold_cap must be 0 or 1");
     t.cl_fold_cap = value;
