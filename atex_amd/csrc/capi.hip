@@ -124,7 +124,7 @@ int atexn_abi_version(void) { return kAbiVersion; }
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_coop") || !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_coop") || !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -134,7 +134,10 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_affine_waves_per_cu")) t.bwd_affine_waves_per_cu = value;
   else if (!strcmp(name, "bwd_min_rows")) t.bwd_min_rows = value;
-  else if (!strcmp(name, "bwd_lds_rows")) {
+  else if (!strcmp(name, "staged_rows")) {
+    ATEXN_REQUIRE(value >= 0 && value <= 2, "staged_rows must be 0, 1 or 2");
+    t.staged_rows = value;
+  } else if (!strcmp(name, "bwd_lds_rows")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "bwd_lds_rows must be 0 or 1");
     t.bwd_lds_rows = value;
   }

@@ -33,6 +33,7 @@ struct Tuning {
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
+  TuneInt staged_rows{1};            // rows beyond the registers staged in LDS, single pass (0: never, 2: however few rows)
   TuneInt bwd_lds_rows{1};           // LayerNorm backward: the single-pass kernel with accumulators in LDS
   TuneInt bwd_min_rows{4};           // resident LayerNorm backward: rows per workgroup worth a partial row
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
@@ -89,6 +90,8 @@ struct RowsPlan {
   int grid = 1;
   size_t fold_lds = 0;  // dynamic LDS of the LayerNorm backward fold
   bool acc_lds = false;  // LayerNorm backward with the column accumulators in LDS (rows_bwd_lds)
+  bool staged = false;   // single pass with the row staged in registers + LDS (rows_*_staged)
+  int nv_lds = 0;        //   vectors per thread kept in LDS (the first 8 stay in registers)
   // split
   int S = 1;
   int64_t chunk = 0;
@@ -112,6 +115,25 @@ inline int64_t resident_limit(RowsKind kind) { return kind == RowsKind::kBwdCols
 constexpr size_t kPlanLdsBytes = 160 * 1024;
 constexpr size_t kPlanBwdLdsReserve = 512;
 inline size_t bwd_lds_bytes(int64_t D) { return size_t(round_up(D, 4)) * 2 * sizeof(float); }
+// Rows staged on chip (rows_fwd_staged / rows_bwd_staged): 512 threads, 8 vectors per thread in
+// registers and the rest in LDS (16 bytes per vector forward, 32 backward: x and dy).
+constexpr int kPlanStagedThreads = 512;
+constexpr int kPlanStagedRegVec = 8;
+inline int staged_lds_vectors(RowsKind kind, int64_t n_vec) {
+  return static_cast<int>(std::max<int64_t>(0, div_up(n_vec, kPlanStagedThreads) - kPlanStagedRegVec));
+}
+inline size_t staged_lds_bytes(RowsKind kind, int64_t n_vec) {
+  return size_t(staged_lds_vectors(kind, n_vec)) * kPlanStagedThreads * (kind == RowsKind::kFwd ? 16 : 32);
+}
+// One workgroup streams a row at a few tens of GB/s (its loads in flight over the memory
+// latency), so staging pays once there are enough rows to keep every CU busy for several of
+// them: measured against the two-stage kernels, [1024, 65536] fp16 planes 65 / 111 -> 53 / 93 us,
+// but 256 such planes 16.8 -> 20.9 us forward (backward 28.4 -> 26.3 us) and a single one twice as slow.
+inline bool staged_fits(RowsKind kind, int V, int64_t n_rows, int64_t D, int cus) {
+  return V > 1 && kind != RowsKind::kBwdCols && tuning().staged_rows && D < (int64_t(1) << 31) &&
+         (tuning().staged_rows == 2 || n_rows >= int64_t(cus) * (kind == RowsKind::kFwd ? 2 : 1)) &&
+         staged_lds_bytes(kind, div_up(D, V)) + kPlanBwdLdsReserve <= kPlanLdsBytes;
+}
 inline bool bwd_lds_fits(int V, int64_t D) {
   return V > 1 && tuning().bwd_lds_rows && div_up(D, V) <= 4096 && bwd_lds_bytes(D) + kPlanBwdLdsReserve <= kPlanLdsBytes;
 }
@@ -186,6 +208,21 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     p.part_rows = p.grid;
     p.off_part = 0;
     p.ws_bytes = align256(sizeof(float) * 2 * size_t(D) * size_t(p.grid));
+    return p;
+  }
+  if (!p.resident && staged_fits(kind, V, n_rows, D, cus)) {
+    p.staged = true;
+    p.threads = kPlanStagedThreads;
+    p.nv_lds = staged_lds_vectors(kind, n_vec);
+    p.fold_lds = staged_lds_bytes(kind, n_vec);
+    // workgroups per CU: what the LDS leaves room for, at most four (2048 threads)
+    const int64_t per_cu = std::max<int64_t>(1, std::min<int64_t>(4, int64_t(kPlanLdsBytes) / int64_t(p.fold_lds + kPlanBwdLdsReserve)));
+    p.grid = static_cast<int>(std::max<int64_t>(1, std::min<int64_t>(n_rows, int64_t(cus) * per_cu)));
+    if (kind == RowsKind::kBwdAffine) {
+      p.part_rows = static_cast<int>(n_rows / C);
+      p.off_part = 0;
+      p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
+    }
     return p;
   }
   if (p.resident) {

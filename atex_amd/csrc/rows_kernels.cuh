@@ -830,6 +830,244 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   }
 }
 
+// ------------------------------------- rows staged in registers and LDS, single pass
+// Rows longer than the register-resident kernels take (4096 vectors) but short enough to sit on
+// chip in one workgroup: the first kStagedRegVec vectors of every thread stay in registers,
+// the rest of the row waits in LDS as raw 16-byte vectors (up to 152 KiB of a gfx950 CU's
+// 160), and the row still makes ONE trip through memory: exact two-pass statistics and the
+// normalisation read the staged copy.  A thread only ever reads back the LDS words it wrote
+// itself, so the staging needs no barrier; the two block-wide sums are the only ones.
+// Channel-first InstanceNorm planes (gamma / beta are scalars of the row; LayerNorm's per-column
+// gamma / beta would be read again for every row, three times the bytes of the row itself from
+// L2: measured slower than the 2-D tiles): forward up to 27 vectors per thread (110592 halves:
+// a 48^3 or 256^2 plane), backward (x and dy staged) up to 17 (69632 halves).  The two-stage
+// kernels (split_*) read such planes twice.
+constexpr int kStagedThreads = 512;
+constexpr int kStagedRegVec = 8;
+
+// Where vector slot idx of a row lies: its first column (clamped to a valid one when the slot
+// is past the row), whether it holds data, and the first element it owns (the overlapping
+// last vector of a ragged row owns only its last D % V elements).
+template <int V>
+struct StagedSlot {
+  int col, lo;
+  bool ok;
+};
+template <int V>
+__device__ __forceinline__ StagedSlot<V> staged_slot(int idx, int d_elems) {
+  const int n_full = d_elems / V;
+  const int rem = d_elems % V;
+  StagedSlot<V> s;
+  const bool full = idx < n_full;
+  const bool tail = rem != 0 && idx == n_full;
+  s.ok = full || tail;
+  s.col = full ? idx * V : (tail ? d_elems - V : 0);
+  s.lo = tail ? V - rem : 0;
+  return s;
+}
+
+// The staged copy is kept as 16-byte register quads (one LDS access each).
+template <typename T, int V>
+__device__ __forceinline__ u32x4 pack_bits(const Pack<T, V>& v) {
+  static_assert(sizeof(T) * V == 16, "staged rows are rows of 16-byte vectors");
+  u32x4 b;
+  __builtin_memcpy(&b, &v, 16);
+  return b;
+}
+template <typename T, int V>
+__device__ __forceinline__ Pack<T, V> bits_pack(const u32x4& b) {
+  Pack<T, V> v;
+  __builtin_memcpy(&v, &b, 16);
+  return v;
+}
+
+template <typename T, int V>
+__global__ void __launch_bounds__(kStagedThreads)
+rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __restrict__ beta, T* y,
+                float* __restrict__ mean_out, float* __restrict__ rstd_out, int64_t n_rows,
+                int d_elems, int C, float eps, int nv_lds) {
+  constexpr int R = kStagedRegVec;
+  constexpr int B = 8;  // vectors per thread whose loads are in flight together (16 measured slower)
+  constexpr int NW = kStagedThreads / kWave;
+  __shared__ float red[2][16];
+  extern __shared__ __attribute__((aligned(16))) unsigned char staged_bytes[];
+  u32x4* stage = reinterpret_cast<u32x4*>(staged_bytes);  // [nv_lds][kStagedThreads]
+  const int tid = static_cast<int>(threadIdx.x);
+  const int64_t D = d_elems;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  StagedSlot<V> rs[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) rs[j] = staged_slot<V>(tid + j * kStagedThreads, d_elems);
+  auto lds_slot = [&](int j) { return staged_slot<V>(tid + (R + j) * kStagedThreads, d_elems); };
+
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
+    const T* xr = x + row * D;
+    T* yr = y + row * D;
+    // ---- load: registers first, then the LDS part in batches; the sum on the way
+    Pack<T, V> reg[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) reg[j] = load_pack<T, V>(xr + rs[j].col);
+    float sum = 0.f;
+    for (int j0 = 0; j0 < nv_lds; j0 += B) {
+      Pack<T, V> pk[B];
+      StagedSlot<V> sl[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        sl[u] = lds_slot(j0 + u < nv_lds ? j0 + u : nv_lds - 1);
+        pk[u] = load_pack<T, V>(xr + sl[u].col);
+      }
+      batch_loaded<T, V, B>(pk);
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        if (j0 + u < nv_lds) {
+          stage[(j0 + u) * kStagedThreads + tid] = pack_bits<T, V>(pk[u]);
+#pragma unroll
+          for (int i = 0; i < V; ++i) sum += (sl[u].ok && i >= sl[u].lo) ? to_f32(pk[u].v[i]) : 0.f;
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) sum += (rs[j].ok && i >= rs[j].lo) ? to_f32(reg[j].v[i]) : 0.f;
+    }
+    const float mean = block_sum1(sum, red[0], NW) * inv_d;
+    // ---- second pass over the staged row: squared deviations
+    float m2 = 0.f;
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float d = (rs[j].ok && i >= rs[j].lo) ? to_f32(reg[j].v[i]) - mean : 0.f;
+        m2 += d * d;
+      }
+    }
+    for (int j = 0; j < nv_lds; ++j) {
+      const StagedSlot<V> sl = lds_slot(j);
+      const Pack<T, V> pk = bits_pack<T, V>(stage[j * kStagedThreads + tid]);
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float d = (sl.ok && i >= sl.lo) ? to_f32(pk.v[i]) - mean : 0.f;
+        m2 += d * d;
+      }
+    }
+    const float rstd = rsqrtf(block_sum1(m2, red[1], NW) * inv_d + eps);
+    if (tid == 0) {
+      mean_out[row] = mean;
+      rstd_out[row] = rstd;
+    }
+    // ---- normalise from the staged copy
+    const int c = static_cast<int>(row % C);
+    const float a = rstd * gamma[c], bs = beta[c];
+    auto emit = [&](const Pack<T, V>& pk, const StagedSlot<V>& sl) {
+      if (!sl.ok) return;
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean) * a + bs);
+      store_pack_from<T, V>(yr + sl.col, o, sl.lo);
+    };
+#pragma unroll
+    for (int j = 0; j < R; ++j) emit(reg[j], rs[j]);
+    for (int j = 0; j < nv_lds; ++j) emit(bits_pack<T, V>(stage[j * kStagedThreads + tid]), lds_slot(j));
+    // (the next row's block sums reuse red[0] only after this row's second barrier)
+  }
+}
+
+// Backward, channel-first InstanceNorm (gamma is the scalar of channel row % C): x and dy
+// staged; the row sums a = sum dy, b = sum dy * xh go to part[n][0][c] = b, part[n][1][c] = a as
+// in rows_bwd_resident.  dx may alias dy, not x.
+template <typename T, int V>
+__global__ void __launch_bounds__(kStagedThreads)
+rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
+                const float* __restrict__ mean_in, const float* __restrict__ rstd_in, T* dx,
+                float* __restrict__ part, int64_t n_rows, int d_elems, int C, int nv_lds) {
+  constexpr int R = kStagedRegVec;
+  constexpr int B = 4;
+  constexpr int NW = kStagedThreads / kWave;
+  __shared__ float2 red[2][16];
+  extern __shared__ __attribute__((aligned(16))) unsigned char staged_bytes[];
+  u32x4* stage = reinterpret_cast<u32x4*>(staged_bytes);  // [nv_lds][2][kStagedThreads]
+  const int tid = static_cast<int>(threadIdx.x);
+  const int64_t D = d_elems;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  StagedSlot<V> rs[R];
+#pragma unroll
+  for (int j = 0; j < R; ++j) rs[j] = staged_slot<V>(tid + j * kStagedThreads, d_elems);
+  auto lds_slot = [&](int j) { return staged_slot<V>(tid + (R + j) * kStagedThreads, d_elems); };
+
+  int it = 0;
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x, ++it) {
+    const T* xr = x + row * D;
+    const T* dyr = dy + row * D;
+    T* dxr = dx + row * D;
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    const int c = static_cast<int>(row % C);
+    const float gm = gamma[c];
+    Pack<T, V> rx[R], rd[R];
+#pragma unroll
+    for (int j = 0; j < R; ++j) {
+      rx[j] = load_pack<T, V>(xr + rs[j].col);
+      rd[j] = load_pack<T, V>(dyr + rs[j].col);
+    }
+    float a1 = 0.f, a2 = 0.f;
+    auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, const StagedSlot<V>& sl) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const bool ok = sl.ok && i >= sl.lo;
+        const float h = ok ? (to_f32(px.v[i]) - mean) * rstd : 0.f;
+        const float d = ok ? to_f32(pd.v[i]) : 0.f;
+        a1 += d;
+        a2 += d * h;
+      }
+    };
+    for (int j0 = 0; j0 < nv_lds; j0 += B) {
+      Pack<T, V> px[B], pd[B];
+      StagedSlot<V> sl[B];
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        sl[u] = lds_slot(j0 + u < nv_lds ? j0 + u : nv_lds - 1);
+        px[u] = load_pack<T, V>(xr + sl[u].col);
+        pd[u] = load_pack<T, V>(dyr + sl[u].col);
+      }
+      batch_loaded<T, V, B>(px, pd);
+#pragma unroll
+      for (int u = 0; u < B; ++u) {
+        if (j0 + u < nv_lds) {
+          stage[((j0 + u) * 2 + 0) * kStagedThreads + tid] = pack_bits<T, V>(px[u]);
+          stage[((j0 + u) * 2 + 1) * kStagedThreads + tid] = pack_bits<T, V>(pd[u]);
+          add(px[u], pd[u], sl[u]);
+        }
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) add(rx[j], rd[j], rs[j]);
+    const float2 s = block_sum2(a1, a2, red[it & 1], NW);
+    if (tid == 0) {
+      const int64_t n = row / C;
+      part[(n * 2 + 0) * C + c] = s.y;
+      part[(n * 2 + 1) * C + c] = s.x;
+    }
+    const float scale = rstd * gm;
+    const float ca = -scale * (s.y * inv_d), cb = -scale * (s.x * inv_d);
+    auto emit = [&](const Pack<T, V>& px, const Pack<T, V>& pd, const StagedSlot<V>& sl) {
+      if (!sl.ok) return;
+      Pack<T, V> o;
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float h = (to_f32(px.v[i]) - mean) * rstd;
+        o.v[i] = from_f32<T>(scale * to_f32(pd.v[i]) + (ca * h + cb));
+      }
+      store_pack_from<T, V>(dxr + sl.col, o, sl.lo);
+    };
+#pragma unroll
+    for (int j = 0; j < R; ++j) emit(rx[j], rd[j], rs[j]);
+    for (int j = 0; j < nv_lds; ++j) {
+      emit(bits_pack<T, V>(stage[(j * 2 + 0) * kStagedThreads + tid]), bits_pack<T, V>(stage[(j * 2 + 1) * kStagedThreads + tid]),
+           lds_slot(j));
+    }
+  }
+}
+
 // ------------------------------------------------------------- column reduction
 // out0[j] = sum_g part[g][0][j], out1[j] = sum_g part[g][1][j] for j < W, g < G, summed
 // in a fixed order (deterministic; the reference likewise uses no atomics,

@@ -132,6 +132,20 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
     return ATEXN_OK;
   }
   if constexpr (AFF && V > 1) {
+    if (p.staged) {
+      static_assert(kStagedThreads == kPlanStagedThreads && kStagedRegVec == kPlanStagedRegVec, "plan_rows sizes the staged launches");
+      // more dynamic LDS than the default limit of a launch: raised once per kernel
+      static const hipError_t raised =
+          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_fwd_staged<T, V>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve));
+      ATEXN_REQUIRE(raised == hipSuccess, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      rows_fwd_staged<T, V><<<p.grid, p.threads, p.fold_lds, st>>>(x, gamma, beta, y, mean, rstd, n_rows,
+                                                                        static_cast<int>(D), C, eps, p.nv_lds);
+      ATEXN_CHECK_LAUNCH("rows_fwd_staged");
+      return ATEXN_OK;
+    }
+  }
+  if constexpr (AFF && V > 1) {
     float2* stats = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
     split_fwd_stats<T, V><<<p.split_grid, kSplitThreads, 0, st>>>(x, stats, n_rows, D, p.S, p.chunk);
     ATEXN_CHECK_LAUNCH("split_fwd_stats");
@@ -287,6 +301,19 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
   }
   if constexpr (AFF && V > 1) {
+    if (p.staged) {
+      static const hipError_t raised =
+          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_staged<T, V>),
+                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve));
+      ATEXN_REQUIRE(raised == hipSuccess, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      if (bwd_stage_mask() & 1) {
+        rows_bwd_staged<T, V><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
+                                                                     static_cast<int>(D), C, p.nv_lds);
+        ATEXN_CHECK_LAUNCH("rows_bwd_staged");
+      }
+      if (!(bwd_stage_mask() & 2)) return ATEXN_OK;
+      return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+    }
     float2* sums = reinterpret_cast<float2*>(static_cast<char*>(ws) + p.off_pairs);
     split_bwd_sums<T, V, true><<<p.split_grid, kSplitThreads, 0, st>>>(dy, x, gamma, mean, rstd, sums, n_rows,
                                                             D, p.S, p.chunk);

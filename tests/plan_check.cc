@@ -69,6 +69,15 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
   }
   const RowsPlan p = plan_rows(kind, r.V, n_rows, D, C, cus);
   EXPECT(p.ragged == (D % r.V != 0), "ragged");
+  if (p.staged) {
+    // the row staged in registers (8 vectors per thread) and LDS, 512 threads
+    EXPECT(!p.resident && r.V > 1 && kind != RowsKind::kBwdCols && n_vec > resident_limit(kind), "staged with n_vec=%lld", (long long)n_vec);
+    EXPECT(p.threads == 512 && p.nv_lds >= 1 && int64_t(8 + p.nv_lds) * 512 >= n_vec, "staged row not covered: nv_lds=%d n_vec=%lld", p.nv_lds, (long long)n_vec);
+    EXPECT(p.fold_lds == size_t(p.nv_lds) * 512 * (kind == RowsKind::kFwd ? 16 : 32) && p.fold_lds + 512 <= 160 * 1024, "staged LDS bytes %zu", p.fold_lds);
+    EXPECT(p.grid >= 1 && p.grid <= n_rows && int64_t(p.grid) * int64_t(p.fold_lds + 512) <= int64_t(cus) * 160 * 1024, "staged grid=%d", p.grid);
+    if (kind == RowsKind::kBwdAffine) EXPECT(p.part_rows == n_rows / C && p.ws_bytes >= sizeof(float) * 2 * size_t(n_rows), "staged partial rows");
+    return;
+  }
   if (p.resident) {
     if (p.acc_lds) {
       // the LayerNorm backward with its column accumulators in LDS

@@ -44,8 +44,9 @@ def run_case(capi, coracle, N, C, S, dtype, channel_first, seed_index, stddev=1.
     rstd32 = rstd_ref.astype(np.float32)
     dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, mean32.astype(np.float64),
                                             rstd32.astype(np.float64), dtype, channel_first)
-    dx, dg, db = capi.in_bwd(util.to_device(dy, dtype), x_keep, gd, torch.from_numpy(mean32).cuda(),
-                             torch.from_numpy(rstd32).cuda(), dtype, channel_first)
+    dyd = util.to_device(dy, dtype)
+    dx, dg, db = capi.in_bwd(dyd, x_keep, gd, torch.from_numpy(mean32).cuda(),
+                             torch.from_numpy(rstd32).cuda(), dtype, channel_first, dx=dyd if in_place else None)
     torch.cuda.synchronize()
     assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx",
                  scale=util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), rstd32, dtype))
@@ -287,6 +288,24 @@ def test_channels_last_cooperative_launch_matches_two_stage(coracle, N, C, S, dt
     assert_close(util.to_host(ref[1]), m_ref, tol["stat"], "mean")
     assert_close(util.to_host(ref[2]), r_ref, tol["stat"], "inv_std")
     assert_close(util.to_host(ref[0]), y_ref, tol["y"], "y")
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,C,S,in_place", [(2, 4, 65536, False), (1, 3, 110592, False), (3, 2, 50176, True),
+                                            (2, 2, 33001, False), (1, 5, 69632, False), (1, 2, 69633, False),
+                                            (2, 3, 34816, True), (1, 2, 55299, False), (40, 16, 36864, False)])
+def test_channel_first_planes_staged_on_chip(capi, coracle, N, C, S, dtype, in_place):
+    """Planes beyond the register-resident limit that still fit one workgroup's registers plus
+    LDS make a single pass (forward up to 27 vectors per thread of 512, backward, which stages x
+    and dy, up to 17): the limits of both directions for 16-bit and float32 planes, one
+    element past them (two-stage kernels again), ragged planes, in place, and more planes than
+    workgroups.  (The planner stages rows only when there are enough of them to fill the chip;
+    the tuning hook lifts that condition here.)"""
+    assert capi.L.atexn_set_tuning(b"staged_rows", 2) == 0
+    try:
+        run_case(capi, coracle, N, C, S, dtype, True, 37, in_place=in_place)
+    finally:
+        assert capi.L.atexn_set_tuning(b"staged_rows", 1) == 0
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
