@@ -6,6 +6,8 @@
 #include "rows_kernels.cuh"
 #include "small_kernels.cuh"
 #include "tiles_kernels.cuh"
+
+#include <atomic>
 #include "status.h"
 
 namespace atexn {
@@ -22,6 +24,25 @@ using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, c
 
 // Row batching (RB > 1) exists for the vector path and rows of at most one wave; the
 // predicate-free EXACT variants exist for the vector path.
+// The kernels that keep a row (or its accumulators) in LDS ask for more dynamic LDS than a
+// launch gets by default: the limit is raised once per kernel and device.
+template <auto Kernel>
+inline hipError_t allow_large_lds() {
+  static std::atomic<uint64_t> done{0};
+  int dev = -1;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    dev = -1;
+  }
+  if (dev >= 0 && ((done.load(std::memory_order_acquire) >> dev) & 1)) return hipSuccess;
+  const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(Kernel),
+                                           hipFuncAttributeMaxDynamicSharedMemorySize,
+                                           static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve));
+  if (e == hipSuccess && dev >= 0) done.fetch_or(uint64_t(1) << dev, std::memory_order_release);
+  if (e != hipSuccess) (void)hipGetLastError();
+  return e;
+}
+
 template <typename T, int V, int TPR, int VPT, bool AFF>
 FwdResidentFn<T, V, AFF> fwd_variant(int rb, bool exact, bool ragged) {
   if constexpr (V > 1) {
@@ -134,11 +155,8 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   if constexpr (AFF && V > 1) {
     if (p.staged) {
       static_assert(kStagedThreads == kPlanStagedThreads && kStagedRegVec == kPlanStagedRegVec, "plan_rows sizes the staged launches");
-      // more dynamic LDS than the default limit of a launch: raised once per kernel
-      static const hipError_t raised =
-          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_fwd_staged<T, V>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve));
-      ATEXN_REQUIRE(raised == hipSuccess, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      const bool lds_ok = allow_large_lds<rows_fwd_staged<T, V>>() == hipSuccess;
+      ATEXN_REQUIRE(lds_ok, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
       rows_fwd_staged<T, V><<<p.grid, p.threads, p.fold_lds, st>>>(x, gamma, beta, y, mean, rstd, n_rows,
                                                                         static_cast<int>(D), C, eps, p.nv_lds);
       ATEXN_CHECK_LAUNCH("rows_fwd_staged");
@@ -266,14 +284,9 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   const int64_t W = AFF ? C : D;
   if constexpr (!AFF && V > 1) {
     if (p.acc_lds) {
-      // more dynamic LDS than the default limit of a launch: raised once per kernel
-      static const hipError_t raised[2] = {
-          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_lds<T, V, false>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve)),
-          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_lds<T, V, true>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve))};
-      ATEXN_REQUIRE(raised[0] == hipSuccess && raised[1] == hipSuccess,
-                    "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      const bool lds_ok = allow_large_lds<rows_bwd_lds<T, V, false>>() == hipSuccess &&
+                          allow_large_lds<rows_bwd_lds<T, V, true>>() == hipSuccess;
+      ATEXN_REQUIRE(lds_ok, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
       static_assert(kBwdLdsThreads == 512 && kBwdLdsVpt == 8, "plan_rows sizes rows_bwd_lds launches");
       const int stages = bwd_stage_mask();
       if (stages & 1) {
@@ -302,10 +315,8 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   }
   if constexpr (AFF && V > 1) {
     if (p.staged) {
-      static const hipError_t raised =
-          hipFuncSetAttribute(reinterpret_cast<const void*>(rows_bwd_staged<T, V>),
-                              hipFuncAttributeMaxDynamicSharedMemorySize, static_cast<int>(kPlanLdsBytes - kPlanBwdLdsReserve));
-      ATEXN_REQUIRE(raised == hipSuccess, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
+      const bool lds_ok = allow_large_lds<rows_bwd_staged<T, V>>() == hipSuccess;
+      ATEXN_REQUIRE(lds_ok, "this device does not give a workgroup %zu bytes of LDS", kPlanLdsBytes - kPlanBwdLdsReserve);
       if (bwd_stage_mask() & 1) {
         rows_bwd_staged<T, V><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
                                                                      static_cast<int>(D), C, p.nv_lds);
