@@ -12,20 +12,24 @@ pytestmark = pytest.mark.gpu
 EPS = 1e-3
 
 
-@pytest.mark.parametrize("case", ["ln_resident", "ln_tiles", "ln_small", "in_channels_last", "in_channel_first"])
+@pytest.mark.parametrize("case", ["ln_resident", "ln_tiles", "ln_small", "ln_accumulators_in_lds", "in_channels_last",
+                                  "in_channel_first", "in_channel_first_staged"])
 def test_graph_replay_matches_eager(case):
     import torch
 
     capi = util.Capi()
     dtype = "f16"
     if case.startswith("ln"):
-        N, D = {"ln_resident": (512, 1024), "ln_tiles": (6, 70001), "ln_small": (5000, 10)}[case]
+        N, D = {"ln_resident": (512, 1024), "ln_tiles": (6, 70001), "ln_small": (5000, 10),
+                "ln_accumulators_in_lds": (300, 18432)}[case]
         x, gamma, beta, dy = util.ln_inputs("plain", N, D, dtype, 30)
         fwd = lambda xd, gd, bd: capi.ln_fwd(xd, gd, bd, EPS, dtype)  # noqa: E731
         bwd = lambda dyd, xd, gd, m, r: capi.ln_bwd(dyd, xd, gd, m, r, dtype)  # noqa: E731
     else:
-        cf = case == "in_channel_first"
-        x, gamma, beta, dy = util.in_inputs(4, 32, 4096, dtype, cf, 31)
+        cf = case != "in_channels_last"
+        # (staged: 512 planes of 36864 elements, two per CU, beyond the registers)
+        N, C, S = (8, 64, 36864) if case == "in_channel_first_staged" else (4, 32, 4096)
+        x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, cf, 31)
         fwd = lambda xd, gd, bd: capi.in_fwd(xd, gd, bd, EPS, dtype, cf)  # noqa: E731
         bwd = lambda dyd, xd, gd, m, r: capi.in_bwd(dyd, xd, gd, m, r, dtype, cf)  # noqa: E731
     print(f"graph capture case={case}", flush=True)
