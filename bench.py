@@ -86,10 +86,14 @@ CASES = {
     "in_2x320x512_cl": ("in", "f16", (2, 320, 8 ** 3, False)),
     "in_2x128x4096_cl": ("in", "f16", (2, 128, 16 ** 3, False)),
     "ln_512x4096_f16": ("ln", "f16", (512, 4096)),
+    # rows of 3072 float32 vectors: the backward keeps its dgamma / dbeta accumulators in LDS
+    "ln_8192x12288_f32": ("ln", "f32", (8192, 12288)),
+    # 1024 channel-first planes of 256 x 256: staged in registers + LDS, single pass
+    "in_16x64x256x256_cf": ("in", "f16", (16, 64, 256 * 256, True)),
 }
 # cases that `--case all` leaves out (single-purpose sweeps and the reference's benchmark table)
 SWEEP_ONLY_CASES = frozenset(
-    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
+    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "in_16x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
 DEFAULT_CASE = "ln_bert"
 # the two shapes the throughput target is stated on, reported on the default run's line
 TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
