@@ -104,3 +104,56 @@ def test_instance_norm_random(coracle, seed):
     dx, dg, db = capi.in_bwd(dyd, x_keep, gd, m, r, dtype, cf, dx=dyd if seed % 2 else None)
     torch.cuda.synchronize()
     _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
+
+
+@pytest.mark.parametrize("seed", range(max(1, N_SEEDS // 2)))
+def test_rows_kept_in_lds_random(coracle, seed):
+    """The kernels that keep a row's accumulators, or part of the row itself, in LDS: LayerNorm
+    rows of 8193 .. 21000 elements (the backward's accumulator kernel takes 16-bit rows from 16385
+    and float32 rows from 8193 up to 20416 / 16384, the 2-D tiles beyond) and channel-first planes
+    of 32769 .. 111000 elements with the staging forced on (few planes), at the edges of every
+    range, ragged and misaligned."""
+    import torch
+
+    capi = util.Capi()
+    rng = np.random.Generator(np.random.PCG64(9000 + seed))
+    dtype = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+    mis = bool(rng.integers(0, 2))
+    in_place = bool(rng.integers(0, 2))
+    wrap = util.misalign if mis else (lambda t: t)
+    if seed % 2 == 0:
+        D = int(rng.choice([rng.integers(8193, 21001), 8193, 16384, 16385, 20416, 20417, 18432, 12288]))
+        N = int(rng.integers(1, 160))
+        print(f"LN long-row random seed={seed} N={N} D={D} dtype={dtype} misaligned={mis} in_place={in_place}", flush=True)
+        x, gamma, beta, dy = util.ln_inputs("row_mean", N, D, dtype, 300 + seed)
+        y_ref, m_ref, r_ref = coracle.ln_fwd(x, gamma, beta, EPS, dtype)
+        xd, dyd = wrap(util.to_device(x, dtype)), wrap(util.to_device(dy, dtype))
+        gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
+        x_keep = xd.clone() if in_place else xd
+        y, m, r = capi.ln_fwd(xd, gd, bd, EPS, dtype, y=xd if in_place else None)
+        torch.cuda.synchronize()
+        dx_ref, dg_ref, db_ref = coracle.ln_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype)
+        dx, dg, db = capi.ln_bwd(dyd, x_keep, gd, m, r, dtype, dx=dyd if in_place else None)
+        torch.cuda.synchronize()
+    else:
+        S = int(rng.choice([rng.integers(32769, 111001), 32769, 69632, 69633, 110592, 34816, 34817, 55296, 55297]))
+        # (at least four channels: a single dgamma that happens to cancel to almost nothing would
+        # be held to a tolerance relative to itself)
+        C = int(rng.integers(4, 9))
+        N = int(rng.integers(1, 4))
+        print(f"IN staged random seed={seed} N={N} C={C} spatial={S} dtype={dtype} misaligned={mis} in_place={in_place}", flush=True)
+        x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, True, 400 + seed)
+        y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, True)
+        xd, dyd = wrap(util.to_device(x, dtype)), wrap(util.to_device(dy, dtype))
+        gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
+        x_keep = xd.clone() if in_place else xd
+        assert capi.L.atexn_set_tuning(b"staged_rows", 2) == 0
+        try:
+            y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, True, y=xd if in_place else None)
+            torch.cuda.synchronize()
+            dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, True)
+            dx, dg, db = capi.in_bwd(dyd, x_keep, gd, m, r, dtype, True, dx=dyd if in_place else None)
+            torch.cuda.synchronize()
+        finally:
+            assert capi.L.atexn_set_tuning(b"staged_rows", 1) == 0
+    _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
