@@ -116,7 +116,6 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   const int rem = RAGGED ? d_elems % V : 0;
   bool vec_ok[VPT];
   int col[VPT];
-  int lo[VPT];  // RAGGED: first element of the vector that this lane owns
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = lane_r + k * tpr;
@@ -124,11 +123,19 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
     const bool tail = RAGGED && idx == n_full;
     vec_ok[k] = full || tail;
     col[k] = full ? idx * V : d_elems - V;
-    lo[k] = tail ? V - rem : 0;
   }
-  auto elem_ok = [&](int r_ok, int k, int i) -> bool {
+  // RAGGED: the last vector of a row starts at D - V and repeats the elements 0 .. lo_t - 1 of
+  // its neighbour.  It is vector k_tail of one lane of the row: the same k for every row (a
+  // scalar), lo_t = 0 in every other lane.  All vectors are summed whole, by the code of an
+  // unragged row, and under a uniform branch on k == k_tail the repeated elements are taken off
+  // again (an error of the order of the rounding those elements cause in the sums anyway); y of
+  // the repeated elements is computed and stored like every other: the same bits as the
+  // neighbour's, from the same inputs.  Per-element ownership tests and guarded stores on every
+  // vector cost the forward of [3355, 10004] 47 us instead of 32.
+  const int k_tail = RAGGED ? n_full / tpr : -1;
+  const int lo_t = (RAGGED && lane_r == n_full % tpr) ? V - rem : 0;
+  auto elem_ok = [&](int r_ok, int k) -> bool {
     if constexpr (EXACT) return true;
-    if constexpr (RAGGED) return vec_ok[k] && r_ok && i >= lo[k];
     return vec_ok[k] && r_ok;
   };
 
@@ -187,9 +194,13 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float v = elem_ok(row_ok[r], k, i) ? to_f32(cur[r][k].v[i]) : 0.f;
+          const float v = elem_ok(row_ok[r], k) ? to_f32(cur[r][k].v[i]) : 0.f;
           f[r][k * V + i] = v;
           s += v;
+        }
+        if (RAGGED && k == k_tail) {
+#pragma unroll
+          for (int i = 0; i < V - 1; ++i) s -= i < lo_t ? f[r][k * V + i] : 0.f;
         }
       }
       mean[r] = s;
@@ -210,9 +221,13 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       for (int k = 0; k < VPT; ++k) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          const float d = elem_ok(row_ok[r], k, i) ? f[r][k * V + i] - mean[r] : 0.f;
+          const float d = elem_ok(row_ok[r], k) ? f[r][k * V + i] - mean[r] : 0.f;
           f[r][k * V + i] = d;
           q += d * d;
+        }
+        if (RAGGED && k == k_tail) {
+#pragma unroll
+          for (int i = 0; i < V - 1; ++i) q -= i < lo_t ? f[r][k * V + i] * f[r][k * V + i] : 0.f;
         }
       }
       rstd[r] = q;
@@ -259,11 +274,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
             }
             o.v[i] = from_f32<T>(res);
           }
-          if constexpr (RAGGED) {
-            store_pack_from<T, V>(yr + col[k], o, lo[k]);
-          } else {
-            store_pack<T, V>(yr + col[k], o);
-          }
+          store_pack<T, V>(yr + col[k], o);
         }
       }
       if (row_ok[r] && lane_r == 0) {
@@ -382,7 +393,6 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   const int rem = RAGGED ? d_elems % V : 0;
   bool vec_ok[VPT];
   int col[VPT];
-  int lo[VPT];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = lane_r + k * tpr;
@@ -390,8 +400,14 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
     const bool tail = RAGGED && idx == n_full;
     vec_ok[k] = full || tail;
     col[k] = full ? idx * V : d_elems - V;
-    lo[k] = tail ? V - rem : 0;
   }
+  // RAGGED: as in the forward kernel, the overlapping last vector (vector k_tail, a scalar, of
+  // one lane; lo_t repeated elements there, 0 elsewhere) is summed whole and its repeated
+  // elements are taken off the row sums under a uniform branch; dx of the repeated elements is
+  // computed and stored like every other (the neighbour's bits); their dgamma / dbeta
+  // accumulators are simply not written out.
+  const int k_tail = RAGGED ? n_full / tpr : -1;
+  const int lo_t = (RAGGED && lane_r == n_full % tpr) ? V - rem : 0;
 
   float g[ROW_AFFINE ? 1 : NE];
   float acc_g[ROW_AFFINE ? 1 : NE], acc_b[ROW_AFFINE ? 1 : NE];
@@ -452,7 +468,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const int e = k * V + i;
-          const bool ok = EXACT || (vec_ok[k] && row_ok[r] && (!RAGGED || i >= lo[k]));
+          const bool ok = EXACT || (vec_ok[k] && row_ok[r]);
           const float h = ok ? (to_f32(cur.px[r][k].v[i]) - cur.mean[r]) * cur.rstd[r] : 0.f;
           const float d = ok ? to_f32(cur.pd[r][k].v[i]) : 0.f;
           xh[r][e] = h;
@@ -467,6 +483,13 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
             a2 += t * h;
             acc_g[e] += d * h;
             acc_b[e] += d;
+          }
+        }
+        if (RAGGED && k == k_tail) {
+#pragma unroll
+          for (int i = 0; i < V - 1; ++i) {
+            a1 -= i < lo_t ? gv[r][k * V + i] : 0.f;
+            a2 -= i < lo_t ? gv[r][k * V + i] * xh[r][k * V + i] : 0.f;
           }
         }
       }
@@ -513,11 +536,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
             const int e = k * V + i;
             o.v[i] = from_f32<T>(scale * gv[r][e] + (ca * xh[r][e] + cb));
           }
-          if constexpr (RAGGED) {
-            store_pack_from<T, V>(dxr + col[k], o, lo[k]);
-          } else {
-            store_pack<T, V>(dxr + col[k], o);
-          }
+          store_pack<T, V>(dxr + col[k], o);
         }
       }
     }
@@ -575,9 +594,9 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
             tg[i] = acc_g[k * V + i];
             tb[i] = acc_b[k * V + i];
           }
-          if constexpr (RAGGED) {
-            store_f32_from<V>(prow + col[k], tg, lo[k]);
-            store_f32_from<V>(prow + D + col[k], tb, lo[k]);
+          if (RAGGED && k == k_tail) {
+            store_f32_from<V>(prow + col[k], tg, lo_t);
+            store_f32_from<V>(prow + D + col[k], tb, lo_t);
           } else {
             store_f32<V>(prow + col[k], tg);
             store_f32<V>(prow + D + col[k], tb);
@@ -708,7 +727,6 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   // unpredicated loads from clamped positions, masked arithmetic (as in rows_bwd_resident)
   bool vec_ok[VPT];
   int col[VPT];
-  int lo[VPT];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = static_cast<int>(threadIdx.x) + k * bdim;
@@ -716,8 +734,14 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     const bool tail = RAGGED && idx == n_full;
     vec_ok[k] = full || tail;
     col[k] = full ? idx * V : d_elems - V;
-    lo[k] = tail ? V - rem : 0;
   }
+  // RAGGED: the overlapping last vector is vector k_tail (a scalar) of one thread, which owns
+  // only its elements lo_t .. V-1 (lo_t = 0 in every other thread).  Vector k_tail takes its sums
+  // and adds to the LDS accumulators element by element (the repeated elements' accumulators are
+  // the neighbour's), under a uniform branch; every other vector runs the code of an unragged
+  // row, and dx of the repeated elements is stored like every other (the neighbour's bits).
+  const int k_tail = RAGGED ? n_full / bdim : -1;
+  const int lo_t = (RAGGED && static_cast<int>(threadIdx.x) == n_full % bdim) ? V - rem : 0;
   float g[VPT][V];
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
@@ -725,7 +749,7 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     if (vec_ok[k]) {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        if (!RAGGED || i >= lo[k]) {
+        if (!RAGGED || k != k_tail || i >= lo_t) {
           acc[col[k] + i] = 0.f;
           acc_b[col[k] + i] = 0.f;
         }
@@ -749,28 +773,33 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       if (vec_ok[k]) {
-        float tg[V], tb[V];
-        if (!RAGGED || lo[k] == 0) {
+        if (RAGGED && k == k_tail) {
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            if (i >= lo_t) {
+              const float h = (to_f32(px[k].v[i]) - mean) * rstd;
+              const float d = to_f32(pd[k].v[i]);
+              const float t = d * g[k][i];
+              a1 += t;
+              a2 += t * h;
+              acc[col[k] + i] += d * h;
+              acc_b[col[k] + i] += d;
+            }
+          }
+        } else {
+          float tg[V], tb[V];
           load_f32<V>(acc + col[k], tg);
           load_f32<V>(acc_b + col[k], tb);
-        }
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const bool ok = !RAGGED || i >= lo[k];
-          const float h = ok ? (to_f32(px[k].v[i]) - mean) * rstd : 0.f;
-          const float d = ok ? to_f32(pd[k].v[i]) : 0.f;
-          const float t = d * g[k][i];
-          a1 += t;
-          a2 += t * h;
-          if (!RAGGED || lo[k] == 0) {
+          for (int i = 0; i < V; ++i) {
+            const float h = (to_f32(px[k].v[i]) - mean) * rstd;
+            const float d = to_f32(pd[k].v[i]);
+            const float t = d * g[k][i];
+            a1 += t;
+            a2 += t * h;
             tg[i] += d * h;
             tb[i] += d;
-          } else if (ok) {  // the overlapping last vector: its own elements only
-            acc[col[k] + i] += d * h;
-            acc_b[col[k] + i] += d;
           }
-        }
-        if (!RAGGED || lo[k] == 0) {
           store_f32<V>(acc + col[k], tg);
           store_f32<V>(acc_b + col[k], tb);
         }
@@ -798,11 +827,7 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
           const float t = to_f32(pd[k].v[i]) * g[k][i];
           o.v[i] = from_f32<T>(rstd * t + (ca * h + cb));
         }
-        if constexpr (RAGGED) {
-          store_pack_from<T, V>(dxr + col[k], o, lo[k]);
-        } else {
-          store_pack<T, V>(dxr + col[k], o);
-        }
+        store_pack<T, V>(dxr + col[k], o);
       }
     }
   }
@@ -811,20 +836,20 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     if (vec_ok[k]) {
-      float tg[V], tb[V];
-      if (!RAGGED || lo[k] == 0) {
-        load_f32<V>(acc + col[k], tg);
-        load_f32<V>(acc_b + col[k], tb);
-        store_f32<V>(prow + col[k], tg);
-        store_f32<V>(prow + D + col[k], tb);
-      } else {
+      if (RAGGED && k == k_tail) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
-          if (i >= lo[k]) {
+          if (i >= lo_t) {
             prow[col[k] + i] = acc[col[k] + i];
             prow[D + col[k] + i] = acc_b[col[k] + i];
           }
         }
+      } else {
+        float tg[V], tb[V];
+        load_f32<V>(acc + col[k], tg);
+        load_f32<V>(acc_b + col[k], tb);
+        store_f32<V>(prow + col[k], tg);
+        store_f32<V>(prow + D + col[k], tb);
       }
     }
   }
@@ -846,11 +871,14 @@ constexpr int kStagedThreads = 512;
 constexpr int kStagedRegVec = 8;
 
 // Where vector slot idx of a row lies: its first column (clamped to a valid one when the slot
-// is past the row), whether it holds data, and the first element it owns (the overlapping
-// last vector of a ragged row owns only its last D % V elements).
+// is past the row) and whether it holds data.  The last vector of a ragged row starts at D - V,
+// so its first V - D % V elements repeat the last elements of its neighbour: the sums take it
+// whole and the repeated elements are taken off again, once per row, by the thread that holds
+// it (it always sits in the LDS part: slot D / V >= 4096); the outputs of the repeated elements
+// are stored like every other, the same bits as the neighbour's from the same inputs.
 template <int V>
 struct StagedSlot {
-  int col, lo;
+  int col;
   bool ok;
 };
 template <int V>
@@ -862,7 +890,6 @@ __device__ __forceinline__ StagedSlot<V> staged_slot(int idx, int d_elems) {
   const bool tail = rem != 0 && idx == n_full;
   s.ok = full || tail;
   s.col = full ? idx * V : (tail ? d_elems - V : 0);
-  s.lo = tail ? V - rem : 0;
   return s;
 }
 
@@ -899,6 +926,11 @@ rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __rest
 #pragma unroll
   for (int j = 0; j < R; ++j) rs[j] = staged_slot<V>(tid + j * kStagedThreads, d_elems);
   auto lds_slot = [&](int j) { return staged_slot<V>(tid + (R + j) * kStagedThreads, d_elems); };
+  // ragged rows: the LDS slot of the overlapping last vector and, in the thread that holds it,
+  // the number of elements it repeats
+  const bool ragged = d_elems % V != 0;
+  const int j_tail = ragged ? (d_elems / V) / kStagedThreads - R : 0;
+  const int lo_t = (ragged && tid == (d_elems / V) % kStagedThreads) ? V - d_elems % V : 0;
 
   for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x) {
     const T* xr = x + row * D;
@@ -922,14 +954,19 @@ rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __rest
         if (j0 + u < nv_lds) {
           stage[(j0 + u) * kStagedThreads + tid] = pack_bits<T, V>(pk[u]);
 #pragma unroll
-          for (int i = 0; i < V; ++i) sum += (sl[u].ok && i >= sl[u].lo) ? to_f32(pk[u].v[i]) : 0.f;
+          for (int i = 0; i < V; ++i) sum += sl[u].ok ? to_f32(pk[u].v[i]) : 0.f;
         }
       }
     }
 #pragma unroll
     for (int j = 0; j < R; ++j) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) sum += (rs[j].ok && i >= rs[j].lo) ? to_f32(reg[j].v[i]) : 0.f;
+      for (int i = 0; i < V; ++i) sum += rs[j].ok ? to_f32(reg[j].v[i]) : 0.f;
+    }
+    if (ragged) {  // the repeated elements of the last vector, off again
+      const Pack<T, V> pk = bits_pack<T, V>(stage[j_tail * kStagedThreads + tid]);
+#pragma unroll
+      for (int i = 0; i < V - 1; ++i) sum -= i < lo_t ? to_f32(pk.v[i]) : 0.f;
     }
     const float mean = block_sum1(sum, red[0], NW) * inv_d;
     // ---- second pass over the staged row: squared deviations
@@ -938,7 +975,7 @@ rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __rest
     for (int j = 0; j < R; ++j) {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const float d = (rs[j].ok && i >= rs[j].lo) ? to_f32(reg[j].v[i]) - mean : 0.f;
+        const float d = rs[j].ok ? to_f32(reg[j].v[i]) - mean : 0.f;
         m2 += d * d;
       }
     }
@@ -947,8 +984,16 @@ rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __rest
       const Pack<T, V> pk = bits_pack<T, V>(stage[j * kStagedThreads + tid]);
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const float d = (sl.ok && i >= sl.lo) ? to_f32(pk.v[i]) - mean : 0.f;
+        const float d = sl.ok ? to_f32(pk.v[i]) - mean : 0.f;
         m2 += d * d;
+      }
+    }
+    if (ragged) {
+      const Pack<T, V> pk = bits_pack<T, V>(stage[j_tail * kStagedThreads + tid]);
+#pragma unroll
+      for (int i = 0; i < V - 1; ++i) {
+        const float d = to_f32(pk.v[i]) - mean;
+        m2 -= i < lo_t ? d * d : 0.f;
       }
     }
     const float rstd = rsqrtf(block_sum1(m2, red[1], NW) * inv_d + eps);
@@ -964,7 +1009,7 @@ rows_fwd_staged(const T* x, const float* __restrict__ gamma, const float* __rest
       Pack<T, V> o;
 #pragma unroll
       for (int i = 0; i < V; ++i) o.v[i] = from_f32<T>((to_f32(pk.v[i]) - mean) * a + bs);
-      store_pack_from<T, V>(yr + sl.col, o, sl.lo);
+      store_pack<T, V>(yr + sl.col, o);
     };
 #pragma unroll
     for (int j = 0; j < R; ++j) emit(reg[j], rs[j]);
@@ -994,6 +1039,11 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
 #pragma unroll
   for (int j = 0; j < R; ++j) rs[j] = staged_slot<V>(tid + j * kStagedThreads, d_elems);
   auto lds_slot = [&](int j) { return staged_slot<V>(tid + (R + j) * kStagedThreads, d_elems); };
+  // ragged rows: the LDS slot of the overlapping last vector and, in the thread that holds it,
+  // the number of elements it repeats
+  const bool ragged = d_elems % V != 0;
+  const int j_tail = ragged ? (d_elems / V) / kStagedThreads - R : 0;
+  const int lo_t = (ragged && tid == (d_elems / V) % kStagedThreads) ? V - d_elems % V : 0;
 
   int it = 0;
   for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x, ++it) {
@@ -1013,9 +1063,8 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
     auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, const StagedSlot<V>& sl) {
 #pragma unroll
       for (int i = 0; i < V; ++i) {
-        const bool ok = sl.ok && i >= sl.lo;
-        const float h = ok ? (to_f32(px.v[i]) - mean) * rstd : 0.f;
-        const float d = ok ? to_f32(pd.v[i]) : 0.f;
+        const float h = sl.ok ? (to_f32(px.v[i]) - mean) * rstd : 0.f;
+        const float d = sl.ok ? to_f32(pd.v[i]) : 0.f;
         a1 += d;
         a2 += d * h;
       }
@@ -1041,6 +1090,17 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
     }
 #pragma unroll
     for (int j = 0; j < R; ++j) add(rx[j], rd[j], rs[j]);
+    if (ragged) {  // the repeated elements of the last vector, off again
+      const Pack<T, V> px = bits_pack<T, V>(stage[(j_tail * 2 + 0) * kStagedThreads + tid]);
+      const Pack<T, V> pd = bits_pack<T, V>(stage[(j_tail * 2 + 1) * kStagedThreads + tid]);
+#pragma unroll
+      for (int i = 0; i < V - 1; ++i) {
+        const float h = (to_f32(px.v[i]) - mean) * rstd;
+        const float d = to_f32(pd.v[i]);
+        a1 -= i < lo_t ? d : 0.f;
+        a2 -= i < lo_t ? d * h : 0.f;
+      }
+    }
     const float2 s = block_sum2(a1, a2, red[it & 1], NW);
     if (tid == 0) {
       const int64_t n = row / C;
@@ -1057,7 +1117,7 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
         const float h = (to_f32(px.v[i]) - mean) * rstd;
         o.v[i] = from_f32<T>(scale * to_f32(pd.v[i]) + (ca * h + cb));
       }
-      store_pack_from<T, V>(dxr + sl.col, o, sl.lo);
+      store_pack<T, V>(dxr + sl.col, o);
     };
 #pragma unroll
     for (int j = 0; j < R; ++j) emit(rx[j], rd[j], rs[j]);
