@@ -727,6 +727,8 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   // unpredicated loads from clamped positions, masked arithmetic (as in rows_bwd_resident)
   bool vec_ok[VPT];
   int col[VPT];
+  int lds_col[VPT];  // where a FULL vector's accumulators sit: a multiple of V, which lets the
+                     // compiler use 16-byte LDS accesses (col[k] may be D - V)
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     const int idx = static_cast<int>(threadIdx.x) + k * bdim;
@@ -734,6 +736,7 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     const bool tail = RAGGED && idx == n_full;
     vec_ok[k] = full || tail;
     col[k] = full ? idx * V : d_elems - V;
+    lds_col[k] = idx * V;
   }
   // RAGGED: the overlapping last vector is vector k_tail (a scalar) of one thread, which owns
   // only its elements lo_t .. V-1 (lo_t = 0 in every other thread).  Vector k_tail takes its sums
@@ -747,12 +750,18 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   for (int k = 0; k < VPT; ++k) {
     load_f32<V>(gamma + col[k], g[k]);
     if (vec_ok[k]) {
+      if (RAGGED && k == k_tail && lo_t != 0) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) {
-        if (!RAGGED || k != k_tail || i >= lo_t) {
-          acc[col[k] + i] = 0.f;
-          acc_b[col[k] + i] = 0.f;
+        for (int i = 0; i < V; ++i) {
+          if (i >= lo_t) {
+            acc[col[k] + i] = 0.f;
+            acc_b[col[k] + i] = 0.f;
+          }
         }
+      } else {
+        const float zero[V] = {};
+        store_f32<V>(acc + lds_col[k], zero);
+        store_f32<V>(acc_b + lds_col[k], zero);
       }
     }
   }
@@ -773,7 +782,7 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
       if (vec_ok[k]) {
-        if (RAGGED && k == k_tail) {
+        if (RAGGED && k == k_tail && lo_t != 0) {  // the one thread that holds the last vector
 #pragma unroll
           for (int i = 0; i < V; ++i) {
             if (i >= lo_t) {
@@ -788,8 +797,8 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
           }
         } else {
           float tg[V], tb[V];
-          load_f32<V>(acc + col[k], tg);
-          load_f32<V>(acc_b + col[k], tb);
+          load_f32<V>(acc + lds_col[k], tg);
+          load_f32<V>(acc_b + lds_col[k], tb);
 #pragma unroll
           for (int i = 0; i < V; ++i) {
             const float h = (to_f32(px[k].v[i]) - mean) * rstd;
@@ -800,8 +809,8 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
             tg[i] += d * h;
             tb[i] += d;
           }
-          store_f32<V>(acc + col[k], tg);
-          store_f32<V>(acc_b + col[k], tb);
+          store_f32<V>(acc + lds_col[k], tg);
+          store_f32<V>(acc_b + lds_col[k], tb);
         }
       }
       // one vector's accumulators at a time: with the LDS reads of all eight vectors moved to
@@ -836,7 +845,7 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
 #pragma unroll
   for (int k = 0; k < VPT; ++k) {
     if (vec_ok[k]) {
-      if (RAGGED && k == k_tail) {
+      if (RAGGED && k == k_tail && lo_t != 0) {
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           if (i >= lo_t) {
@@ -846,10 +855,10 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
         }
       } else {
         float tg[V], tb[V];
-        load_f32<V>(acc + col[k], tg);
-        load_f32<V>(acc_b + col[k], tb);
-        store_f32<V>(prow + col[k], tg);
-        store_f32<V>(prow + D + col[k], tb);
+        load_f32<V>(acc + lds_col[k], tg);
+        load_f32<V>(acc_b + lds_col[k], tb);
+        store_f32<V>(prow + lds_col[k], tg);
+        store_f32<V>(prow + D + lds_col[k], tb);
       }
     }
   }
