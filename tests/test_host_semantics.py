@@ -233,6 +233,32 @@ def test_kernel_level_validation(L):
     assert b"static buffer" in L.atexn_last_error()
 
 
+def test_every_planning_parameter_is_settable(L):
+    """Each parameter of the planner (struct Tuning in csrc/plan.h) is reachable through
+    atexn_set_tuning under its own name and accepts its default; the one that runs only part of
+    a backward call exists in the benchmark build alone."""
+    import os
+    import re
+
+    plan_h = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "atex_amd", "csrc", "plan.h")
+    names = re.findall(r"^\s*TuneInt\s+(\w+)\{(\d+)\};", open(plan_h).read(), re.M)
+    assert len(names) >= 20
+    for name, default in names:
+        rc = L.atexn_set_tuning(name.encode(), int(default))
+        if name == "bwd_stage_mask":
+            assert rc == 1
+        else:
+            assert rc == 0, (name, default, L.atexn_last_error())
+    # a plan follows its parameter: planes staged on chip need no statistics workspace
+    rows = (1, 0, 16, 64, 65536)  # dtype f16, channel-first, N, C, D
+    assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
+    assert L.atexn_set_tuning(b"staged_rows", 0) == 0
+    try:
+        assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) > 0
+    finally:
+        assert L.atexn_set_tuning(b"staged_rows", 1) == 0
+
+
 def test_workspace_queries_without_gpu(L):
     """Usable on a host without a GPU (they assume 256 CUs) and monotone in the obvious way."""
     assert L.atexn_layer_norm_fwd_workspace_bytes(1, 8192, 1024) == 0       # register-resident rows
