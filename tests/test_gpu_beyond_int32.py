@@ -142,6 +142,7 @@ def _params(P, device):
     ((1 << 28) + 5, 10, "one thread per row"),
     ((1 << 18) + 1, 8200, "one workgroup per row, ragged"),
     (2, (1 << 31) + 9, "2-D tiles, a row longer than 2^31"),
+    ((1 << 17) + 7, 16390, "backward with its accumulators in LDS, ragged"),
 ])
 def test_layer_norm_beyond_int32(N, D, family):
     import torch
@@ -165,6 +166,7 @@ def test_layer_norm_beyond_int32(N, D, family):
 @pytest.mark.parametrize("N,C,D,family", [
     (512, 512, 8200, "planes in registers"),
     (2, 4, (1 << 28) + 3, "planes split over workgroups"),
+    (64, 1024, 32780, "planes staged in registers and LDS"),
 ])
 def test_instance_norm_channel_first_beyond_int32(N, C, D, family):
     import torch
