@@ -134,6 +134,10 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "bwd_waves_per_cu")) t.bwd_waves_per_cu = value;
   else if (!strcmp(name, "bwd_affine_waves_per_cu")) t.bwd_affine_waves_per_cu = value;
   else if (!strcmp(name, "bwd_min_rows")) t.bwd_min_rows = value;
+  else if (!strcmp(name, "bwd_lds_vpt")) {
+    ATEXN_REQUIRE(value == 4 || value == 8, "bwd_lds_vpt must be 4 or 8");
+    t.bwd_lds_vpt = value;
+  }
   else if (!strcmp(name, "staged_rows")) {
     ATEXN_REQUIRE(value >= 0 && value <= 2, "staged_rows must be 0, 1 or 2");
     t.staged_rows = value;

@@ -34,6 +34,7 @@ struct Tuning {
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   TuneInt staged_rows{1};            // rows beyond the registers staged in LDS, single pass (0: never, 2: however few rows)
+  TuneInt bwd_lds_vpt{4};            //   its vectors per lane: 4 (up to 640 / 1024 threads) or 8 (up to 512)
   TuneInt bwd_lds_rows{1};           // LayerNorm backward: the single-pass kernel with accumulators in LDS
   TuneInt bwd_min_rows{4};           // resident LayerNorm backward: rows per workgroup worth a partial row
   // Two-stage kernels: stage 2 walks its chunk / slab from the end (what stage 1 touched last
@@ -198,7 +199,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     p.resident = true;
     p.acc_lds = true;
     p.tpr = 0;
-    p.vpt = 8;
+    p.vpt = t.bwd_lds_vpt;
     p.threads = static_cast<int>(round_up(div_up(n_vec, p.vpt), 64));
     p.rpb = 1;
     p.rb = 1;

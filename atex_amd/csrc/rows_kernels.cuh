@@ -704,17 +704,23 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
 // LDS words and the accumulation needs no barrier; per row it reads and writes 16 * D
 // bytes of LDS per workgroup, about a sixth of the time the CU's share of the memory
 // bandwidth needs for the row.  xh and g are recomputed from the raw vectors for the dx
-// pass instead of being kept (8 vectors per lane: they would not fit).
+// pass instead of being kept.  4 vectors per lane on up to 640 (16-bit) / 1024 (float32) threads;
+// with 8 per lane on at most 512 threads a CU has too few waves ([8192, 18432] fp16 226 -> 202 us).
 // dx may alias dy, not x.
 constexpr int kBwdLdsThreads = 512;
 constexpr int kBwdLdsVpt = 8;
+// Largest workgroup of a rows_bwd_lds<.., VPT> launch: rows of at most 20416 elements (the LDS
+// limit) and 4096 vectors.  16-bit rows at 4 vectors per lane: 2552 vectors on 640 threads.
+template <int V, int VPT>
+constexpr int bwd_lds_max_threads() {
+  return VPT == 8 ? kBwdLdsThreads : (V == 8 ? 640 : 1024);
+}
 
-template <typename T, int V, bool RAGGED>
-__global__ void __launch_bounds__(kBwdLdsThreads)
+template <typename T, int V, bool RAGGED, int VPT = kBwdLdsVpt>
+__global__ void __launch_bounds__((bwd_lds_max_threads<V, VPT>()))
 rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in, T* dx,
              float* __restrict__ part, int64_t n_rows, int d_elems) {
-  constexpr int VPT = kBwdLdsVpt;
   __shared__ float2 sum_buf[2][16];
   extern __shared__ __attribute__((aligned(16))) float acc[];  // [2][d_elems rounded up to 4]
   float* const acc_b = acc + (d_elems + 3) / 4 * 4;

@@ -290,10 +290,16 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
       static_assert(kBwdLdsThreads == 512 && kBwdLdsVpt == 8, "plan_rows sizes rows_bwd_lds launches");
       const int stages = bwd_stage_mask();
       if (stages & 1) {
-        if (p.ragged) {
-          rows_bwd_lds<T, V, true><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, static_cast<int>(D));
+        const int Di = static_cast<int>(D);
+        if (p.vpt == 4) {
+          (void)allow_large_lds<rows_bwd_lds<T, V, false, 4>>();
+          (void)allow_large_lds<rows_bwd_lds<T, V, true, 4>>();
+          if (p.ragged) rows_bwd_lds<T, V, true, 4><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di);
+          else rows_bwd_lds<T, V, false, 4><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di);
+        } else if (p.ragged) {
+          rows_bwd_lds<T, V, true><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di);
         } else {
-          rows_bwd_lds<T, V, false><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, static_cast<int>(D));
+          rows_bwd_lds<T, V, false><<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows, Di);
         }
         ATEXN_CHECK_LAUNCH("rows_bwd_lds");
       }

@@ -82,7 +82,9 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
     if (p.acc_lds) {
       // the LayerNorm backward with its column accumulators in LDS
       EXPECT(kind == RowsKind::kBwdCols && r.V > 1 && n_vec > resident_limit(kind) && n_vec <= 4096, "acc_lds with n_vec=%lld", (long long)n_vec);
-      EXPECT(p.tpr == 0 && p.vpt == 8 && p.threads <= 512 && !p.exact, "acc_lds launch shape");
+      EXPECT(p.tpr == 0 && (p.vpt == 4 || p.vpt == 8) && !p.exact, "acc_lds launch shape");
+      EXPECT(p.threads <= (p.vpt == 8 ? 512 : (r.V == 8 ? 640 : 1024)) && int64_t(p.threads) * p.vpt >= n_vec,
+             "acc_lds threads=%d vpt=%d n_vec=%lld", p.threads, p.vpt, (long long)n_vec);
       EXPECT(p.fold_lds >= sizeof(float) * 2 * size_t(round_up(D, 4)) && p.fold_lds + 512 <= 160 * 1024, "acc_lds LDS bytes %zu", p.fold_lds);
       EXPECT(p.grid >= 1 && p.grid <= cus, "acc_lds grid=%d: one workgroup per CU", p.grid);
     } else {
@@ -95,7 +97,7 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
       EXPECT(int64_t(p.threads) * p.vpt >= n_vec, "row not covered: threads=%d vpt=%d n_vec=%lld", p.threads, p.vpt,
              (long long)n_vec);
       // the launch bounds of the block-per-row kernels (768 threads with 2 vectors per thread, 512 otherwise)
-      EXPECT(p.threads <= (p.vpt == 2 ? 768 : 512), "threads=%d vpt=%d exceed the kernel's launch bounds", p.threads, p.vpt);
+      if (!p.acc_lds) EXPECT(p.threads <= (p.vpt == 2 ? 768 : 512), "threads=%d vpt=%d exceed the kernel's launch bounds", p.threads, p.vpt);
     } else {
       EXPECT((p.tpr & (p.tpr - 1)) == 0 && p.tpr >= 8 && p.tpr <= 256, "tpr=%d", p.tpr);
       EXPECT(int64_t(p.tpr) * p.vpt >= n_vec, "row not covered: tpr=%d vpt=%d n_vec=%lld", p.tpr, p.vpt, (long long)n_vec);
