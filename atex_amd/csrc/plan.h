@@ -53,6 +53,7 @@ struct Tuning {
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
   TuneInt fwd_vpt2_max_vec{1024};
   TuneInt bwd_vpt2_max_vec{1536};
+  TuneInt fwd_vpt4_max_vec{3072};    // LayerNorm forward, a workgroup per row: 4 vectors per lane up to this many vectors (768 threads)
 #ifdef ATEXN_BENCH_BUILD
   // Only in the benchmark build of the library (libatex_norms_hip_bench.so): which stages of a
   // backward call over resident rows run (bit 0: the row kernel, bit 1: the column reduction),
@@ -187,7 +188,8 @@ inline SmallPlan plan_small(RowsKind kind, int V, int64_t n_rows, int64_t D, int
   return p;
 }
 
-// V: vector width in elements (see route_rows).
+// V: vector width in elements (see route_rows).  C: the channel count of a channel-first input
+// (row r takes gamma[r % C]), 0 for LayerNorm.
 inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
   const Tuning& t = tuning();
   RowsPlan p;
@@ -253,7 +255,11 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     } else {
       p.tpr = 0;
       const int vpt2_max = kind == RowsKind::kFwd ? t.fwd_vpt2_max_vec : t.bwd_vpt2_max_vec;
-      p.vpt = n_vec <= vpt2_max ? 2 : (n_vec <= 2048 ? 4 : 8);
+      // LayerNorm forward: 4 vectors per lane on up to 768 threads beat 8 on 512 ([2048, 20480]
+      // halves 35 -> 28 us); channel-first planes of that size, with no gamma / beta vectors
+      // to read, are faster with the 8 loads per lane in flight, and so is every backward
+      const int vpt4_max = kind == RowsKind::kFwd && C == 0 ? t.fwd_vpt4_max_vec.load() : 2048;
+      p.vpt = n_vec <= vpt2_max ? 2 : (n_vec <= vpt4_max ? 4 : 8);
     }
     if (p.tpr > 64) {
       p.threads = 512;

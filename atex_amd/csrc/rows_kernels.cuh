@@ -58,7 +58,7 @@ constexpr int fold_groups_per_pass() {
 // budget the compiler works against (512 VGPRs per SIMD lane / waves per SIMD).
 template <int TPR, int VPT>
 constexpr int resident_fwd_max_threads() {
-  return TPR != 0 ? 256 : (VPT == 2 ? 1024 : 512);
+  return TPR != 0 ? 256 : (VPT == 2 ? 1024 : (VPT == 4 ? 768 : 512));
 }
 template <int TPR, bool BWD_COLS, int RB, int VPT>
 constexpr int resident_bwd_max_threads() {

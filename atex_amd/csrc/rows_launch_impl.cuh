@@ -141,7 +141,7 @@ template <typename T, int V, bool AFF>
 int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
                int C, float eps, T* y, float* mean, float* rstd, void* ws, size_t ws_bytes,
                hipStream_t st) {
-  const RowsPlan p = plan_rows(RowsKind::kFwd, V, n_rows, D, C, cu_count());
+  const RowsPlan p = plan_rows(RowsKind::kFwd, V, n_rows, D, AFF ? C : 0, cu_count());
   ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && (p.ws_bytes == 0 || ws != nullptr),
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   if (p.resident) {
@@ -277,7 +277,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
                int64_t n_rows, int64_t D, int C, T* dx, float* dgamma, float* dbeta, void* ws,
                size_t ws_bytes, hipStream_t st) {
   const RowsPlan p =
-      plan_rows(AFF ? RowsKind::kBwdAffine : RowsKind::kBwdCols, V, n_rows, D, C, cu_count());
+      plan_rows(AFF ? RowsKind::kBwdAffine : RowsKind::kBwdCols, V, n_rows, D, AFF ? C : 0, cu_count());
   ATEXN_REQUIRE(ws_bytes >= p.ws_bytes && ws != nullptr,
                 "workspace too small: need %zu bytes, got %zu", p.ws_bytes, ws_bytes);
   float* part = reinterpret_cast<float*>(static_cast<char*>(ws) + p.off_part);

@@ -140,6 +140,15 @@ def test_backward_accumulators_in_lds(capi, coracle, N, D, dtype, in_place):
     run_case(capi, coracle, "plain", N, D, dtype, 19, in_place=in_place)
 
 
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,D", [(300, 24576), (33, 24571), (700, 22528), (65, 12288), (64, 12285), (3, 24584)])
+def test_forward_four_vectors_per_lane_wide(capi, coracle, N, D, dtype):
+    """Rows of 2049 .. 3072 vectors run the forward with 4 vectors per lane on up to 768
+    threads: the largest such row for either element size, ragged ends just below it, and the
+    first row that goes back to 8 vectors per lane."""
+    run_case(capi, coracle, "plain", N, D, dtype, 23)
+
+
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 @pytest.mark.parametrize("N,D", [(10, 1000000), (100, 100000), (4, 400001), (3, 1000003), (1000, 40000),
                                  (300, 33000), (2, 2 ** 20 + 7)])
