@@ -419,9 +419,10 @@ struct ClPlan {
   int64_t slab_len = 0;
   int64_t n_work = 0;
   int grid = 1;
-  // More slabs per instance than kClFoldAbove: a small launch between the two stages adds up
-  // the slab partials of every instance once (folded[N][2][C]) instead of every stage-2
-  // workgroup doing it for itself.
+  // More slabs per instance than kClFoldAbove (twice that when four or more lanes of a stage-2
+  // workgroup share a channel): a small launch between the two stages adds up the slab partials
+  // of every instance once (folded[N][2][C]) instead of every stage-2 workgroup doing it for
+  // itself.
   bool fold = false;
   bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
   int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
@@ -502,14 +503,18 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   // the elements of a register-resident slab are addressed with 32-bit offsets from its first
   // pixel
   const bool slab32 = (int64_t(16) * ppb + 1) * C < (int64_t(1) << 32);
+  // A stage-2 workgroup combines the S slab partials of its channels on fold_p lanes per
+  // channel, and in one memory round trip while a lane has at most kPlanClFoldRegs of them.
+  // Up to fold_above slabs it does so itself; beyond, a launch of its own does it once per
+  // instance (128 when four lanes share a channel, i.e. tiles of 8 vectors:
+  // [1, 64, 256^2] forward 15.9 -> 14.0 us without the extra launch).
+  const int cap = p.TPP * V;
+  const int fold_p = cap >= 256 ? 1 : std::min(64, 256 / cap);
+  const int fold_above = fold_p >= 4 ? 2 * kClFoldAbove : kClFoldAbove;
   {
-    // A stage-2 workgroup combines the S slab partials of its channels on fold_p lanes per
-    // channel, and in one memory round trip while a lane has at most kPlanClFoldRegs of them.
     // An instance small enough to be register-resident with that many slabs gets no more:
     // its launches are bound by dependent round trips, not by the number of workgroups.
-    const int cap = p.TPP * V;
-    const int fold_p = cap >= 256 ? 1 : std::min(64, 256 / cap);
-    const int64_t s_reg = std::min<int64_t>(int64_t(kPlanClFoldRegs) * fold_p, kClFoldAbove);
+    const int64_t s_reg = std::min<int64_t>(int64_t(kPlanClFoldRegs) * fold_p, fold_above);
     if (t.cl_fold_cap && slab32 && S > s_reg && div_up(round_up(div_up(D, s_reg), ppb), ppb) <= max_u) S = s_reg;
   }
   p.slab_len = round_up(div_up(D, S), ppb);
@@ -530,7 +535,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   // merge of either, folded[N][2][C]
   p.off_a = 0;
   p.off_fold = 2 * sect;
-  p.fold = p.S > kClFoldAbove && N <= 65535;
+  p.fold = p.S > fold_above && N <= 65535;
   // (the backward holds x and dy: 16 pixels per thread of both measured no better than two stages)
   if (t.cl_fused && slab32 && V > 1 && p.S == 1 && per_thread <= (bwd ? 8 : 16)) {
     p.fused = true;
