@@ -119,6 +119,17 @@ __device__ __forceinline__ void forget_derived(Pack<T, V>& v) {
 // compiler must have issued all the loads before it and cannot sink a load down to its use
 // (left alone it sometimes emits load, wait, use, load, wait, use, ... and a batch then pays
 // one memory latency per load instead of one per batch).
+// Makes the compiler wait, at this point, for the loads that a[0..N) come from (an empty asm
+// statement per value, which takes it as an operand).  Before a loop that prefetches: a wait
+// left to the first use inside the loop is counted in operations still allowed in flight as
+// seen from the loop's entry, and on the way round the loop it then holds up for the prefetch
+// that was just issued.
+template <int N>
+__device__ __forceinline__ void values_arrived(float (&a)[N]) {
+#pragma unroll
+  for (int i = 0; i < N; ++i) asm volatile("" : "+v"(a[i]));
+}
+
 template <typename T, int V, int N>
 __device__ __forceinline__ void batch_loaded(Pack<T, V> (&a)[N]) {
   static_assert(N <= 8, "at most 8 vectors per statement");

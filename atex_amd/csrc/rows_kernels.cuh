@@ -138,6 +138,13 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
     if constexpr (EXACT) return true;
     return vec_ok[k] && r_ok;
   };
+  // A workgroup per row, row not a whole number of vectors per lane: a vector slot past the row
+  // holds the row's last vector once more.  It is left out of the sums, a vector at a time, and
+  // otherwise treated like every other, its store included (the same bits to the same address
+  // as its owner's).  Stores under a condition would make the number of memory operations in
+  // flight unknown to the compiler, whose waits for the current row then also wait for the
+  // prefetched next one ([10000, 10232] halves 98.8 us against 76.0 us for [10000, 10240]).
+  constexpr bool DUP_SLOTS = !EXACT && TPR == 0;
 
   float g[GB_REGS ? NE : 1], b[GB_REGS ? NE : 1];
   if constexpr (GB_REGS) {
@@ -192,15 +199,30 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       float s = 0.f;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
+        if constexpr (DUP_SLOTS) {
+          float sv = 0.f;
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float v = elem_ok(row_ok[r], k) ? to_f32(cur[r][k].v[i]) : 0.f;
-          f[r][k * V + i] = v;
-          s += v;
-        }
-        if (RAGGED && k == k_tail) {
+          for (int i = 0; i < V; ++i) {
+            const float v = to_f32(cur[r][k].v[i]);
+            f[r][k * V + i] = v;
+            sv += v;
+          }
+          if (RAGGED && k == k_tail) {
 #pragma unroll
-          for (int i = 0; i < V - 1; ++i) s -= i < lo_t ? f[r][k * V + i] : 0.f;
+            for (int i = 0; i < V - 1; ++i) sv -= i < lo_t ? f[r][k * V + i] : 0.f;
+          }
+          s += vec_ok[k] ? sv : 0.f;
+        } else {
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const float v = elem_ok(row_ok[r], k) ? to_f32(cur[r][k].v[i]) : 0.f;
+            f[r][k * V + i] = v;
+            s += v;
+          }
+          if (RAGGED && k == k_tail) {
+#pragma unroll
+            for (int i = 0; i < V - 1; ++i) s -= i < lo_t ? f[r][k * V + i] : 0.f;
+          }
         }
       }
       mean[r] = s;
@@ -219,15 +241,30 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       float q = 0.f;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
+        if constexpr (DUP_SLOTS) {
+          float qv = 0.f;
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          const float d = elem_ok(row_ok[r], k) ? f[r][k * V + i] - mean[r] : 0.f;
-          f[r][k * V + i] = d;
-          q += d * d;
-        }
-        if (RAGGED && k == k_tail) {
+          for (int i = 0; i < V; ++i) {
+            const float d = f[r][k * V + i] - mean[r];
+            f[r][k * V + i] = d;
+            qv += d * d;
+          }
+          if (RAGGED && k == k_tail) {
 #pragma unroll
-          for (int i = 0; i < V - 1; ++i) q -= i < lo_t ? f[r][k * V + i] * f[r][k * V + i] : 0.f;
+            for (int i = 0; i < V - 1; ++i) qv -= i < lo_t ? f[r][k * V + i] * f[r][k * V + i] : 0.f;
+          }
+          q += vec_ok[k] ? qv : 0.f;
+        } else {
+#pragma unroll
+          for (int i = 0; i < V; ++i) {
+            const float d = elem_ok(row_ok[r], k) ? f[r][k * V + i] - mean[r] : 0.f;
+            f[r][k * V + i] = d;
+            q += d * d;
+          }
+          if (RAGGED && k == k_tail) {
+#pragma unroll
+            for (int i = 0; i < V - 1; ++i) q -= i < lo_t ? f[r][k * V + i] * f[r][k * V + i] : 0.f;
+          }
         }
       }
       rstd[r] = q;
@@ -259,7 +296,8 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
           load_f32<V>(gamma + col[k], tg);
           load_f32<V>(beta + col[k], tb);
         }
-        if (EXACT || (vec_ok[k] && row_ok[r])) {
+        // (a workgroup per row never sees a row past the end)
+        if (EXACT || DUP_SLOTS || (vec_ok[k] && row_ok[r])) {
           Pack<T, V> o;
 #pragma unroll
           for (int i = 0; i < V; ++i) {
@@ -313,7 +351,21 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
   } else if constexpr (PREFETCH) {
     Pack<T, V> cur[RB][VPT];
     RowAffine cur_ra;
-    if (row0 < n_rows) load_batch(row0, cur, cur_ra);
+    if (row0 < n_rows) {
+      load_batch(row0, cur, cur_ra);
+      // The first batch is waited for here, outside the loop.  Otherwise the wait sits at the
+      // batch's first use inside the loop, counted in memory operations still allowed in
+      // flight as seen from this side of the loop's entry; on the way round the loop the
+      // operations in flight there are the prefetch just issued, and that wait, needless then,
+      // holds every row up for it ([10000, 10232] halves forward 98.8 us; 76.0 us for
+      // [10000, 10240], whose instantiation happens to issue gamma / beta after the batch).
+#pragma unroll
+      for (int r = 0; r < RB; ++r) batch_loaded<T, V, VPT>(cur[r]);
+      if constexpr (GB_REGS) {
+        values_arrived(g);
+        values_arrived(b);
+      }
+    }
     for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
       Pack<T, V> nxt[RB][VPT];
       RowAffine nxt_ra;
@@ -545,10 +597,26 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   // and rows on several waves are faster peeled, [16384, 4096] 81.9 -> 76.6 us, [8192, 2048]
   // 26.6 -> 22.7 us; rows on lane groups are not, [262144, 128] 42.5 against 45.3 us.)
   constexpr bool PEELED = TPR == 0 || TPR > kWave;
+  // the first batch and gamma are waited for before the loop (see values_arrived)
+  auto first_batch_arrived = [&](Batch& t) {
+#pragma unroll
+    for (int r = 0; r < RB; ++r) {
+      batch_loaded<T, V, VPT>(t.px[r]);
+      batch_loaded<T, V, VPT>(t.pd[r]);
+    }
+    values_arrived(t.mean);
+    values_arrived(t.rstd);
+    if constexpr (ROW_AFFINE) {
+      values_arrived(t.gm);
+    } else {
+      values_arrived(g);
+    }
+  };
   if constexpr (PREFETCH && PEELED) {
     if (row0 < n_rows) {
       Batch cur;
       load_batch(row0, cur);
+      first_batch_arrived(cur);
       int it = 0;
       for (; row0 + stride < n_rows; row0 += stride, ++it) {
         Batch nxt;
@@ -560,7 +628,10 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
     }
   } else if constexpr (PREFETCH) {
     Batch cur;
-    if (row0 < n_rows) load_batch(row0, cur);
+    if (row0 < n_rows) {
+      load_batch(row0, cur);
+      first_batch_arrived(cur);
+    }
     for (int it = 0; row0 < n_rows; row0 += stride, ++it) {
       Batch nxt;
       const bool more = row0 + stride < n_rows;
