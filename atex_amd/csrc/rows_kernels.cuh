@@ -321,34 +321,10 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
       }
     }
   };
-  // Two shapes of the prefetching loop.  PEELED: a loop that always requests the next batch and
-  // the last batch after it; otherwise the request sits under a condition inside one loop, and
-  // the waits behind it, which must assume that it was not made, also wait for the next batch
-  // before the current one is finished.  Which is faster is a matter of measurement per
-  // variant (rows on lane groups: peeled, [262144, 128] forward 25.8 -> 21.6 us; a workgroup per
-  // row: not peeled, [16384, 4096] forward 43.8 against 62.5 us peeled).
-  constexpr bool PEELED = TPR != 0;
-  if constexpr (PREFETCH && PEELED) {
-    if (row0 < n_rows) {
-      Pack<T, V> cur[RB][VPT];
-      RowAffine cur_ra;
-      load_batch(row0, cur, cur_ra);
-      int it = 0;
-      for (; row0 + stride < n_rows; row0 += stride, ++it) {
-        Pack<T, V> nxt[RB][VPT];
-        RowAffine nxt_ra;
-        load_batch(row0 + stride, nxt, nxt_ra);
-        process(cur, cur_ra, row0, it);
-#pragma unroll
-        for (int r = 0; r < RB; ++r) {
-#pragma unroll
-          for (int k = 0; k < VPT; ++k) cur[r][k] = nxt[r][k];
-        }
-        cur_ra = nxt_ra;
-      }
-      process(cur, cur_ra, row0, it);
-    }
-  } else if constexpr (PREFETCH) {
+  // Prefetch: the next batch is requested, under a condition, before the current one is worked
+  // on.  (A loop that always requests and handles the last batch after it measured the same
+  // once the first batch was made to arrive before the loop, see below, and is gone.)
+  if constexpr (PREFETCH) {
     Pack<T, V> cur[RB][VPT];
     RowAffine cur_ra;
     if (row0 < n_rows) {
@@ -593,10 +569,6 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       }
     }
   };
-  // (the two shapes of the prefetching loop: see the forward kernel.  Here a workgroup per row
-  // and rows on several waves are faster peeled, [16384, 4096] 81.9 -> 76.6 us, [8192, 2048]
-  // 26.6 -> 22.7 us; rows on lane groups are not, [262144, 128] 42.5 against 45.3 us.)
-  constexpr bool PEELED = TPR == 0 || TPR > kWave;
   // the first batch and gamma are waited for before the loop (see values_arrived)
   auto first_batch_arrived = [&](Batch& t) {
 #pragma unroll
@@ -612,21 +584,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       values_arrived(g);
     }
   };
-  if constexpr (PREFETCH && PEELED) {
-    if (row0 < n_rows) {
-      Batch cur;
-      load_batch(row0, cur);
-      first_batch_arrived(cur);
-      int it = 0;
-      for (; row0 + stride < n_rows; row0 += stride, ++it) {
-        Batch nxt;
-        load_batch(row0 + stride, nxt);
-        process(cur, row0, it);
-        cur = nxt;
-      }
-      process(cur, row0, it);
-    }
-  } else if constexpr (PREFETCH) {
+  if constexpr (PREFETCH) {
     Batch cur;
     if (row0 < n_rows) {
       load_batch(row0, cur);
