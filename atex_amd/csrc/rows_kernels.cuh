@@ -800,19 +800,44 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
       }
     }
   }
-  int it = 0;
-  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x, ++it) {
+  // PREFETCH (4 vectors per lane): the next row's vectors are requested before the current row
+  // is worked on; the first row and gamma arrive before the loop (see values_arrived).  The
+  // 16-bit instantiations then sit at their register limit (168 of 170 for 640 threads) and
+  // spill 5 to 10 values; [8192, 18432] halves still 191 -> 178 us, [2048, 18432] 65 -> 59 us
+  // (requesting the row later, behind the accumulation, spills the same).  float32: no spill,
+  // and no difference either.
+  constexpr bool PREFETCH = VPT <= 4;
+  auto load_row = [&](int64_t row, Pack<T, V>(&qx)[VPT], Pack<T, V>(&qd)[VPT]) {
     const T* xr = x + row * D;
     const T* dyr = dy + row * D;
-    const float mean = mean_in[row], rstd = rstd_in[row];
-    Pack<T, V> px[VPT], pd[VPT];
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
-      px[k] = load_pack<T, V>(xr + col[k]);
-      pd[k] = load_pack<T, V>(dyr + col[k]);
+      qx[k] = load_pack<T, V>(xr + col[k]);
+      qd[k] = load_pack<T, V>(dyr + col[k]);
     }
-    batch_loaded<T, V, VPT>(px);
-    batch_loaded<T, V, VPT>(pd);
+  };
+  Pack<T, V> px[VPT], pd[VPT];
+  if constexpr (PREFETCH) {
+    if (static_cast<int64_t>(blockIdx.x) < n_rows) {
+      load_row(blockIdx.x, px, pd);
+      batch_loaded<T, V, VPT>(px);
+      batch_loaded<T, V, VPT>(pd);
+#pragma unroll
+      for (int k = 0; k < VPT; ++k) values_arrived(g[k]);
+    }
+  }
+  int it = 0;
+  for (int64_t row = blockIdx.x; row < n_rows; row += gridDim.x, ++it) {
+    const float mean = mean_in[row], rstd = rstd_in[row];
+    Pack<T, V> nx[PREFETCH ? VPT : 1], nd[PREFETCH ? VPT : 1];
+    const bool more = PREFETCH && row + gridDim.x < n_rows;
+    if constexpr (PREFETCH) {
+      if (more) load_row(row + gridDim.x, nx, nd);
+    } else {
+      load_row(row, px, pd);
+      batch_loaded<T, V, VPT>(px);
+      batch_loaded<T, V, VPT>(pd);
+    }
     float a1 = 0.f, a2 = 0.f;
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
@@ -872,6 +897,15 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
           o.v[i] = from_f32<T>(rstd * t + (ca * h + cb));
         }
         store_pack<T, V>(dxr + col[k], o);
+      }
+    }
+    if constexpr (PREFETCH) {
+      if (more) {
+#pragma unroll
+        for (int k = 0; k < VPT; ++k) {
+          px[k] = nx[k];
+          pd[k] = nd[k];
+        }
       }
     }
   }
