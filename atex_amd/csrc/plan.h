@@ -511,11 +511,23 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   const int cap = p.TPP * V;
   const int fold_p = cap >= 256 ? 1 : std::min(64, 256 / cap);
   const int fold_above = fold_p >= 4 ? 2 * kClFoldAbove : kClFoldAbove;
-  {
-    // An instance small enough to be register-resident with that many slabs gets no more:
-    // its launches are bound by dependent round trips, not by the number of workgroups.
-    const int64_t s_reg = std::min<int64_t>(int64_t(kPlanClFoldRegs) * fold_p, fold_above);
-    if (t.cl_fold_cap && slab32 && S > s_reg && div_up(round_up(div_up(D, s_reg), ppb), ppb) <= max_u) S = s_reg;
+  if (t.cl_fold_cap && slab32 && !single_pass) {
+    // An instance small enough for register-resident slabs that stage 2 can fold by itself gets
+    // no more slabs than that takes: its launches are bound by dependent round trips, and every
+    // further slab is more partials for every stage-2 workgroup to read.  The count: a workgroup
+    // per CU (a second wave of workgroups measured slower: [4, 64, 128^2] 10.7 / 13.0 us with 64
+    // slabs against 13.2 / 14.7 us with 128, [3, 64, 20000] forward 12.2 against 14.3 us), but
+    // at least as many as leave a thread 8 vectors (16 measured slower: [2, 64, 32768] forward
+    // 12.0 against 13.0 us), else max_u.
+    const int64_t one_per_cu = std::max<int64_t>(1, cus / std::max<int64_t>(N * p.CT, 1));
+    const int64_t s_fold = std::min<int64_t>(int64_t(kPlanClFoldRegs) * fold_p, fold_above);
+    for (const int u_lim : {8, max_u}) {
+      const int64_t s_try = std::max(std::min(one_per_cu, s_fold), div_up(D, int64_t(ppb) * u_lim));
+      if (s_try <= s_fold) {
+        S = std::min(S, s_try);
+        break;
+      }
+    }
   }
   p.slab_len = round_up(div_up(D, S), ppb);
   p.S = static_cast<int>(div_up(D, p.slab_len));
