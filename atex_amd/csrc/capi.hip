@@ -146,7 +146,9 @@ int atexn_set_tuning(const char* name, int value) {
     t.bwd_lds_rows = value;
   }
   else if (!strcmp(name, "split_items_per_cu")) t.split_items_per_cu = value;
+  else if (!strcmp(name, "split_bwd_items_per_cu")) t.split_bwd_items_per_cu = value;
   else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
+  else if (!strcmp(name, "cl_bwd_big_items")) t.cl_bwd_big_items = value;
   else if (!strcmp(name, "tile_items_per_cu")) t.tile_items_per_cu = value;
   else if (!strcmp(name, "fwd_rows_batch") || !strcmp(name, "bwd_rows_batch")) {
     ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),

@@ -28,8 +28,10 @@ struct Tuning {
   TuneInt bwd_waves_per_cu{8};       // resident LayerNorm backward: waves kept resident per CU
                                      //   (each block adds a partial row to the column reduction)
   TuneInt bwd_affine_waves_per_cu{32};  // resident channel-first backward (no partial rows)
-  TuneInt split_items_per_cu{2};     // split rows: (row, chunk) work items per CU
+  TuneInt split_items_per_cu{2};     // split rows: (row, chunk) work items per CU, forward
+  TuneInt split_bwd_items_per_cu{4};  //   and backward
   TuneInt cl_items_per_cu{2};        // channels-last: (n, slab, tile) work items per CU
+  TuneInt cl_bwd_big_items{1};       //   the same for the backward of tensors of 2^25 elements and more
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
@@ -320,7 +322,8 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   }
   // split rows
   const int64_t gran = int64_t(256) * V;  // one block sweep
-  const int64_t want = div_up(int64_t(cus) * t.split_items_per_cu, std::max<int64_t>(n_rows, 1));
+  const int items = kind == RowsKind::kFwd ? t.split_items_per_cu.load() : t.split_bwd_items_per_cu.load();
+  const int64_t want = div_up(int64_t(cus) * items, std::max<int64_t>(n_rows, 1));
   const int64_t max_s = std::max<int64_t>(1, D / (gran * 4));
   int64_t S = std::max<int64_t>(1, std::min<int64_t>(std::min<int64_t>(want, max_s), 1024));
   p.chunk = round_up(div_up(D, S), gran);
@@ -495,7 +498,13 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   while ((1 << p.tpp_shift) < p.TPP) ++p.tpp_shift;
   p.CT = static_cast<int>(div_up(p.CV, p.TPP));
   const int ppb = 256 / p.TPP;
-  const int64_t want = div_up(int64_t(cus) * t.cl_items_per_cu, std::max<int64_t>(N * p.CT, 1));
+  // The backward of a large tensor gets half as many slabs: every slab is a partial dgamma / dbeta
+  // row for stage 2 to fold before it can start ([8, 64, 512^2] 248 -> 224 us, [2, 128^3, 32]
+  // 229 -> 220 us, [32, 128, 128^2] 117 -> 106 us; below 2^25 elements the second workgroup per
+  // CU is worth more: [64, 64, 4096] 29.1 against 30.2 us).
+  const bool big = N * C * D >= (int64_t(1) << 25);
+  const int items = bwd && big ? t.cl_bwd_big_items.load() : t.cl_items_per_cu.load();
+  const int64_t want = div_up(int64_t(cus) * items, std::max<int64_t>(N * p.CT, 1));
   const int64_t max_s = std::max<int64_t>(1, D / (int64_t(ppb) * 4));
   // the kernels index the slab partials of an instance ([S][2][C] floats) with 32 bits
   const int64_t s_cap = std::min<int64_t>(4096, std::max<int64_t>(1, ((int64_t(1) << 31) - 1) / std::max<int64_t>(C, 1)));
