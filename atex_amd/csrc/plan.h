@@ -53,7 +53,7 @@ struct Tuning {
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
-  TuneInt fwd_vpt2_max_vec{1024};
+  TuneInt fwd_vpt2_max_vec{1536};    // LayerNorm forward, a workgroup per row: 2 vectors per lane up to this many vectors (768 threads)
   TuneInt bwd_vpt2_max_vec{1536};
   TuneInt fwd_vpt4_max_vec{3072};    // LayerNorm forward, a workgroup per row: 4 vectors per lane up to this many vectors (768 threads)
 #ifdef ATEXN_BENCH_BUILD
@@ -256,7 +256,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.vpt = n_vec <= 256 ? 2 : (n_vec <= 384 ? 3 : 2);
     } else {
       p.tpr = 0;
-      const int vpt2_max = kind == RowsKind::kFwd ? t.fwd_vpt2_max_vec : t.bwd_vpt2_max_vec;
+      // (the LayerNorm forward takes fewer vectors per lane on more threads further up than the
+      // channel-first one, here and below: [4092, 8200] halves 30.5 -> 22.9 us with 2 per lane,
+      // planes of 9000 .. 12288 halves 3 % slower)
+      const int vpt2_max = kind == RowsKind::kFwd ? (C == 0 ? t.fwd_vpt2_max_vec.load() : 1024) : t.bwd_vpt2_max_vec.load();
       // LayerNorm forward: 4 vectors per lane on up to 768 threads beat 8 on 512 ([2048, 20480]
       // halves 35 -> 28 us); channel-first planes of that size, with no gamma / beta vectors
       // to read, are faster with the 8 loads per lane in flight, and so is every backward
