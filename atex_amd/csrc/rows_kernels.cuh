@@ -60,9 +60,11 @@ template <int TPR, int VPT>
 constexpr int resident_fwd_max_threads() {
   return TPR != 0 ? 256 : (VPT == 2 ? 1024 : (VPT == 4 ? 768 : 512));
 }
-template <int TPR, bool BWD_COLS, int RB, int VPT>
+template <int TPR, bool BWD_COLS, int RB, int VPT, bool EXACT = false>
 constexpr int resident_bwd_max_threads() {
-  if (TPR == 0 && VPT == 2) return 768;
+  // (LayerNorm rows that are exactly 2 vectors per lane go up to 1024 threads: the exact
+  // instantiation fits the 128 registers that leaves a lane)
+  if (TPR == 0 && VPT == 2) return BWD_COLS && EXACT ? 1024 : 768;
   if (TPR > 64) return 512;
   return (TPR != 0 && !BWD_COLS) ? 256 : 512;
 }
@@ -393,7 +395,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // RB / EXACT / prefetch as in the forward kernel.
 template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
           bool RAGGED = false>
-__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT>()))
+__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT, EXACT>()))
 rows_bwd_resident(const T* dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* dx,
