@@ -482,6 +482,10 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   };
 
   constexpr bool PREFETCH = VPT * RB <= (TPR == 0 ? 2 : 4);
+  // A workgroup per row whose row is not a whole number of vectors per lane: as in the forward
+  // kernel, a vector slot past the row holds the row's last vector again, and is masked out of
+  // the row sums only; dx of it is stored like every other (the same bits as its owner's).
+  constexpr bool DUP_SLOTS = !EXACT && TPR == 0;
   auto process = [&](Batch& cur, int64_t row0, int it) {
     bool row_ok[RB];
 #pragma unroll
@@ -495,22 +499,25 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       float a1 = 0.f, a2 = 0.f;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
+        // DUP_SLOTS: the vector is worked on whatever it is and only its share of the row
+        // sums is dropped (its column accumulators are never written out)
+        float v1 = 0.f, v2 = 0.f;
 #pragma unroll
         for (int i = 0; i < V; ++i) {
           const int e = k * V + i;
-          const bool ok = EXACT || (vec_ok[k] && row_ok[r]);
+          const bool ok = EXACT || DUP_SLOTS || (vec_ok[k] && row_ok[r]);
           const float h = ok ? (to_f32(cur.px[r][k].v[i]) - cur.mean[r]) * cur.rstd[r] : 0.f;
           const float d = ok ? to_f32(cur.pd[r][k].v[i]) : 0.f;
           xh[r][e] = h;
           if constexpr (ROW_AFFINE) {
             gv[r][e] = d;
-            a1 += d;
-            a2 += d * h;
+            v1 += d;
+            v2 += d * h;
           } else {
             const float t = d * g[e];
             gv[r][e] = t;
-            a1 += t;
-            a2 += t * h;
+            v1 += t;
+            v2 += t * h;
             acc_g[e] += d * h;
             acc_b[e] += d;
           }
@@ -518,10 +525,12 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
         if (RAGGED && k == k_tail) {
 #pragma unroll
           for (int i = 0; i < V - 1; ++i) {
-            a1 -= i < lo_t ? gv[r][k * V + i] : 0.f;
-            a2 -= i < lo_t ? gv[r][k * V + i] * xh[r][k * V + i] : 0.f;
+            v1 -= i < lo_t ? gv[r][k * V + i] : 0.f;
+            v2 -= i < lo_t ? gv[r][k * V + i] * xh[r][k * V + i] : 0.f;
           }
         }
+        a1 += DUP_SLOTS && !vec_ok[k] ? 0.f : v1;
+        a2 += DUP_SLOTS && !vec_ok[k] ? 0.f : v2;
       }
       s1[r] = a1;
       s2[r] = a2;
@@ -559,7 +568,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       T* dxr = dx + row * D;
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        if (EXACT || (vec_ok[k] && row_ok[r])) {
+        if (EXACT || DUP_SLOTS || (vec_ok[k] && row_ok[r])) {
           Pack<T, V> o;
 #pragma unroll
           for (int i = 0; i < V; ++i) {
