@@ -168,9 +168,6 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "fwd_vpt4_max_vec")) {
     ATEXN_REQUIRE(value >= 2048 && value <= 3072, "fwd_vpt4_max_vec must be in [2048, 3072]");
     t.fwd_vpt4_max_vec = value;
-  } else if (!strcmp(name, "bwd_vpt2_exact_max_vec")) {
-    ATEXN_REQUIRE(value >= 1024 && value <= 2048, "bwd_vpt2_exact_max_vec must be in [1024, 2048]");
-    t.bwd_vpt2_exact_max_vec = value;
   } else if (!strcmp(name, "bwd_vpt2_max_vec")) {
     ATEXN_REQUIRE(value >= 1024 && value <= 1536, "bwd_vpt2_max_vec must be in [1024, 1536]");
     t.bwd_vpt2_max_vec = value;

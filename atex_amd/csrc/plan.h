@@ -55,7 +55,6 @@ struct Tuning {
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
   TuneInt fwd_vpt2_max_vec{1536};    // LayerNorm forward, a workgroup per row: 2 vectors per lane up to this many vectors (768 threads)
   TuneInt bwd_vpt2_max_vec{1536};
-  TuneInt bwd_vpt2_exact_max_vec{2048};  // LayerNorm backward, rows of a multiple of 128 vectors: 2 per lane up to here (1024 threads)
   TuneInt fwd_vpt4_max_vec{3072};    // LayerNorm forward, a workgroup per row: 4 vectors per lane up to this many vectors (768 threads)
 #ifdef ATEXN_BENCH_BUILD
   // Only in the benchmark build of the library (libatex_norms_hip_bench.so): which stages of a
@@ -266,9 +265,6 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       // to read, are faster with the 8 loads per lane in flight, and so is every backward
       const int vpt4_max = kind == RowsKind::kFwd && C == 0 ? t.fwd_vpt4_max_vec.load() : 2048;
       p.vpt = n_vec <= vpt2_max ? 2 : (n_vec <= vpt4_max ? 4 : 8);
-      // LayerNorm backward: rows that are exactly 2 vectors per lane on a whole number of waves
-      // (the instantiation without masks fits 1024 threads' registers) stay at 2 per lane
-      if (kind == RowsKind::kBwdCols && !p.ragged && n_vec <= t.bwd_vpt2_exact_max_vec && n_vec % 128 == 0) p.vpt = 2;
     }
     if (p.tpr > 64) {
       p.threads = 512;

@@ -60,11 +60,9 @@ template <int TPR, int VPT>
 constexpr int resident_fwd_max_threads() {
   return TPR != 0 ? 256 : (VPT == 2 ? 1024 : (VPT == 4 ? 768 : 512));
 }
-template <int TPR, bool BWD_COLS, int RB, int VPT, bool EXACT = false>
+template <int TPR, bool BWD_COLS, int RB, int VPT>
 constexpr int resident_bwd_max_threads() {
-  // (LayerNorm rows that are exactly 2 vectors per lane go up to 1024 threads: the exact
-  // instantiation fits the 128 registers that leaves a lane)
-  if (TPR == 0 && VPT == 2) return BWD_COLS && EXACT ? 1024 : 768;
+  if (TPR == 0 && VPT == 2) return 768;
   if (TPR > 64) return 512;
   return (TPR != 0 && !BWD_COLS) ? 256 : 512;
 }
@@ -395,7 +393,7 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // RB / EXACT / prefetch as in the forward kernel.
 template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
           bool RAGGED = false>
-__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT, EXACT>()))
+__global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT>()))
 rows_bwd_resident(const T* dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* dx,
@@ -481,7 +479,9 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
     }
   };
 
-  constexpr bool PREFETCH = VPT * RB <= (TPR == 0 ? 2 : 4);
+  // (a channel-first plane per workgroup: the launch has a workgroup per plane or nearly, no next
+  // row to request, and the extra registers cost a wave per SIMD)
+  constexpr bool PREFETCH = VPT * RB <= (TPR == 0 && ROW_AFFINE ? 2 : 4);
   // A workgroup per row whose row is not a whole number of vectors per lane: as in the forward
   // kernel, a vector slot past the row holds the row's last vector again, and is masked out of
   // the row sums only; dx of it is stored like every other (the same bits as its owner's).

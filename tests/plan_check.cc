@@ -97,7 +97,7 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
       EXPECT(int64_t(p.threads) * p.vpt >= n_vec, "row not covered: threads=%d vpt=%d n_vec=%lld", p.threads, p.vpt,
              (long long)n_vec);
       // the launch bounds of the block-per-row kernels (768 threads with 2 vectors per thread, 512 otherwise)
-      if (!p.acc_lds) EXPECT(p.threads <= (p.vpt == 2 ? (kind == RowsKind::kBwdCols && p.exact ? 1024 : 768) : (p.vpt == 4 && kind == RowsKind::kFwd ? 768 : 512)), "threads=%d vpt=%d exceed the kernel's launch bounds", p.threads, p.vpt);
+      if (!p.acc_lds) EXPECT(p.threads <= (p.vpt == 2 ? 768 : (p.vpt == 4 && kind == RowsKind::kFwd ? 768 : 512)), "threads=%d vpt=%d exceed the kernel's launch bounds", p.threads, p.vpt);
     } else {
       EXPECT((p.tpr & (p.tpr - 1)) == 0 && p.tpr >= 8 && p.tpr <= 256, "tpr=%d", p.tpr);
       EXPECT(int64_t(p.tpr) * p.vpt >= n_vec, "row not covered: tpr=%d vpt=%d n_vec=%lld", p.tpr, p.vpt, (long long)n_vec);

@@ -151,10 +151,10 @@ def test_forward_four_vectors_per_lane_wide(capi, coracle, N, D, dtype):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("N,D", [(300, 16384), (65, 14336), (130, 13312), (64, 8192), (65, 7168), (3, 6656)])
-def test_backward_two_vectors_per_lane_on_1024_threads(capi, coracle, N, D, dtype):
-    """Rows of 1537 .. 2048 vectors that are a multiple of 128 vectors run the backward with
-    exactly 2 vectors per lane on up to 1024 threads (for float32 these are 6656 .. 8192
-    elements); the other shapes here take 4 per lane."""
+def test_backward_four_vectors_per_lane(capi, coracle, N, D, dtype):
+    """Rows of 1537 .. 2048 vectors run the backward with 4 vectors per lane and the next row
+    prefetched (for float32 these are 6148 .. 8192 elements), exact multiples of the workgroup
+    and not, more rows than workgroups and fewer."""
     run_case(capi, coracle, "plain", N, D, dtype, 29)
 
 
