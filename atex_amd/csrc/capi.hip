@@ -150,7 +150,10 @@ int atexn_set_tuning(const char* name, int value) {
   else if (!strcmp(name, "cl_items_per_cu")) t.cl_items_per_cu = value;
   else if (!strcmp(name, "cl_bwd_big_items")) t.cl_bwd_big_items = value;
   else if (!strcmp(name, "tile_items_per_cu")) t.tile_items_per_cu = value;
-  else if (!strcmp(name, "fwd_rows_batch") || !strcmp(name, "bwd_rows_batch")) {
+  else if (!strcmp(name, "fwd_rows_batch_v1")) {
+    ATEXN_REQUIRE(value == 1 || value == 2 || value == 4, "fwd_rows_batch_v1 must be 1, 2 or 4");
+    t.fwd_rows_batch_v1 = value;
+  } else if (!strcmp(name, "fwd_rows_batch") || !strcmp(name, "bwd_rows_batch")) {
     ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),
                   "rows batch must be 1, 2 (or 4, forward only)");
     (name[0] == 'f' ? t.fwd_rows_batch : t.bwd_rows_batch) = value;

@@ -34,6 +34,7 @@ struct Tuning {
   TuneInt cl_bwd_big_items{1};       //   the same for the backward of tensors of 2^25 elements and more
   TuneInt tile_items_per_cu{4};      // LayerNorm long rows: (row slab, column tile) tiles per CU
   TuneInt fwd_rows_batch{4};         // resident kernels, rows <= one wave: rows per batch of a
+  TuneInt fwd_rows_batch_v1{1};      //   (forward with one vector per lane)
   TuneInt bwd_rows_batch{2};         //   lane group (fwd 1, 2, 4; bwd 1, 2; vector path only)
   TuneInt staged_rows{1};            // rows beyond the registers staged in LDS, single pass (0: never, 2: however few rows)
   TuneInt bwd_lds_vpt{4};            //   its vectors per lane: 4 (up to 640 / 1024 threads) or 8 (up to 512)
@@ -280,8 +281,11 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
         // and measured slower
         // forward: as many rows per batch as still leave the next batch prefetched (4 vectors per
         // lane in flight: [16384, 1024] halves 12.1 -> 11.1 us with 2 rows of 2 vectors against 4)
-        p.rb = kind == RowsKind::kFwd ? std::min(t.fwd_rows_batch.load(), std::max(1, 4 / p.vpt))
-                                      : (p.vpt == 1 ? t.bwd_rows_batch.load() : 1);
+        // (and with one vector per lane a single row per batch, the next one prefetched, beats
+        // four: [262144, 128] 21.6 -> 20.9 us, [1000000, 100] 84 -> 77 us)
+        const int fwd_rb = p.vpt == 1 ? t.fwd_rows_batch_v1.load()
+                                      : std::min(t.fwd_rows_batch.load(), std::max(1, 4 / p.vpt));
+        p.rb = kind == RowsKind::kFwd ? fwd_rb : (p.vpt == 1 ? t.bwd_rows_batch.load() : 1);
       }
       if (kind == RowsKind::kBwdCols) {
         // bigger blocks -> fewer partial rows for the column reduction
