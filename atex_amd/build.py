@@ -58,7 +58,7 @@ def _hipcc() -> str:
 def _deps_mtime() -> float:
     m = 0.0
     for f in os.listdir(CSRC):
-        if f.endswith((".cuh", ".h")):
+        if f.endswith(".h"):
             m = max(m, os.path.getmtime(os.path.join(CSRC, f)))
     m = max(m, os.path.getmtime(os.path.join(HERE, "..", "include", "atex_norms.h")))
     return m

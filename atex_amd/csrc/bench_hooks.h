@@ -1,0 +1,29 @@
+/* Entry points that exist only in the benchmark build of the library
+ * (libatex_norms_hip_bench.so: the product sources compiled with -DATEXN_BENCH_BUILD).  The
+ * product library exports none of them and keeps no process-wide state; bench.py and the tests
+ * that force a particular kernel family load the benchmark build for these. */
+#ifndef ATEXN_BENCH_HOOKS_H_
+#define ATEXN_BENCH_HOOKS_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* Sets one launch-planning parameter (struct Tuning in plan.h lists the names) for the whole
+ * process.  A *_workspace_bytes query and the call it sizes must run under the same settings.
+ * "bwd_stage_mask" (1: only the row kernel of a backward call, 2: only its column reduction,
+ * 3: both) is the one parameter whose non-default values give incomplete results. */
+int atexn_set_tuning(const char* name, int value);
+
+/* Text description of the kernels a backward call of the given shape launches and whether
+ * bwd_stage_mask can time its row kernel alone ("...; alone=1"). */
+int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C, int64_t D,
+                             char* out, size_t out_bytes);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

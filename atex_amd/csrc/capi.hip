@@ -6,13 +6,19 @@
 //  cc/kernels/fused_instance_norm_op.cc:328-406, :430-534) minus tensor allocation,
 // which stays with the caller.
 #include <algorithm>
+#include <atomic>
+#include <cstdio>
 #include <cstring>
+#include <exception>
 #include <mutex>
 #include <vector>
 
 #include "cpu_kernels.h"
 #include "plan.h"
 #include "status.h"
+#ifdef ATEXN_BENCH_BUILD
+#include "bench_hooks.h"
+#endif
 
 using namespace atexn;
 
@@ -77,27 +83,45 @@ int check_same_device(const atexn_tensor* first, const Ts*... rest) {
 
 constexpr int kMaxDevices = 64;
 std::mutex g_scratch_mutex;
-void* g_scratch_ptr[kMaxDevices] = {};
+std::atomic<void*> g_scratch_ptr[kMaxDevices];
 
-// Address of `scratch` on the current device (looked up on the first call per device).
+// Address of `scratch` on the current device: looked up once per device (under the lock), read
+// with one atomic load afterwards.
 int static_scratch(void** out) {
   int dev = -1;
   hipError_t e = hipGetDevice(&dev);
   if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "hipGetDevice: %s", hipGetErrorString(e));
   ATEXN_REQUIRE(dev >= 0 && dev < kMaxDevices, "device ordinal %d not supported (limit %d)", dev,
                 kMaxDevices);
-  std::lock_guard<std::mutex> lock(g_scratch_mutex);
-  if (g_scratch_ptr[dev] == nullptr) {
-    void* p = nullptr;
-    e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
-    if (e != hipSuccess || p == nullptr) {
-      (void)hipGetLastError();
-      return set_error(ATEXN_LAUNCH_ERROR, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
-                       hipGetErrorString(e));
+  void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+  if (p == nullptr) {
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+    if (p == nullptr) {
+      e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+      if (e != hipSuccess || p == nullptr) {
+        (void)hipGetLastError();
+        return set_error(ATEXN_LAUNCH_ERROR, "hipGetSymbolAddress(scratch) on device %d: %s", dev,
+                         hipGetErrorString(e));
+      }
+      g_scratch_ptr[dev].store(p, std::memory_order_release);
     }
-    g_scratch_ptr[dev] = p;
   }
-  *out = g_scratch_ptr[dev];
+  *out = p;
+  return ATEXN_OK;
+}
+
+// The host kernels start threads and allocate: whatever they throw (std::system_error when a
+// thread cannot be created, std::bad_alloc) stops here and becomes a status.
+template <typename F>
+int guarded_cpu_call(const char* what, F&& f) {
+  try {
+    f();
+  } catch (const std::exception& e) {
+    return set_error(ATEXN_LAUNCH_ERROR, "%s: %s", what, e.what());
+  } catch (...) {
+    return set_error(ATEXN_LAUNCH_ERROR, "%s: unknown exception", what);
+  }
   return ATEXN_OK;
 }
 
@@ -117,14 +141,16 @@ const char* atexn_status_string(int status) {
 const char* atexn_last_error(void) { return last_error(); }
 int atexn_abi_version(void) { return kAbiVersion; }
 
-/* Debugging / benchmarking hook (declared in the header): sets a launch-planning parameter by
- * name for the whole process.  Returns ATEXN_INVALID_ARGUMENT for an unknown name or a value
- * out of range.  Every setting computes complete, correct results; the one switch that does
- * not (running only part of a backward call) exists in the benchmark build alone. */
+#ifdef ATEXN_BENCH_BUILD
+/* ------------------------------------------------------ benchmark build only (bench_hooks.h) */
+
+/* Sets a launch-planning parameter by name for the whole process.  Returns
+ * ATEXN_INVALID_ARGUMENT for an unknown name or a value out of range.  Every setting but
+ * bwd_stage_mask != 3 computes complete, correct results. */
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_coop") || !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -157,11 +183,9 @@ int atexn_set_tuning(const char* name, int value) {
     ATEXN_REQUIRE(value == 1 || value == 2 || (value == 4 && name[0] == 'f'),
                   "rows batch must be 1, 2 (or 4, forward only)");
     (name[0] == 'f' ? t.fwd_rows_batch : t.bwd_rows_batch) = value;
-#ifdef ATEXN_BENCH_BUILD
   } else if (!strcmp(name, "bwd_stage_mask")) {
     ATEXN_REQUIRE(value >= 1 && value <= 3, "bwd_stage_mask must be 1, 2 or 3");
     t.bwd_stage_mask = value;
-#endif
   } else if (!strcmp(name, "bwd_wave_groups")) {
     ATEXN_REQUIRE(value == 1 || value == 2, "bwd_wave_groups must be 1 (on) or 2 (off)");
     t.bwd_wave_groups = value == 1;
@@ -186,9 +210,6 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "cl_fold_cap")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_fold_cap must be 0 or 1");
     t.cl_fold_cap = value;
-  } else if (!strcmp(name, "cl_coop")) {
-    ATEXN_REQUIRE(value == 0 || value == 1, "cl_coop must be 0 or 1");
-    t.cl_coop = value;
   } else if (!strcmp(name, "reverse_second_pass")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "reverse_second_pass must be 0 or 1");
     t.reverse_second_pass = value;
@@ -196,6 +217,49 @@ int atexn_set_tuning(const char* name, int value) {
   else return set_error(ATEXN_INVALID_ARGUMENT, "unknown tuning parameter '%s'", name);
   return ATEXN_OK;
 }
+
+/* Which kernels a backward call of this shape launches, as text: the row / plane kernel family,
+ * its launch geometry, and whether a separate column reduction follows (the part that
+ * bwd_stage_mask = 1 leaves out).  op: 0 LayerNorm [N, D] (C ignored), 1 InstanceNorm.  Returns
+ * the length written (0 on a bad argument). */
+int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C, int64_t D,
+                             char* out, size_t out_bytes) {
+  if (!out || out_bytes == 0 || !dtype_ok(dtype) || N <= 0 || D <= 0 || (op == 1 && C <= 0)) return 0;
+  const int vec = 16 / elem_size(dtype);
+  const int cus = cu_count();
+  int n = 0;
+  if (op == 1 && layout == ATEXN_LAYOUT_N_C) {
+    const ClPlan p = plan_cl(true, C >= vec ? vec : 1, N, C, D, cus);
+    if (p.fused)
+      n = snprintf(out, out_bytes, "cl_bwd_fused (u=%d, grid %lld x %d)%s; alone=0", p.fused_u, (long long)N,
+                   p.CT, N > 1 ? " + col_reduce" : "");
+    else
+      n = snprintf(out, out_bytes, "cl_bwd_sums + %scl_bwd_apply (S=%d slabs, tiles=%d, U=%d); alone=0",
+                   p.fold ? "col_reduce + " : "", p.S, p.CT, p.U);
+  } else {
+    const bool affine = op == 1;
+    const RowsKind kind = affine ? RowsKind::kBwdAffine : RowsKind::kBwdCols;
+    const int64_t rows = affine ? N * C : N;
+    const RowsRoute r = route_rows(kind, !affine, vec, rows, D);
+    if (r.small) {
+      n = snprintf(out, out_bytes, "small_bwd + col_reduce; alone=1");
+    } else if (r.tiles) {
+      const TilePlan p = plan_tiles(true, vec, rows, D, cus);
+      n = snprintf(out, out_bytes, "tile_bwd_sums + merge_row_sums + tile_bwd_apply%s; alone=0",
+                   p.sums_RS > 1 ? " + col_reduce" : "");
+    } else {
+      const RowsPlan p = plan_rows(kind, r.V, rows, D, affine ? static_cast<int>(C) : 0, cus);
+      const char* k = p.acc_lds ? "rows_bwd_lds" : p.staged ? "rows_bwd_staged" : p.resident ? "rows_bwd_resident" : "";
+      if (k[0])
+        n = snprintf(out, out_bytes, "%s (grid %d x %d threads, tpr=%d vpt=%d rb=%d) + col_reduce over %d partial rows; alone=1",
+                     k, p.grid, p.threads, p.tpr, p.vpt, p.rb, p.part_rows);
+      else
+        n = snprintf(out, out_bytes, "split_bwd_sums + split_bwd_apply (S=%d chunks) + col_reduce; alone=0", p.S);
+    }
+  }
+  return n < 0 ? 0 : (static_cast<size_t>(n) < out_bytes ? n : static_cast<int>(out_bytes) - 1);
+}
+#endif  // ATEXN_BENCH_BUILD
 
 /* ------------------------------------------------------------------ kernel level */
 
@@ -334,8 +398,9 @@ int atexn_layer_norm_fwd_cpu(int dtype, const void* x, const float* gamma, const
   ATEXN_REQUIRE(N >= 0 && D >= 0, "negative size N=%lld D=%lld", (long long)N, (long long)D);
   if (N == 0 || D == 0) return ATEXN_OK;
   ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
-  cpu::layer_norm_fwd(dtype, x, gamma, beta, N, D, epsilon, y, mean, inv_std);
-  return ATEXN_OK;
+  return guarded_cpu_call("layer_norm_fwd_cpu", [&] {
+    cpu::layer_norm_fwd(dtype, x, gamma, beta, N, D, epsilon, y, mean, inv_std);
+  });
 }
 
 int atexn_layer_norm_bwd_cpu(int dtype, const void* dy, const void* x, const float* gamma,
@@ -353,8 +418,9 @@ int atexn_layer_norm_bwd_cpu(int dtype, const void* dy, const void* x, const flo
   }
   ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
   ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
-  cpu::layer_norm_bwd(dtype, dy, x, gamma, mean, inv_std, N, D, dx, dgamma, dbeta);
-  return ATEXN_OK;
+  return guarded_cpu_call("layer_norm_bwd_cpu", [&] {
+    cpu::layer_norm_bwd(dtype, dy, x, gamma, mean, inv_std, N, D, dx, dgamma, dbeta);
+  });
 }
 
 int atexn_instance_norm_fwd_cpu(int dtype, int layout, const void* x, const float* gamma,
@@ -365,9 +431,10 @@ int atexn_instance_norm_fwd_cpu(int dtype, int layout, const void* x, const floa
   ATEXN_REQUIRE(N >= 0 && C >= 0 && D >= 0, "negative size");
   if (N == 0 || C == 0 || D == 0) return ATEXN_OK;
   ATEXN_REQUIRE(x && gamma && beta && y && mean && inv_std, "NULL pointer argument");
-  cpu::instance_norm_fwd(dtype, layout == ATEXN_LAYOUT_NC_, x, gamma, beta, N, C, D, epsilon, y, mean,
-                         inv_std);
-  return ATEXN_OK;
+  return guarded_cpu_call("instance_norm_fwd_cpu", [&] {
+    cpu::instance_norm_fwd(dtype, layout == ATEXN_LAYOUT_NC_, x, gamma, beta, N, C, D, epsilon, y, mean,
+                           inv_std);
+  });
 }
 
 int atexn_instance_norm_bwd_cpu(int dtype, int layout, const void* dy, const void* x,
@@ -387,9 +454,10 @@ int atexn_instance_norm_bwd_cpu(int dtype, int layout, const void* dy, const voi
   }
   ATEXN_REQUIRE(dy && x && gamma && mean && inv_std && dx && dgamma && dbeta, "NULL pointer argument");
   ATEXN_REQUIRE(dx != x, "dx must not alias x (it may alias dy)");
-  cpu::instance_norm_bwd(dtype, layout == ATEXN_LAYOUT_NC_, dy, x, gamma, mean, inv_std, N, C, D, dx,
-                         dgamma, dbeta);
-  return ATEXN_OK;
+  return guarded_cpu_call("instance_norm_bwd_cpu", [&] {
+    cpu::instance_norm_bwd(dtype, layout == ATEXN_LAYOUT_NC_, dy, x, gamma, mean, inv_std, N, C, D, dx,
+                           dgamma, dbeta);
+  });
 }
 
 /* ---------------------------------------------------------------------- op level */

@@ -16,11 +16,9 @@
 // and their use.
 #pragma once
 
-#include <hip/hip_cooperative_groups.h>
-
 #include <type_traits>
 
-#include "norm_common.cuh"
+#include "norm_common.hip.h"
 
 namespace atexn {
 
@@ -960,129 +958,6 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
             const int64_t q = rev ? flip - p : p;
             apply(load_pack_last<T, V>(x + boff + q * C), load_pack_last<T, V>(dy + boff + q * C), q);
           });
-    }
-  }
-}
-
-// ------------------------------------------------- one cooperative launch per direction
-// When every slab of the launch is register-resident and the whole grid can be co-resident on
-// the chip, the two stages run as ONE cooperative kernel: a workgroup loads its slab once,
-// publishes the slab's partials, crosses a grid-wide barrier (cooperative_groups; the runtime
-// checks co-residency at launch and owns the barrier state, so no counter needs clearing and no
-// wave spins on a workgroup that cannot be scheduled), folds the partials of its instance and
-// applies from registers.  x (and dy) are read once.  Counterpart of the reference's
-// single-kernel channels-last variant (fused_instance_norm_op.cu:1066-1165), which only takes
-// instances that fit one block's shared memory.
-// The partials are written by workgroups on other XCDs, whose L2s are not coherent with this
-// one: the barrier's device-scope release / acquire makes them visible, and they are read
-// through pointers the compiler may not assume unaliased.
-// y may alias x (dx may alias dy): a workgroup holds all of its elements before it stores any.
-// At least two waves per SIMD (two workgroups per CU): the register budget that keeps a grid
-// of two workgroups per CU co-resident.
-template <typename T, int V, int U>
-__global__ void __launch_bounds__(kClThreads, 2)
-cl_fwd_coop(const T* x, float* pstat, const float* __restrict__ gamma,
-            const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
-            float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift,
-            int64_t slab_len, float eps) {
-  __shared__ float lds[V * kClThreads];
-  __shared__ float sm_mean[kClMaxTileChannels];
-  __shared__ float sm_sc[kClMaxTileChannels];
-  __shared__ float sm_bt[kClMaxTileChannels];
-  const int CV = C / V;
-  const int TPP = 1 << tpp_shift;
-  const int cap = TPP * V;
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
-  Pack<T, V> raw[U];
-  bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
-  float mean[V], m2[V];
-  cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(g.p1 - g.p0), TPP, lds, mean, m2);
-  if (g.ch_ok && g.slot == 0) {
-    const int64_t o = ((g.n * S + g.s) * 2) * C + g.coff;
-    store_f32<V>(pstat + o, mean);
-    store_f32<V>(pstat + o + C, m2);
-  }
-  cooperative_groups::this_grid().sync();
-#pragma unroll
-  for (int u = 0; u < U; ++u) forget_derived<T, V>(raw[u]);
-  cl_fold_stats<true>(pstat, g, S, slab_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
-                rstd_out);
-  __syncthreads();
-  if (g.ch_ok) {
-    ClFwdCoef<V, false> k;
-    k.load(g, tpp_shift, sm_mean, sm_sc, sm_bt);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (ok[u]) {
-        store_pack<T, V>(y + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
-                         k.template apply<T>(raw[u]));
-      }
-    }
-  }
-}
-
-template <typename T, int V, int U>
-__global__ void __launch_bounds__(kClThreads, 2)
-cl_bwd_coop(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
-            const float* __restrict__ mean_in, const float* __restrict__ rstd_in, float* part,
-            T* dx, float* __restrict__ dgamma, float* __restrict__ dbeta, int64_t N, int64_t D,
-            int C, int S, int tpp_shift, int64_t slab_len, int cw_shift) {
-  __shared__ float lds[2 * V * kClThreads];
-  __shared__ float sm_mu[kClMaxTileChannels];
-  __shared__ float sm_sc[kClMaxTileChannels];
-  __shared__ float sm_ca[kClMaxTileChannels];
-  __shared__ float sm_cb[kClMaxTileChannels];
-  __shared__ float red_buf[2][16];
-  const int CV = C / V;
-  const int TPP = 1 << tpp_shift;
-  const int cap = TPP * V;
-  const float inv_d = 1.0f / static_cast<float>(D);
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
-  Pack<T, V> rx[U], rd[U];
-  bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-  cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
-  {
-    float mu[V], rs[V];
-#pragma unroll
-    for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
-    if (g.ch_ok) {
-      load_f32<V>(mean_in + g.n * C + g.coff, mu);
-      load_f32<V>(rstd_in + g.n * C + g.coff, rs);
-    }
-    float acc[2 * V];
-    cl_resident_sums<T, V, U>(rx, rd, ok, mu, rs, TPP, lds, acc);
-    if (g.ch_ok && g.slot == 0) {
-      float* o = part + ((g.n * S + g.s) * 2) * C + g.coff;
-      float t0[V], t1[V];
-#pragma unroll
-      for (int i = 0; i < V; ++i) {
-        t0[i] = acc[i];
-        t1[i] = acc[V + i];
-      }
-      store_f32<V>(o, t0);
-      store_f32<V>(o + C, t1);
-    }
-  }
-  cooperative_groups::this_grid().sync();
-#pragma unroll
-  for (int u = 0; u < U; ++u) {
-    forget_derived<T, V>(rx[u]);
-    forget_derived<T, V>(rd[u]);
-  }
-  __syncthreads();  // lds is free again
-  cl_fold_sums<true>(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
-               red_buf, lds, dgamma, dbeta, cw_shift);
-  if (g.ch_ok) {
-    ClBwdCoef<V, false> k;
-    k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
-#pragma unroll
-    for (int u = 0; u < U; ++u) {
-      if (ok[u]) {
-        store_pack<T, V>(dx + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
-                         k.template apply<T>(rx[u], rd[u]));
-      }
     }
   }
 }

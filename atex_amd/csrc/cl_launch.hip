@@ -1,5 +1,5 @@
 // Channels-last InstanceNorm kernels instantiated for the three storage types.
-#include "cl_launch_impl.cuh"
+#include "cl_launch_impl.hip.h"
 
 namespace atexn {
 ATEXN_INSTANTIATE_CL(float)

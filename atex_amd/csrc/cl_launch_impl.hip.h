@@ -1,34 +1,13 @@
 // Launchers for the channels-last InstanceNorm kernels, templated on the storage type.
 #pragma once
 
-#include "cl_kernels.cuh"
+#include "cl_kernels.hip.h"
 #include "plan.h"
 #include "status.h"
 
 namespace atexn {
 
-// A cooperative launch is not recorded into a stream capture here: callers that capture get
-// the two-stage kernels.
-inline bool stream_is_capturing(hipStream_t st) {
-  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
-    (void)hipGetLastError();
-    return true;
-  }
-  return status != hipStreamCaptureStatusNone;
-}
-
 static_assert(kPlanClFoldRegs == 2 * kClFoldRegs, "the planner and the kernels must agree on the fold's register limit");
-
-// True if the kernel was enqueued.  False if the runtime refused the launch (typically: more
-// workgroups than the device can hold at once); the error is cleared and the caller falls
-// back to its multi-launch path.
-inline bool launch_cooperative(const void* fn, dim3 grid, int threads, void** args, hipStream_t st) {
-  const hipError_t e = hipLaunchCooperativeKernel(fn, grid, dim3(threads), args, 0, st);
-  if (e == hipSuccess) return true;
-  (void)hipGetLastError();
-  return false;
-}
 
 template <typename T, int V>
 int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64_t C, int64_t D,
@@ -90,20 +69,6 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
 #undef ATEXN_CL_FWD_FUSED
       ATEXN_CHECK_LAUNCH("cl_fwd_fused");
       return ATEXN_OK;
-    }
-    if (p.coop && !stream_is_capturing(st)) {
-      const T* xa = x;
-      float* ps = pstat;
-      T* ya = y;
-      int64_t Da = D, sl = p.slab_len;
-      int Ca = Ci, Sa = p.S, sh = p.tpp_shift;
-      float ea = eps;
-      void* args[] = {&xa, &ps, &gamma, &beta, &ya, &mean, &rstd, &Da, &Ca, &Sa, &sh, &sl, &ea};
-      const void* fn = p.U == 4    ? reinterpret_cast<const void*>(cl_fwd_coop<T, V, 4>)
-                       : p.U == 8  ? reinterpret_cast<const void*>(cl_fwd_coop<T, V, 8>)
-                                   : reinterpret_cast<const void*>(cl_fwd_coop<T, V, 16>);
-      if (launch_cooperative(fn, grid, kClThreads, args, st)) return ATEXN_OK;
-      // refused (the grid cannot be co-resident here): the two-stage kernels below
     }
     // a channel count that is not a multiple of V: the last channel vector of a pixel overlaps
     // its neighbour and owns only its last C % V elements
@@ -190,18 +155,6 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       ATEXN_CHECK_LAUNCH("cl_bwd_fused");
       if (N > 1) return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N), C, st);
       return ATEXN_OK;
-    }
-    if (p.coop && !stream_is_capturing(st)) {
-      const T* dya = dy;
-      const T* xa = x;
-      float* pa = part;
-      T* dxa = dx;
-      int64_t Na = N, Da = D, sl = p.slab_len;
-      int Ca = Ci, Sa = p.S, sh = p.tpp_shift, cws = cw_shift;
-      void* args[] = {&dya, &xa, &gamma, &mean, &rstd, &pa, &dxa, &dgamma, &dbeta, &Na, &Da, &Ca, &Sa, &sh, &sl, &cws};
-      const void* fn = p.U == 4 ? reinterpret_cast<const void*>(cl_bwd_coop<T, V, 4>)
-                                : reinterpret_cast<const void*>(cl_bwd_coop<T, V, 8>);
-      if (launch_cooperative(fn, grid, kClThreads, args, st)) return ATEXN_OK;
     }
     if (C % V != 0) {
       if (p.U == 4) { ATEXN_CL_BWD(4, true); return ATEXN_OK; }

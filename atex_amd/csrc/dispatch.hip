@@ -4,9 +4,9 @@
 #include <cstdio>
 #include <cstring>
 
-#include "norm_common.cuh"
+#include "norm_common.hip.h"
 #include "plan.h"
-#include "rows_kernels.cuh"
+#include "rows_kernels.hip.h"
 #include "status.h"
 
 namespace atexn {
@@ -26,10 +26,17 @@ int set_error(int code, const char* fmt, ...) {
 
 const char* last_error() { return g_last_error; }
 
+#ifdef ATEXN_BENCH_BUILD
 Tuning& tuning() {
   static Tuning t;
   return t;
 }
+#else
+const Tuning& tuning() {
+  static const Tuning t;
+  return t;
+}
+#endif
 
 int cu_count() {
   static std::atomic<int> cached[64];

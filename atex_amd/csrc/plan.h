@@ -17,11 +17,22 @@
 
 namespace atexn {
 
-// Launch-planning parameters (process-wide; defaults chosen by measurement on MI355X).  They are
-// only ever changed through atexn_set_tuning, a debugging / benchmarking hook; each is an atomic
-// so that a change made while other threads plan launches is a clean switch, not a data race.
-// (A workspace query and the call it sizes must still see the same values.)
+// Launch-planning parameters; the defaults were chosen by measurement on MI355X.  In the
+// product library they are constants: it keeps no process-wide state, and a workspace query and
+// the call it sizes always see the same plan.  Only the benchmark build of the library
+// (-DATEXN_BENCH_BUILD, libatex_norms_hip_bench.so) can change them, through atexn_set_tuning,
+// for A/B measurements and for tests that force a particular kernel family; there each is an
+// atomic so that a change made while other threads plan launches is a clean switch.
+#ifdef ATEXN_BENCH_BUILD
 using TuneInt = std::atomic<int>;
+#else
+struct TuneInt {
+  int v;
+  constexpr TuneInt(int x) : v(x) {}
+  constexpr int load() const { return v; }
+  constexpr operator int() const { return v; }
+};
+#endif
 struct Tuning {
   TuneInt fwd_waves_per_cu{16};      // resident forward: waves kept resident per CU
   TuneInt bwd_ln_threads{512};       // resident LayerNorm backward, rows <= one wave: block size
@@ -47,10 +58,6 @@ struct Tuning {
   TuneInt cl_fold_cap{1};     // channels-last: no more slabs than a stage-2 fold takes from registers
   TuneInt cl_fused_split{1};  // channels-last single pass: narrower channel tiles so that an instance fits
   TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
-  // channels-last: both stages in one cooperative launch when every slab is register-resident
-  // and the grid fits the chip at once.  Off: the grid-wide barrier of the cooperative-groups
-  // runtime measured 50 us on MI355X (the whole two-stage forward takes 15 us).
-  TuneInt cl_coop{0};
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
@@ -65,7 +72,11 @@ struct Tuning {
   TuneInt bwd_stage_mask{3};
 #endif
 };
+#ifdef ATEXN_BENCH_BUILD
 Tuning& tuning();
+#else
+const Tuning& tuning();
+#endif
 inline int bwd_stage_mask() {
 #ifdef ATEXN_BENCH_BUILD
   return tuning().bwd_stage_mask;
@@ -153,7 +164,7 @@ struct RowsRoute {
   bool tiles = false;
   bool small = false;
 };
-// LDS of the LayerNorm backward's fold: same constants as rows_kernels.cuh
+// LDS of the LayerNorm backward's fold: same constants as rows_kernels.hip.h
 constexpr int kPlanFoldLdsBytes = 64 * 1024;
 constexpr int kPlanFoldMaxWaves = 8;
 constexpr int kPlanSmallMaxVec = 4;
@@ -351,7 +362,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
   return p;
 }
 
-// LayerNorm rows too long for registers: 2-D tiles of R rows x CW columns (tiles_kernels.cuh).
+// LayerNorm rows too long for registers: 2-D tiles of R rows x CW columns (tiles_kernels.hip.h).
 // The forward statistics still come from the chunked stage 1 of the split path (S chunks).
 struct TilePlan {
   int V = 1;
@@ -439,14 +450,10 @@ struct ClPlan {
   bool fold = false;
   bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
   int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
-  // Several register-resident slabs per instance, few enough workgroups to be on the chip
-  // together: candidates for the single cooperative launch (the runtime has the last word on
-  // co-residency; the two-stage kernels remain the fallback, on the same workspace).
-  bool coop = false;
   size_t off_a = 0, off_fold = 0, ws_bytes = 0;
 };
 constexpr int kClFoldAbove = 64;
-// slab partials per lane that a stage-2 fold takes in one round trip (cl_kernels.cuh: twice
+// slab partials per lane that a stage-2 fold takes in one round trip (cl_kernels.hip.h: twice
 // kClFoldRegs)
 constexpr int kPlanClFoldRegs = 32;
 
@@ -572,8 +579,6 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
     p.fused = true;
     p.fused_u = std::max(1, pow2_ceil(per_thread));
   }
-  p.coop = t.cl_coop && !p.fused && !p.fold && V > 1 && C % V == 0 && p.S > 1 && p.U > 0 &&
-           p.n_work <= int64_t(cus) * 4;
   p.ws_bytes = p.off_fold + align256(sizeof(float) * 2 * size_t(N) * size_t(C));
   return p;
 }

@@ -10,12 +10,12 @@
 //     the registers, each pass one all-reduce across the row's lanes (DPP, LDS across waves);
 //   * "split" kernels for channel-first planes that do not fit: a row is cut into S
 //     chunks, stage 1 writes per-chunk partials, stage 2 merges them and applies
-//     (LayerNorm rows that do not fit go to tiles_kernels.cuh, many tiny rows to
-//     small_kernels.cuh).
+//     (LayerNorm rows that do not fit go to tiles_kernels.hip.h, many tiny rows to
+//     small_kernels.hip.h).
 // All of them use 16-byte accesses at element alignment; rows may have any length.
 #pragma once
 
-#include "norm_common.cuh"
+#include "norm_common.hip.h"
 
 namespace atexn {
 

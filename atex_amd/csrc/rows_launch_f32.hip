@@ -1,5 +1,5 @@
 // Contiguous-row kernels instantiated for one storage type.
-#include "rows_launch_impl.cuh"
+#include "rows_launch_impl.hip.h"
 
 namespace atexn {
 ATEXN_INSTANTIATE_ROWS(float)

@@ -3,9 +3,9 @@
 #pragma once
 
 #include "plan.h"
-#include "rows_kernels.cuh"
-#include "small_kernels.cuh"
-#include "tiles_kernels.cuh"
+#include "rows_kernels.hip.h"
+#include "small_kernels.hip.h"
+#include "tiles_kernels.hip.h"
 
 #include <atomic>
 #include "status.h"
@@ -177,7 +177,7 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
   }
 }
 
-// Many rows of at most four vectors: one thread per row (small_kernels.cuh).
+// Many rows of at most four vectors: one thread per row (small_kernels.hip.h).
 template <typename T, bool AFF>
 int small_fwd_launch(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
                      int C, float eps, T* y, float* mean, float* rstd, hipStream_t st) {
@@ -217,7 +217,7 @@ int small_bwd_launch(const T* dy, const T* x, const float* gamma, const float* m
   return launch_col_reduce(part, dgamma, dbeta, p.part_rows, AFF ? C : D, st);
 }
 
-// LayerNorm rows too long for registers, any D and alignment (tiles_kernels.cuh).
+// LayerNorm rows too long for registers, any D and alignment (tiles_kernels.hip.h).
 template <typename T>
 int tiles_fwd(const T* x, const float* gamma, const float* beta, int64_t n_rows, int64_t D,
               float eps, T* y, float* mean, float* rstd, void* ws, size_t ws_bytes,

@@ -11,7 +11,7 @@
 // twice by the same thread with the same values).  Needs D >= V.
 #pragma once
 
-#include "norm_common.cuh"
+#include "norm_common.hip.h"
 
 namespace atexn {
 

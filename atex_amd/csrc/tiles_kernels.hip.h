@@ -21,7 +21,7 @@
 //          backward  tile_bwd_sums -> merge_row_sums -> tile_bwd_apply [-> col_reduce]
 #pragma once
 
-#include "norm_common.cuh"
+#include "norm_common.hip.h"
 
 namespace atexn {
 

@@ -74,9 +74,14 @@ SIGNATURES = {
     "atexn_fused_instance_norm": (_i, [_tp, _tp, _tp, _f, ctypes.c_char_p, _tp, _tp, _tp, _vp, _sz, _vp]),
     "atexn_fused_instance_norm_grad_workspace_bytes": (_sz, [_tp, ctypes.c_char_p]),
     "atexn_fused_instance_norm_grad": (_i, [_tp, _tp, _tp, _tp, _tp, ctypes.c_char_p, _tp, _tp, _tp, _vp, _sz, _vp]),
-    # debugging / benchmarking hook
-    "atexn_set_tuning": (_i, [ctypes.c_char_p, _i]),
 }
+# the two extra entry points of the benchmark build (csrc/bench_hooks.h)
+BENCH_SIGNATURES = {
+    "atexn_set_tuning": (_i, [ctypes.c_char_p, _i]),
+    "atexn_bench_describe_bwd": (_i, [_i, _i, _i, _i64, _i64, _i64, ctypes.c_char_p, _sz]),
+}
+BENCH_LIB_PATH = LIB_PATH.replace(".so", "_bench.so")
+_bench_lib = None
 
 
 def lib() -> ctypes.CDLL:
@@ -96,10 +101,27 @@ def lib() -> ctypes.CDLL:
     return _lib
 
 
-def check(status: int) -> None:
+def bench_lib() -> ctypes.CDLL:
+    """The benchmark build of the library: the same sources plus atexn_set_tuning (launch-planning
+    parameters, process-wide) and atexn_bench_describe_bwd.  For bench.py and for tests that
+    force a particular kernel family; the product path never loads it."""
+    global _bench_lib
+    if _bench_lib is None:
+        if not os.path.exists(BENCH_LIB_PATH):
+            raise ImportError(f"{BENCH_LIB_PATH} is missing: build it with `python -m atex_amd.build`")
+        L = ctypes.CDLL(BENCH_LIB_PATH)
+        for name, (res, args) in {**SIGNATURES, **BENCH_SIGNATURES}.items():
+            fn = getattr(L, name)
+            fn.restype = res
+            fn.argtypes = args
+        _bench_lib = L
+    return _bench_lib
+
+
+def check(status: int, L=None) -> None:
     if status == ATEXN_OK:
         return
-    L = lib()
+    L = L or lib()
     msg = L.atexn_last_error().decode("utf-8", "replace")
     name = L.atexn_status_string(status).decode()
     if status == ATEXN_INVALID_ARGUMENT:

@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the fused LayerNorm / InstanceNorm forward + backward on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case NAME] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--case NAME] [--no-cpu] [--cold-only]
 
 One "step" is one forward plus one backward call of the hot path (kernel-level C ABI of
 libatex_norms_hip.so) over one batch of synthetic input that is already resident in HBM.
@@ -20,6 +20,10 @@ Output: ONE JSON line on stdout.
                reduction); every other figure comes from the product library
   targets      (default case only) the second target shape, InstanceNorm x fp16 [8,128,128,64]
                in both layouts: us per call, GB/s, fraction of peak, roofline of its backward
+  configs      (default case only) every other benchmark configuration -- the fp32 [32,1024]
+               plumbing case, the hidden-size sweep in fp16 and bf16, the 3-D volume in both
+               layouts -- each with us per call (fwd, bwd, fwd+bwd), GB/s, % of peak and torch's
+               copy / add on the same tensors as streaming references
   cpu_baseline the C oracle's float flavour (OpenMP over rows) on the same workload, timed
                on this machine's host cores; `unfused_composite` inside it is the unfused op
                sequence a framework would run instead (torch on the CPU, autograd backward)
@@ -148,27 +152,20 @@ def make_host_inputs(op, dtype, dims, seed):
     return x, gamma, beta, dy
 
 
-_BENCH_LIB = None
+# --tune given: every measurement goes through the benchmark build (the product library has no
+# launch-planning switches)
+USE_BENCH_LIB_EVERYWHERE = False
 
 
 def bench_lib():
-    """The benchmark build of the library (adds the "bwd_stage_mask" switch), or None."""
-    global _BENCH_LIB
-    if _BENCH_LIB is None:
-        import ctypes
+    """The benchmark build of the library (launch-planning switches, among them "bwd_stage_mask",
+    and the plan description), or None when it has not been built."""
+    from atex_amd.nv_norms import _capi
 
-        from atex_amd.nv_norms import _capi
-
-        path = _capi.LIB_PATH.replace(".so", "_bench.so")
-        if not os.path.exists(path):
-            return None
-        L = ctypes.CDLL(path)
-        for name, (res, args) in _capi.SIGNATURES.items():
-            fn = getattr(L, name)
-            fn.restype = res
-            fn.argtypes = args
-        _BENCH_LIB = L
-    return _BENCH_LIB
+    try:
+        return _capi.bench_lib()
+    except ImportError:
+        return None
 
 
 class GpuCase:
@@ -181,7 +178,7 @@ class GpuCase:
 
         self.torch = torch
         self.capi = _capi
-        self.L = _capi.lib()
+        self.L = bench_lib() if USE_BENCH_LIB_EVERYWHERE else _capi.lib()
         self.op, self.dtype, self.dims = op, dtype, dims
         self.code = {"f32": 0, "f16": 1, "bf16": 2}[dtype]
         tdt = {"f32": torch.float32, "f16": torch.float16, "bf16": torch.bfloat16}[dtype]
@@ -232,7 +229,7 @@ class GpuCase:
                                            s["mean"].data_ptr(), s["rstd"].data_ptr(), self.ws.data_ptr(),
                                            self.ws.numel(), self.stream)
         if st != 0:
-            self.capi.check(st)
+            self.capi.check(st, self.L)
 
     def bwd(self, i):
         s = self.sets[i % self.n_sets]
@@ -250,7 +247,7 @@ class GpuCase:
                                            N, C, D, s["dx"].data_ptr(), self.dgamma.data_ptr(),
                                            self.dbeta.data_ptr(), self.ws.data_ptr(), self.ws.numel(), self.stream)
         if st != 0:
-            self.capi.check(st)
+            self.capi.check(st, self.L)
 
     def time_loop(self, fn, steps, warmup):
         """Average milliseconds per call of fn(i), events on the launch stream."""
@@ -356,26 +353,25 @@ def composite_cpu(op, dtype, d, x, gamma, beta, dy, threads, max_seconds=8.0):
             "note": "torch CPU, unfused op sequence with autograd; composite restatement, not tf.keras"}
 
 
-def resident_rows_bwd(op, dtype, dims):
-    """Whether the backward of the case runs the register-resident row kernel followed by the
-    column reduction (rows of at most 2048 vectors for LayerNorm, planes of at most 4096 for
-    channel-first InstanceNorm; a vector is 16 bytes)."""
-    vec = 16 // ESIZE[dtype]
+def describe_bwd(op, dtype, dims):
+    """(text, alone): the kernels the backward of the case launches, from the library's own
+    planner (benchmark build), and whether its row kernel can be timed without the column
+    reduction that follows it."""
+    import ctypes
+
+    LB = bench_lib()
+    if LB is None:
+        return "backward call (benchmark build of the library missing: no plan description)", False
+    buf = ctypes.create_string_buffer(512)
+    code = {"f32": 0, "f16": 1, "bf16": 2}[dtype]
     if op == "ln":
-        return dims[1] <= 2048 * vec
-    return bool(dims[3]) and dims[2] <= 4096 * vec
-
-
-def roofline_kernel(op, dtype, dims, alone):
-    if op == "in" and not dims[3]:
-        return "cl_bwd_sums + cl_bwd_apply (channels-last backward, the whole call)"
-    if op == "in" and not resident_rows_bwd(op, dtype, dims):
-        return "split_bwd_sums + split_bwd_apply + col_reduce (backward of planes too long for registers, the whole call)"
-    if op == "ln" and not resident_rows_bwd(op, dtype, dims):
-        return "tile_bwd_sums + merge_row_sums + tile_bwd_apply (backward of rows too long for registers, the whole call)"
-    if alone:
-        return "rows_bwd_resident (backward row kernel: dx and the dgamma / dbeta partials), timed without col_reduce"
-    return "rows_bwd_resident + col_reduce (the whole backward call)"
+        n = LB.atexn_bench_describe_bwd(0, code, 0, dims[0], 0, dims[1], buf, 512)
+    else:
+        N, C, D, cf = dims
+        n = LB.atexn_bench_describe_bwd(1, code, 0 if cf else 1, N, C, D, buf, 512)
+    text = buf.value.decode() if n > 0 else "backward call"
+    plan, _, alone = text.partition("; alone=")
+    return plan, alone == "1"
 
 
 def torch_mod():
@@ -388,7 +384,7 @@ def time_row_kernel_alone(case, steps, warmup):
     """Average ms of the backward call without its final column reduction (the dominant kernel
     alone), through the benchmark build of the library; None if that build is missing or the
     case's backward has no separate column reduction to switch off."""
-    if not resident_rows_bwd(case.op, case.dtype, case.dims):
+    if not describe_bwd(case.op, case.dtype, case.dims)[1]:
         return None
     LB = bench_lib()
     if LB is None:
@@ -406,8 +402,9 @@ def time_row_kernel_alone(case, steps, warmup):
         case.L = product
 
 
-def measure(name, steps, warmup, extras=True):
-    """Times one case; returns (result dict, GpuCase)."""
+def measure(name, steps, warmup, extras=True, streaming=True):
+    """Times one case; returns (result dict, GpuCase).  extras: the hot-cache and HIP-graph
+    legs; streaming: torch's copy / add on the same tensors."""
     op, dtype, dims = CASES[name]
     fb, bb = algorithmic_bytes(op, dtype, dims)
     case = GpuCase(op, dtype, dims)
@@ -438,9 +435,13 @@ def measure(name, steps, warmup, extras=True):
         "gbps": {"fwd": fb / (ms_fwd * 1e-3) / 1e9, "bwd": bb / (ms_bwd * 1e-3) / 1e9},
         "roofline": {"bound": "hbm", "achieved": achieved, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": achieved / HBM_PEAK_GBPS, "traffic": MEASURED_TRAFFIC.get(name),
-                     "kernel": roofline_kernel(op, dtype, dims, ms_alone is not None),
+                     "kernel": describe_bwd(op, dtype, dims)[0] +
+                               (": the row kernel timed alone, without col_reduce" if ms_alone is not None
+                                else ": the whole backward call"),
                      "us": ms_roof * 1e3},
     }
+    if streaming:
+        res["streaming_reference"] = streaming_reference(case, steps, warmup)
     if not extras:
         return res, case
 
@@ -475,25 +476,38 @@ def measure(name, steps, warmup, extras=True):
         print(f"hip graph timing skipped: {e}", file=sys.stderr)
     res["us_per_call"]["fwd_bwd_hip_graph"] = None if ms_step_graph is None else ms_step_graph * 1e3
 
-    # what plain streaming kernels reach on the same tensors and rotation (torch's elementwise
-    # kernels): a copy (1 read + 1 write, the forward's traffic) and an add (2 reads + 1 write,
-    # the backward's)
-    tensor_bytes = case.sets[0]["x"].numel() * ESIZE[dtype]
-    ms_copy = case.time_loop(lambda i: case.sets[i % case.n_sets]["y"].copy_(case.sets[i % case.n_sets]["x"]),
-                             steps, warmup)
-    torch = case.torch
-    ms_add = case.time_loop(lambda i: torch.add(case.sets[i % case.n_sets]["x"], case.sets[i % case.n_sets]["dy"],
-                                                out=case.sets[i % case.n_sets]["dx"]), steps, warmup)
-    res["streaming_reference"] = {
-        "copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
-        "add_us": ms_add * 1e3, "add_gbps": 3 * tensor_bytes / (ms_add * 1e-3) / 1e9,
-        "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"}
     return res, case
 
 
-def run_case(name, steps, warmup, with_cpu=True, with_targets=False):
+def streaming_reference(case, steps, warmup):
+    """What plain streaming kernels reach on the same tensors and rotation (torch's elementwise
+    kernels): a copy (1 read + 1 write, the forward's traffic) and an add (2 reads + 1 write,
+    the backward's)."""
+    torch = case.torch
+    tensor_bytes = case.sets[0]["x"].numel() * ESIZE[case.dtype]
+    ms_copy = case.time_loop(lambda i: case.sets[i % case.n_sets]["y"].copy_(case.sets[i % case.n_sets]["x"]),
+                             steps, warmup)
+    ms_add = case.time_loop(lambda i: torch.add(case.sets[i % case.n_sets]["x"], case.sets[i % case.n_sets]["dy"],
+                                                out=case.sets[i % case.n_sets]["dx"]), steps, warmup)
+    return {
+        "copy_us": ms_copy * 1e3, "copy_gbps": 2 * tensor_bytes / (ms_copy * 1e-3) / 1e9,
+        "add_us": ms_add * 1e3, "add_gbps": 3 * tensor_bytes / (ms_add * 1e-3) / 1e9,
+        "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"}
+
+
+# the benchmark configurations beside the default case and the targets, on the default run's line
+CONFIG_CASES = ("ln_cfg0", "ln_128_f16", "ln_128_bf16", "ln_4096_f16", "ln_4096_bf16", "ln_12288_f16",
+                "ln_12288_bf16", "in3d_ndhwc", "in3d_ncdhw")
+
+
+def steps_for(name, steps):
+    """Fewer timed steps for the 268 MB-per-tensor volumes (a step there is a third of a millisecond)."""
+    return max(10, steps // 10) if "3d" in name else steps
+
+
+def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=False):
     op, dtype, dims = CASES[name]
-    m, case = measure(name, steps, warmup)
+    m, case = measure(name, steps, warmup, extras=not cold_only)
     out = {
         "metric": "LN/IN fwd+bwd achieved HBM GB/s",
         "value": m["value"],
@@ -513,7 +527,7 @@ def run_case(name, steps, warmup, with_cpu=True, with_targets=False):
         "pct_of_hbm_peak": m["pct_of_hbm_peak"],
         "us_per_call": m["us_per_call"],
         "gbps": m["gbps"],
-        "streaming_reference": m["streaming_reference"],
+        "streaming_reference": m.get("streaming_reference"),
         "roofline": m["roofline"],
     }
     del case
@@ -523,7 +537,7 @@ def run_case(name, steps, warmup, with_cpu=True, with_targets=False):
         for tname in TARGET_CASES:
             if tname == name:
                 continue
-            t, tcase = measure(tname, steps, warmup, extras=False)
+            t, tcase = measure(tname, steps, warmup, extras=False, streaming=not cold_only)
             del tcase
             torch_mod().cuda.empty_cache()
             out["targets"][tname] = {
@@ -532,6 +546,20 @@ def run_case(name, steps, warmup, with_cpu=True, with_targets=False):
                 "value": t["value"], "pct_of_hbm_peak": t["pct_of_hbm_peak"],
                 "roofline": t["roofline"],
             }
+            if "streaming_reference" in t:
+                out["targets"][tname]["streaming_reference"] = t["streaming_reference"]
+        # every other benchmark configuration
+        out["configs"] = {}
+        for cname in CONFIG_CASES:
+            if cname == name:
+                continue
+            c, ccase = measure(cname, steps_for(cname, steps), warmup, extras=False, streaming=not cold_only)
+            del ccase
+            torch_mod().cuda.empty_cache()
+            out["configs"][cname] = {k: c[k] for k in ("workload", "us_per_call", "gbps", "value", "pct_of_hbm_peak",
+                                                       "roofline", "streaming_reference") if k in c}
+            out["configs"][cname]["dtype"] = CASES[cname][1]
+            out["configs"][cname]["steps"] = steps_for(cname, steps)
     if with_cpu:
         out["cpu_baseline"] = cpu_baseline(op, dtype, dims)
     return out
@@ -548,7 +576,10 @@ def main():
                     help="set a launch-planning parameter (atexn_set_tuning) before measuring, "
                          "in the product and the benchmark build of the library; for A/B runs")
     ap.add_argument("--no-targets", action="store_true",
-                    help="default case only: skip the InstanceNorm target shapes")
+                    help="default case only: skip the InstanceNorm target shapes and the other configurations")
+    ap.add_argument("--cold-only", action="store_true",
+                    help="only the rotating-buffer (cold) legs: no hot-cache loop, no HIP-graph replay, no "
+                         "torch copy / add; what a rocprofv3 kernel trace of this file should average over")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
                          "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
@@ -562,22 +593,24 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU (no CPU fallback exists for the product path)")
     for item in args.tune:
-        from atex_amd.nv_norms import _capi
-
+        global USE_BENCH_LIB_EVERYWHERE
+        USE_BENCH_LIB_EVERYWHERE = True
         key, _, val = item.partition("=")
-        for L in (_capi.lib(), bench_lib()):
-            if L is not None and L.atexn_set_tuning(key.encode(), int(val)) != 0:
-                sys.exit(f"--tune {item}: {L.atexn_last_error().decode()}")
+        L = bench_lib()
+        if L is None:
+            sys.exit("--tune needs the benchmark build of the library (python -m atex_amd.build)")
+        if L.atexn_set_tuning(key.encode(), int(val)) != 0:
+            sys.exit(f"--tune {item}: {L.atexn_last_error().decode()}")
     if args.case == "all":
         for name in CASES:
             if name in SWEEP_ONLY_CASES:
                 continue
-            steps = args.steps if "3d" not in name else max(10, args.steps // 10)
-            r = run_case(name, steps, args.warmup, with_cpu=False)
+            r = run_case(name, steps_for(name, args.steps), args.warmup, with_cpu=False, cold_only=args.cold_only)
             print(json.dumps(r), flush=True)
         return
     print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu,
-                              with_targets=args.case == DEFAULT_CASE and not args.no_targets)), flush=True)
+                              with_targets=args.case == DEFAULT_CASE and not args.no_targets,
+                              cold_only=args.cold_only)), flush=True)
     if args.copy_calibration:
         src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
         dst = torch.empty_like(src)

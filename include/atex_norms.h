@@ -24,7 +24,8 @@
  *     rsqrt(biased_variance + epsilon) (reference: cc/kernels/norm_util.h:253-258);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); every call is
  *     asynchronous on it, re-entrant, allocates nothing and keeps no device state
- *     (atexn_layer_norm_bwd_static is the one exception, see there);
+ *     (atexn_layer_norm_bwd_static is the one exception, see there); the library has no
+ *     process-wide settings: launch plans depend on the sizes and the device alone;
  *   - the device the stream belongs to must be the calling thread's current device: launch
  *     plans and workspace sizes are made for the current device's compute-unit count;
  *   - data pointers need only the alignment of their element type (2 or 4 bytes): the
@@ -73,16 +74,6 @@ const char* atexn_status_string(int status);
 const char* atexn_last_error(void);
 /* ABI version of this header: bumps when a signature changes. */
 int atexn_abi_version(void);
-
-/* Debugging / benchmarking hook, not needed by a drop-in user: sets one launch-planning
- * parameter (resident waves per CU, rows per batch, work items per CU of the two-stage kernels,
- * single-pass channels-last on / off, ...) for the whole process; the names are listed in
- * csrc/plan.h (struct Tuning).  Every value it accepts still gives complete and correct results,
- * only a different launch plan.  The parameters are the one piece of process-wide HOST state of
- * the library: a *_workspace_bytes query and the call it sizes must run under the same
- * settings, so change them only while no other thread is between the two.  Returns
- * ATEXN_INVALID_ARGUMENT for an unknown name or a value out of range. */
-int atexn_set_tuning(const char* name, int value);
 
 /* ------------------------------------------------------------------ kernel level */
 

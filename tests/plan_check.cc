@@ -8,8 +8,9 @@
 #include "plan.h"
 
 namespace atexn {
-Tuning& tuning() {
-  static Tuning t;
+// the product library's planner: its parameters are constants
+const Tuning& tuning() {
+  static const Tuning t;
   return t;
 }
 }  // namespace atexn

@@ -214,10 +214,11 @@ def test_deterministic(capi):
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
 def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
     """Instances that fit one workgroup's registers take single-pass kernels; the two-stage
-    kernels stay reachable through the tuning hook.  Both must meet the oracle."""
+    kernels stay reachable through the benchmark build's tuning hook.  Both must meet the
+    oracle."""
     import torch
 
-    capi = util.Capi()
+    capi = util.Capi(bench=True)
     x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 77)
     y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
     dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, m_ref.astype(np.float32), r_ref.astype(np.float32),
@@ -245,62 +246,18 @@ def test_channels_last_single_pass_matches_two_stage(coracle, N, C, S, dtype):
         capi.L.atexn_set_tuning(b"cl_fused", 1)
 
 
-@pytest.mark.parametrize("dtype", ["f16", "f32"])
-@pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (4, 32, 4096), (16, 128, 2048), (3, 8, 30000)])
-def test_channels_last_cooperative_launch_matches_two_stage(coracle, N, C, S, dtype):
-    """Both stages in one cooperative launch (switched on through the tuning hook; where the
-    runtime refuses the launch the two-stage kernels run): the same arithmetic on the same
-    partials, so every float32 output must have the bits of the two-stage result, and 16-bit
-    outputs may differ only in the last place of a few rounding ties."""
-    import torch
-
-    capi = util.Capi()
-    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 78)
-    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
-    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
-    print(f"IN channels-last cooperative N={N} C={C} spatial={S} {dtype}", flush=True)
-    ref = None
-    try:
-        for coop in (0, 1):
-            assert capi.L.atexn_set_tuning(b"cl_coop", coop) == 0
-            y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
-            dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
-            torch.cuda.synchronize()
-            if ref is None:
-                ref = (y, m, r, dx, dg, db)
-            else:
-                for name, a, b in zip(("y", "mean", "inv_std", "dx", "dgamma", "dbeta"), (y, m, r, dx, dg, db), ref):
-                    if a.dtype == torch.float32:
-                        assert torch.equal(a.view(torch.uint8), b.view(torch.uint8)), name
-                        continue
-                    # 16-bit outputs: the same float32 arithmetic, but the compiler is free to
-                    # round a multiply-add straight to 16 bits in one kernel and through
-                    # float32 in the other; the two differ in the last place of a few ties
-                    af, bf = a.float(), b.float()
-                    differing = af != bf
-                    assert int(differing.sum()) <= 1e-3 * af.numel(), name
-                    ulp = torch.maximum(af.abs(), bf.abs()) * (2.0 ** -10 if a.dtype == torch.float16 else 2.0 ** -7)
-                    assert bool(((af - bf).abs() <= 1.01 * ulp).all()), name
-    finally:
-        capi.L.atexn_set_tuning(b"cl_coop", 0)
-    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
-    tol = TOL[dtype]
-    assert_close(util.to_host(ref[1]), m_ref, tol["stat"], "mean")
-    assert_close(util.to_host(ref[2]), r_ref, tol["stat"], "inv_std")
-    assert_close(util.to_host(ref[0]), y_ref, tol["y"], "y")
-
-
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("N,C,S,in_place", [(2, 4, 65536, False), (1, 3, 110592, False), (3, 2, 50176, True),
                                             (2, 2, 33001, False), (1, 5, 69632, False), (1, 2, 69633, False),
                                             (2, 3, 34816, True), (1, 2, 55299, False), (40, 16, 36864, False)])
-def test_channel_first_planes_staged_on_chip(capi, coracle, N, C, S, dtype, in_place):
+def test_channel_first_planes_staged_on_chip(coracle, N, C, S, dtype, in_place):
     """Planes beyond the register-resident limit that still fit one workgroup's registers plus
     LDS make a single pass (forward up to 27 vectors per thread of 512, backward, which stages x
     and dy, up to 17): the limits of both directions for 16-bit and float32 planes, one
     element past them (two-stage kernels again), ragged planes, in place, and more planes than
     workgroups.  (The planner stages rows only when there are enough of them to fill the chip;
-    the tuning hook lifts that condition here.)"""
+    the benchmark build's tuning hook lifts that condition here.)"""
+    capi = util.Capi(bench=True)
     assert capi.L.atexn_set_tuning(b"staged_rows", 2) == 0
     try:
         run_case(capi, coracle, N, C, S, dtype, True, 37, in_place=in_place)

@@ -45,12 +45,17 @@ def test_every_declared_symbol_is_exported(L):
     for n in names:
         assert hasattr(L, n), f"{n} is declared in atex_norms.h but not exported"
     assert set(names) <= set(_capi.SIGNATURES), set(names) - set(_capi.SIGNATURES)
-    # and nothing beyond the header: every exported atexn_* symbol of the product library (and
-    # of its benchmark variant) is declared
-    for path in (_capi.LIB_PATH, _capi.LIB_PATH.replace(".so", "_bench.so")):
+    # and nothing beyond the header: every exported atexn_* symbol of the product library is
+    # declared there; its benchmark variant adds exactly what csrc/bench_hooks.h declares (the
+    # process-wide tuning switch among them, which the product library must not have)
+    hooks = open(os.path.join(ROOT, "atex_amd", "csrc", "bench_hooks.h")).read()
+    hooks = re.sub(r"/\*.*?\*/", "", hooks, flags=re.S)
+    hook_names = set(re.findall(r"\b(atexn_[a-z0-9_]+)\s*\(", hooks))
+    assert hook_names == set(_capi.BENCH_SIGNATURES) and "atexn_set_tuning" in hook_names
+    for path, want in ((_capi.LIB_PATH, set(names)), (_capi.BENCH_LIB_PATH, set(names) | hook_names)):
         out = subprocess.run(["nm", "-D", "--defined-only", path], capture_output=True, text=True, check=True).stdout
         exported = {line.split()[-1] for line in out.splitlines() if line.split()[-1].startswith("atexn_")}
-        assert exported == set(names), (path, exported ^ set(names))
+        assert exported == want, (path, exported ^ want)
     assert L.atexn_abi_version() == 2
     assert L.atexn_status_string(0) == b"OK"
     assert L.atexn_status_string(1) == b"INVALID_ARGUMENT"
@@ -222,10 +227,8 @@ def test_kernel_level_validation(L):
     assert L.atexn_layer_norm_bwd(1, FAKE, 0x2000, FAKE, FAKE, FAKE, 8192, 1024, 0x3000, FAKE, FAKE,
                                   0x4000, need - 256, None) == 1
     assert b"workspace too small" in L.atexn_last_error()
-    assert L.atexn_set_tuning(b"no_such_parameter", 1) == 1
-    # running only part of a backward call is not something the product library can be told
-    assert L.atexn_set_tuning(b"bwd_stage_mask", 1) == 1
-    assert b"unknown tuning parameter" in L.atexn_last_error()
+    # the product library has no process-wide settings at all
+    assert not hasattr(L, "atexn_set_tuning")
     # the static-scratch backward refuses what does not fit its buffer before it touches a device
     assert L.atexn_layer_norm_bwd_workspace_bytes(1, 2048, 12288) > (8 << 20)
     assert L.atexn_layer_norm_bwd_static(1, FAKE, 0x2000, FAKE, FAKE, FAKE, 2048, 12288, 0x3000, FAKE,
@@ -233,30 +236,37 @@ def test_kernel_level_validation(L):
     assert b"static buffer" in L.atexn_last_error()
 
 
-def test_every_planning_parameter_is_settable(L):
-    """Each parameter of the planner (struct Tuning in csrc/plan.h) is reachable through
-    atexn_set_tuning under its own name and accepts its default; the one that runs only part of
-    a backward call exists in the benchmark build alone."""
+def test_every_planning_parameter_is_settable_in_the_benchmark_build():
+    """Each parameter of the planner (struct Tuning in csrc/plan.h) is reachable through the
+    benchmark build's atexn_set_tuning under its own name and accepts its default."""
     import os
     import re
+
+    L = _capi.bench_lib()
+    assert L.atexn_set_tuning(b"no_such_parameter", 1) == 1
+    assert b"unknown tuning parameter" in L.atexn_last_error()
 
     plan_h = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "atex_amd", "csrc", "plan.h")
     names = re.findall(r"^\s*TuneInt\s+(\w+)\{(\d+)\};", open(plan_h).read(), re.M)
     assert len(names) >= 20
     for name, default in names:
         rc = L.atexn_set_tuning(name.encode(), int(default))
-        if name == "bwd_stage_mask":
-            assert rc == 1
-        else:
-            assert rc == 0, (name, default, L.atexn_last_error())
+        assert rc == 0, (name, default, L.atexn_last_error())
     # a plan follows its parameter: planes staged on chip need no statistics workspace
     rows = (1, 0, 16, 64, 65536)  # dtype f16, channel-first, N, C, D
     assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
     assert L.atexn_set_tuning(b"staged_rows", 0) == 0
     try:
         assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) > 0
+        # ... and the product library, loaded beside it, is not affected
+        assert _capi.lib().atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
     finally:
         assert L.atexn_set_tuning(b"staged_rows", 1) == 0
+    buf = ctypes.create_string_buffer(256)
+    assert L.atexn_bench_describe_bwd(0, 1, 0, 8192, 0, 1024, buf, 256) > 0
+    assert b"rows_bwd_resident" in buf.value and b"alone=1" in buf.value
+    assert L.atexn_bench_describe_bwd(1, 1, 1, 8, 64, 16384, buf, 256) > 0
+    assert b"cl_bwd_sums" in buf.value and b"alone=0" in buf.value
 
 
 def test_workspace_queries_without_gpu(L):

@@ -90,3 +90,61 @@ def test_static_scratch_limit_and_empty():
     capi.capi.check(st)
     torch.cuda.synchronize()
     assert float(dg.abs().max()) == 0.0 and float(db.abs().max()) == 0.0
+
+
+def test_static_scratch_allocates_nothing_and_replays_from_a_graph():
+    """The use the entry point exists for: one eager warm-up call (which looks the scratch
+    address up), then the call recorded into a HIP graph and replayed.  Device memory in use
+    does not move across an eager call (outputs are allocated beforehand), and every replay has
+    the bits of atexn_layer_norm_bwd, with eager work and synchronisations between replays."""
+    import torch
+
+    from oracle import oracle as O
+
+    capi = util.Capi()
+    dtype, N, D = "f16", 2048, 1024
+    print(f"no-alloc LN bwd under graph capture dtype={dtype} N={N} D={D}", flush=True)
+    x, gamma, beta, dy = util.ln_inputs("row_mean", N, D, dtype, 44)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    _, mean, rstd = capi.ln_fwd(xd, gd, bd, EPS, dtype)
+    dx_ref, dg_ref, db_ref = capi.ln_bwd(dyd, xd, gd, mean, rstd, dtype)
+    dx = torch.empty_like(xd)
+    dg = torch.empty(D, dtype=torch.float32, device="cuda")
+    db = torch.empty(D, dtype=torch.float32, device="cuda")
+
+    def call(stream):
+        st = capi.L.atexn_layer_norm_bwd_static(
+            O.DTYPE_CODE[dtype], dyd.data_ptr(), xd.data_ptr(), gd.data_ptr(), mean.data_ptr(),
+            rstd.data_ptr(), N, D, dx.data_ptr(), dg.data_ptr(), db.data_ptr(), stream)
+        capi.capi.check(st)
+
+    call(torch.cuda.current_stream().cuda_stream)  # warm-up: the one-time symbol lookup
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    call(torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before, (free_before, free_after)
+    assert _same_bits(dx, dx_ref) and _same_bits(dg, dg_ref) and _same_bits(db, db_ref)
+
+    graph = torch.cuda.CUDAGraph()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        call(side.cuda_stream)
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=side):
+        call(side.cuda_stream)
+    for replay in range(3):
+        for t in (dx, dg, db):
+            t.fill_(float("nan"))
+        junk = torch.randn(1 << 20, device="cuda").sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        del junk
+        assert _same_bits(dx, dx_ref), f"replay {replay}: dx differs"
+        assert _same_bits(dg, dg_ref), f"replay {replay}: dgamma differs"
+        assert _same_bits(db, db_ref), f"replay {replay}: dbeta differs"

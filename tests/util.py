@@ -146,16 +146,21 @@ def to_host(t, dtype: str | None = None) -> np.ndarray:
 
 # ------------------------------------------------------------ kernel-level C ABI
 class Capi:
-    """Calls the kernel-level entry points of libatex_norms_hip.so on torch device memory."""
+    """Calls the kernel-level entry points of libatex_norms_hip.so on torch device memory.
+    bench=True: through the benchmark build of the library instead, the only one whose launch
+    planning can be changed (atexn_set_tuning), for tests that force a kernel family."""
 
-    def __init__(self):
+    def __init__(self, bench=False):
         import torch
 
         from atex_amd.nv_norms import _capi
 
         self.torch = torch
         self.capi = _capi
-        self.L = _capi.lib()
+        self.L = _capi.bench_lib() if bench else _capi.lib()
+
+    def _check(self, status):
+        self.capi.check(status, self.L)
 
     def _ws(self, nbytes, device):
         if nbytes == 0:
@@ -178,7 +183,7 @@ class Capi:
         mean = t.empty(N, dtype=t.float32, device=x.device)
         rstd = t.empty(N, dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_layer_norm_fwd_workspace_bytes(code, N, D), x.device)
-        self.capi.check(self.L.atexn_layer_norm_fwd(
+        self._check(self.L.atexn_layer_norm_fwd(
             code, self._p(x), self._p(gamma), self._p(beta), N, D, eps, self._p(y), self._p(mean),
             self._p(rstd), wp, wb, self._stream(x.device)))
         return y, mean, rstd
@@ -191,7 +196,7 @@ class Capi:
         dg = t.empty(D, dtype=t.float32, device=x.device)
         db = t.empty(D, dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_layer_norm_bwd_workspace_bytes(code, N, D), x.device)
-        self.capi.check(self.L.atexn_layer_norm_bwd(
+        self._check(self.L.atexn_layer_norm_bwd(
             code, self._p(dy), self._p(x), self._p(gamma), self._p(mean), self._p(rstd), N, D,
             self._p(dx), self._p(dg), self._p(db), wp, wb, self._stream(x.device)))
         return dx, dg, db
@@ -209,7 +214,7 @@ class Capi:
         mean = t.empty((N, C), dtype=t.float32, device=x.device)
         rstd = t.empty((N, C), dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_instance_norm_fwd_workspace_bytes(code, layout, N, C, D), x.device)
-        self.capi.check(self.L.atexn_instance_norm_fwd(
+        self._check(self.L.atexn_instance_norm_fwd(
             code, layout, self._p(x), self._p(gamma), self._p(beta), N, C, D, eps, self._p(y),
             self._p(mean), self._p(rstd), wp, wb, self._stream(x.device)))
         return y, mean, rstd
@@ -223,7 +228,7 @@ class Capi:
         dg = t.empty(C, dtype=t.float32, device=x.device)
         db = t.empty(C, dtype=t.float32, device=x.device)
         ws, wp, wb = self._ws(self.L.atexn_instance_norm_bwd_workspace_bytes(code, layout, N, C, D), x.device)
-        self.capi.check(self.L.atexn_instance_norm_bwd(
+        self._check(self.L.atexn_instance_norm_bwd(
             code, layout, self._p(dy), self._p(x), self._p(gamma), self._p(mean), self._p(rstd),
             N, C, D, self._p(dx), self._p(dg), self._p(db), wp, wb, self._stream(x.device)))
         return dx, dg, db
