@@ -195,13 +195,17 @@ __device__ __forceinline__ unsigned cl_slab_offset(const ClGeom& g, int C, int u
   return static_cast<unsigned>(g.slot + u * g.ppb) * static_cast<unsigned>(C) + static_cast<unsigned>(g.coff);
 }
 
-template <typename T, int V, int U, bool LAST = false>
+// FULL: the host has checked that every slab of the launch has exactly U pixels per slot and that
+// every channel tile is complete, so every lane's every vector is valid: ok[] are compile-time
+// constants and the masks they feed disappear from the arithmetic (a third of the instructions
+// of the statistics, which run after the loads and are what the stage-1 kernels wait on).
+template <typename T, int V, int U, bool LAST = false, bool FULL = false>
 __device__ __forceinline__ void cl_load_slab(const T* slab, const ClGeom& g, int C,
                                              Pack<T, V> (&raw)[U], bool (&ok)[U]) {
 #pragma unroll
   for (int u = 0; u < U; ++u) {
-    ok[u] = g.ch_ok && g.slot + u * g.ppb < g.slab_n;
-    const bool inside = g.slot + u * g.ppb < g.slab_n;
+    const bool inside = FULL || g.slot + u * g.ppb < g.slab_n;
+    ok[u] = FULL || (g.ch_ok && inside);
     const T* src = slab + (inside ? cl_slab_offset(g, C, u) : static_cast<unsigned>(g.coff));
     raw[u] = LAST ? load_pack_last<T, V>(src) : load_pack<T, V>(src);
   }
@@ -214,12 +218,13 @@ template <typename T, int V, int U>
 __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], const bool (&ok)[U],
                                                   float inv_n, int TPP, float* lds,
                                                   float (&mean)[V], float (&m2)[V]) {
+  const float one = mix_one();
 #pragma unroll
   for (int i = 0; i < V; ++i) mean[i] = 0.f;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
 #pragma unroll
-    for (int i = 0; i < V; ++i) mean[i] += ok[u] ? to_f32(raw[u].v[i]) : 0.f;
+    for (int i = 0; i < V; ++i) mean[i] = ok[u] ? add_f32<T>(mean[i], raw[u].v[i], one) : mean[i];
   }
   cl_block_sum<V>(mean, lds, TPP);
 #pragma unroll
@@ -231,7 +236,7 @@ __device__ __forceinline__ void cl_resident_stats(const Pack<T, V> (&raw)[U], co
   for (int u = 0; u < U; ++u) {
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      const float d = ok[u] ? to_f32(raw[u].v[i]) - mean[i] : 0.f;
+      const float d = ok[u] ? sub_f32<T>(raw[u].v[i], mean[i], one) : 0.f;
       m2[i] = __builtin_fmaf(d, d, m2[i]);
     }
   }
@@ -387,11 +392,12 @@ struct ClFwdCoef {
   template <typename T>
   __device__ __forceinline__ Pack<T, V> apply(const Pack<T, V>& pk) const {
     Pack<T, V> o;
+    const float one = mix_one();
 #pragma unroll
     for (int i = 0; i < V; ++i) {
       // subtract the mean first: x * scale - mean * scale would cancel badly when |mean| >> std.
       // (explicit fused multiply-adds: every kernel that applies these constants rounds alike)
-      o.v[i] = from_f32<T>(__builtin_fmaf(to_f32(pk.v[i]) - mean[i], sc[i], bt[i]));
+      o.v[i] = from_f32<T>(__builtin_fmaf(sub_f32<T>(pk.v[i], mean[i], one), sc[i], bt[i]));
     }
     return o;
   }
@@ -404,16 +410,18 @@ __device__ __forceinline__ void cl_resident_sums(const Pack<T, V> (&rx)[U], cons
                                                  const bool (&ok)[U], const float (&mu)[V],
                                                  const float (&rs)[V], int TPP, float* lds,
                                                  float (&acc)[2 * V]) {
+  const float one = mix_one();
 #pragma unroll
   for (int i = 0; i < 2 * V; ++i) acc[i] = 0.f;
 #pragma unroll
   for (int u = 0; u < U; ++u) {
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      const float d = ok[u] ? to_f32(rd[u].v[i]) : 0.f;
-      const float xh = ok[u] ? (to_f32(rx[u].v[i]) - mu[i]) * rs[i] : 0.f;
-      acc[i] = __builtin_fmaf(d, xh, acc[i]);
-      acc[V + i] += d;
+      // (a masked-out vector leaves the sums as they are; the half operands feed the
+      // multiply-adds directly)
+      const float xh = sub_f32<T>(rx[u].v[i], mu[i], one) * rs[i];
+      acc[i] = ok[u] ? __builtin_fmaf(to_f32(rd[u].v[i]), xh, acc[i]) : acc[i];
+      acc[V + i] = ok[u] ? add_f32<T>(acc[V + i], rd[u].v[i], one) : acc[V + i];
     }
   }
   cl_block_sum<2 * V>(acc, lds, TPP);
@@ -597,9 +605,10 @@ struct ClBwdCoef {
   template <typename T>
   __device__ __forceinline__ Pack<T, V> apply(const Pack<T, V>& px, const Pack<T, V>& pd) const {
     Pack<T, V> o;
+    const float one = mix_one();
 #pragma unroll
     for (int i = 0; i < V; ++i) {
-      o.v[i] = from_f32<T>(__builtin_fmaf(sc[i], to_f32(pd.v[i]), __builtin_fmaf(ca[i], to_f32(px.v[i]) - mu[i], cb[i])));
+      o.v[i] = from_f32<T>(__builtin_fmaf(sc[i], to_f32(pd.v[i]), __builtin_fmaf(ca[i], sub_f32<T>(px.v[i], mu[i], one), cb[i])));
     }
     return o;
   }
@@ -616,7 +625,7 @@ struct ClBwdCoef {
 // U == 0 streams the slab in batches of 8 pixels per thread: per-thread running (mean, m2)
 // by batch-wise Chan updates (wf_lanes_push), combined over the block around the slab mean
 // (m2 = sum over threads of m2_t + n_t (mean_t - mean)^2, every term non-negative).
-template <typename T, int V, int U, bool RG>
+template <typename T, int V, int U, bool RG, bool FULL = false>
 __global__ void __launch_bounds__(kClThreads)
 cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int C, int S,
              int tpp_shift, int64_t slab_len) {
@@ -630,7 +639,7 @@ cl_fwd_stats(const T* __restrict__ x, float* __restrict__ pstat, int64_t D, int 
   if constexpr (U > 0) {
     Pack<T, V> raw[U];
     bool ok[U];
-    cl_load_slab<T, V, U>(xn + g.p0 * C, g, C, raw, ok);
+    cl_load_slab<T, V, U, false, FULL>(xn + g.p0 * C, g, C, raw, ok);
     cl_resident_stats<T, V, U>(raw, ok, inv_n, TPP, lds, mean, m2);
   } else {
     WfLanes<V> run;
@@ -756,7 +765,7 @@ cl_merge_stats(const float* __restrict__ pstat, float* __restrict__ folded, int6
 // ---------------------------------------------------------------- forward, stage 2
 // y may alias x: stage 1 has completed (it is an earlier launch on the same stream) and
 // every thread reads a vector before it writes the same vector.
-template <typename T, int V, int U, bool RG>
+template <typename T, int V, int U, bool RG, bool FULL = false>
 __global__ void __launch_bounds__(kClThreads, 2)  // two workgroups per CU: a grid of 2 x CUs slabs runs in one round
 cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restrict__ gamma,
              const float* __restrict__ beta, T* y, float* __restrict__ mean_out,
@@ -771,7 +780,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
   // resident slab: its loads are issued first and fly while the partials are merged
   Pack<T, V> raw[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
-  if constexpr (U > 0) cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
+  if constexpr (U > 0) cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
   cl_fold_stats<(U > 0)>(pstat, g, S, cnt_len, D, C, cap, eps, gamma, beta, sm_mean, sm_sc, sm_bt, mean_out,
                 rstd_out);
   __syncthreads();
@@ -818,7 +827,7 @@ cl_fwd_apply(const T* x, const float* __restrict__ pstat, const float* __restric
 
 // --------------------------------------------------------------- backward, stage 1
 // part[(n * S + s)][0][c] = sum dy * xh, part[...][1][c] = sum dy over the slab.
-template <typename T, int V, int U, bool RG>
+template <typename T, int V, int U, bool RG, bool FULL = false>
 __global__ void __launch_bounds__(kClThreads)
 cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
             const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
@@ -832,8 +841,8 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool ok[U > 0 ? U : 1];
   if constexpr (U > 0) {
-    cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-    cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+    cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   }
   float mu[V], rs[V];
 #pragma unroll
@@ -895,7 +904,7 @@ cl_bwd_sums(const T* __restrict__ dy, const T* __restrict__ x,
 // Every block first folds the S slab partials of its instance and channel tile into LDS and
 // produces its share of dgamma / dbeta (cl_fold_sums), which spares a third launch, then
 // writes dx for its slab.
-template <typename T, int V, int U, bool RG>
+template <typename T, int V, int U, bool RG, bool FULL = false>
 __global__ void __launch_bounds__(kClThreads, 2)  // two workgroups per CU: a grid of 2 x CUs slabs runs in one round
 cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
              const float* __restrict__ mean_in, const float* __restrict__ rstd_in,
@@ -916,8 +925,8 @@ cl_bwd_apply(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   Pack<T, V> rx[U > 0 ? U : 1], rd[U > 0 ? U : 1];
   bool okp[U > 0 ? U : 1];
   if constexpr (U > 0) {
-    cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, rx, okp);
-    cl_load_slab<T, V, U, true>(dy + (g.n * D + g.p0) * C, g, C, rd, okp);
+    cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, okp);
+    cl_load_slab<T, V, U, true, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, okp);
   }
   cl_fold_sums<(U > 0)>(part, g, N, S, C, cap, inv_d, gamma, mean_in, rstd_in, sm_mu, sm_sc, sm_ca, sm_cb,
                red_buf, fold_lds, dgamma, dbeta, cw_shift);

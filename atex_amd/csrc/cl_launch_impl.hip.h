@@ -2,12 +2,35 @@
 #pragma once
 
 #include "cl_kernels.hip.h"
+#include "cl_single_kernels.hip.h"
 #include "plan.h"
 #include "status.h"
 
 namespace atexn {
 
+static_assert(kPlanClSingleMaxCap == kClSingleMaxCap && kPlanClSingleMaxSlabs == kClSingleMaxSlabs &&
+                  kPlanClSingleMaxOwned == kClSingleMaxOwned,
+              "the planner and the single-launch kernels must agree on their limits");
+
+// The single-launch kernels tag what they exchange with a number taken per call, which a graph
+// replay would repeat: callers that capture get the two-stage kernels.
+inline bool stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 static_assert(kPlanClFoldRegs == 2 * kClFoldRegs, "the planner and the kernels must agree on the fold's register limit");
+
+// Whether every register-resident slab of the plan holds exactly U pixels per pixel slot and
+// every channel tile is complete (the kernels' FULL instantiations: no lane is ever masked).
+inline bool cl_slabs_full(const ClPlan& p, int64_t C, int64_t D) {
+  const int64_t ppb = kClThreads >> p.tpp_shift;
+  return p.U > 0 && C % (int64_t(p.TPP) * p.V) == 0 && D % p.slab_len == 0 && p.slab_len == int64_t(p.U) * ppb;
+}
 
 template <typename T, int V>
 int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64_t C, int64_t D,
@@ -26,9 +49,9 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
   ATEXN_REQUIRE(p.CT <= 65535, "channel count %lld too large (channels-last limit 65535 * 2048)",
                 (long long)C);
   const dim3 grid(static_cast<unsigned>(N), p.S, p.CT);
-#define ATEXN_CL_FWD(U_, RG_)                                                                  \
+#define ATEXN_CL_FWD(U_, RG_, ...)                                                             \
   do {                                                                                        \
-    cl_fwd_stats<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, pstat, D, Ci, p.S, p.tpp_shift,  \
+    cl_fwd_stats<T, V, U_, RG_, ##__VA_ARGS__><<<grid, kClThreads, 0, st>>>(x, pstat, D, Ci, p.S, p.tpp_shift,  \
                                                        p.slab_len);                           \
     ATEXN_CHECK_LAUNCH("cl_fwd_stats");                                                       \
     if (p.fold) {                                                                             \
@@ -37,7 +60,7 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       cl_merge_stats<<<mgrid, kClThreads, 0, st>>>(pstat, folded, D, Ci, p.S, p.slab_len);    \
       ATEXN_CHECK_LAUNCH("cl_merge_stats");                                                   \
     }                                                                                         \
-    cl_fwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(x, p.fold ? folded : pstat, gamma,  \
+    cl_fwd_apply<T, V, U_, RG_, ##__VA_ARGS__><<<grid, kClThreads, 0, st>>>(x, p.fold ? folded : pstat, gamma,  \
                                                        beta, y, mean, rstd, D, Ci,            \
                                                        p.fold ? 1 : p.S,                      \
                                                        p.fold ? D : p.slab_len, p.tpp_shift,  \
@@ -70,6 +93,27 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       ATEXN_CHECK_LAUNCH("cl_fwd_fused");
       return ATEXN_OK;
     }
+    if (p.single && static_cast<const void*>(y) != static_cast<const void*>(x) && !stream_is_capturing(st)) {
+      char* w = static_cast<char*>(ws);
+      cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
+      cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
+      const unsigned tag = next_call_tag();
+      const int polls = tuning().cl_single_polls;
+#define ATEXN_CL_FWD_SINGLE(U_, FULL_)                                                          \
+  cl_fwd_single<T, V, U_, FULL_><<<grid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, \
+                                                              rstd, D, Ci, p.S, p.tpp_shift,     \
+                                                              p.slab_len, eps, tag, polls)
+      if (cl_slabs_full(p, C, D)) {
+        if (p.U == 4) ATEXN_CL_FWD_SINGLE(4, true);
+        else ATEXN_CL_FWD_SINGLE(8, true);
+      } else {
+        if (p.U == 4) ATEXN_CL_FWD_SINGLE(4, false);
+        else ATEXN_CL_FWD_SINGLE(8, false);
+      }
+#undef ATEXN_CL_FWD_SINGLE
+      ATEXN_CHECK_LAUNCH("cl_fwd_single");
+      return ATEXN_OK;
+    }
     // a channel count that is not a multiple of V: the last channel vector of a pixel overlaps
     // its neighbour and owns only its last C % V elements
     if (C % V != 0) {
@@ -78,6 +122,12 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       if (p.U == 16) { ATEXN_CL_FWD(16, true); return ATEXN_OK; }
       ATEXN_CL_FWD(0, true);
       return ATEXN_OK;
+    }
+    // every slab has exactly U pixels per slot and every channel tile is complete: no masks
+    if (cl_slabs_full(p, C, D)) {
+      if (p.U == 4) { ATEXN_CL_FWD(4, false, true); return ATEXN_OK; }
+      if (p.U == 8) { ATEXN_CL_FWD(8, false, true); return ATEXN_OK; }
+      if (p.U == 16) { ATEXN_CL_FWD(16, false, true); return ATEXN_OK; }
     }
     if (p.U == 4) { ATEXN_CL_FWD(4, false); return ATEXN_OK; }
     if (p.U == 8) { ATEXN_CL_FWD(8, false); return ATEXN_OK; }
@@ -108,9 +158,9 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
   // how stage 2 deals the dgamma / dbeta columns to its workgroups (after the fold launch a
   // partial row per instance is left)
   const int cw_shift = cl_dparam_chunk_shift(p.fold ? N : N * p.S, 2 * C, N * p.S * p.CT);
-#define ATEXN_CL_BWD(U_, RG_)                                                                  \
+#define ATEXN_CL_BWD(U_, RG_, ...)                                                             \
   do {                                                                                        \
-    cl_bwd_sums<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S, \
+    cl_bwd_sums<T, V, U_, RG_, ##__VA_ARGS__><<<grid, kClThreads, 0, st>>>(dy, x, mean, rstd, part, D, Ci, p.S, \
                                                       p.tpp_shift, p.slab_len);               \
     ATEXN_CHECK_LAUNCH("cl_bwd_sums");                                                        \
     if (p.fold) {                                                                             \
@@ -118,7 +168,7 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
                                        static_cast<int>(N), int64_t(p.S) * 2 * C, 2 * C);     \
       if (rc != ATEXN_OK) return rc;                                                          \
     }                                                                                         \
-    cl_bwd_apply<T, V, U_, RG_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd,           \
+    cl_bwd_apply<T, V, U_, RG_, ##__VA_ARGS__><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd,           \
                                                        p.fold ? folded : part, dx,            \
                                                        dgamma, dbeta, N, D, Ci,               \
                                                        p.fold ? 1 : p.S,                      \
@@ -156,11 +206,38 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       if (N > 1) return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N), C, st);
       return ATEXN_OK;
     }
+    if (p.single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && !stream_is_capturing(st)) {
+      char* w = static_cast<char*>(ws);
+      cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
+      cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
+      cl_word* finals_dev = reinterpret_cast<cl_word*>(w + p.off_finals_dev);
+      const unsigned tag = next_call_tag();
+      const int polls = tuning().cl_single_polls;
+      const int Ni = static_cast<int>(N);
+#define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
+  cl_bwd_single<T, V, U_, FULL_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, \
+                                                              finals_dev, dx, dgamma, dbeta, Ni, D, Ci, \
+                                                              p.S, p.tpp_shift, p.slab_len, tag, polls)
+      if (cl_slabs_full(p, C, D)) {
+        if (p.U == 4) ATEXN_CL_BWD_SINGLE(4, true);
+        else ATEXN_CL_BWD_SINGLE(8, true);
+      } else {
+        if (p.U == 4) ATEXN_CL_BWD_SINGLE(4, false);
+        else ATEXN_CL_BWD_SINGLE(8, false);
+      }
+#undef ATEXN_CL_BWD_SINGLE
+      ATEXN_CHECK_LAUNCH("cl_bwd_single");
+      return ATEXN_OK;
+    }
     if (C % V != 0) {
       if (p.U == 4) { ATEXN_CL_BWD(4, true); return ATEXN_OK; }
       if (p.U == 8) { ATEXN_CL_BWD(8, true); return ATEXN_OK; }
       ATEXN_CL_BWD(0, true);
       return ATEXN_OK;
+    }
+    if (cl_slabs_full(p, C, D)) {
+      if (p.U == 4) { ATEXN_CL_BWD(4, false, true); return ATEXN_OK; }
+      if (p.U == 8) { ATEXN_CL_BWD(8, false, true); return ATEXN_OK; }
     }
     if (p.U == 4) { ATEXN_CL_BWD(4, false); return ATEXN_OK; }
     if (p.U == 8) { ATEXN_CL_BWD(8, false); return ATEXN_OK; }

@@ -1,0 +1,445 @@
+// Channels-last InstanceNorm in ONE launch per direction, for launches whose slabs are all
+// register-resident and whose workgroups are all on the chip at once (two per CU).
+//
+// The two-stage kernels (cl_kernels.hip.h) read x (and dy) twice and pay a kernel boundary
+// between the statistics and their use.  Here a workgroup keeps its slab in registers and the
+// workgroups of an instance exchange their per-slab statistics through memory while they run:
+//
+//   1. every workgroup publishes the per-channel partials of its slab;
+//   2. workgroup s of an instance OWNS channel s (s + S, ... when a tile has more channels than
+//      the instance has slabs): one wave, a lane per slab, waits for that channel's partials,
+//      folds them and publishes the channel's final statistics;
+//   3. every workgroup waits for the finals of its channels (a lane per channel), derives the
+//      per-channel constants and applies them to the slab it still holds.
+//
+// Each published value travels as an 8-byte word (value, tag) written by one store: the tag
+// names this call (a process-wide call counter handed in by the host), so a word either still
+// holds some older call's tag or is complete: no separate flag, no fence, no counter to clear.
+// The second word of a pair carries the complemented tag, so that 64 bits of arbitrary memory
+// contents would have to match before garbage in a fresh workspace is taken for data.  Readers
+// use device-scope loads, which go past the vector and L2 caches' stale lines; writers use plain
+// stores, which reach the L2 of their XCD: every workgroup of an instance runs on the same XCD
+// (the host only takes this path when the instance index, the fastest grid coordinate, is
+// congruent to the workgroup id modulo the eight XCDs), and that L2 is where those loads look.
+// A hop costs about 2 us, against about 3.5 us for the kernel boundary and the second read.
+//
+// Nothing here can hang: every wait is a bounded number of polls.  A workgroup whose wait runs
+// out (its peers are not resident: another kernel holds the CUs; or the placement assumption
+// does not hold on this device) stops relying on anyone and recomputes, with the same code and
+// therefore to the same bits, the partials of every slab of its instance from x itself.  That
+// is why the host keeps callers that pass y == x (dx == dy) on the two-stage kernels: a peer may
+// already have overwritten its part of x by then.
+//
+// Counterpart in the reference: the single-kernel channels-last variant that keeps an instance
+// in one block's shared memory (fused_instance_norm_op.cu:1066-1165); it stops at D <= 372.
+#pragma once
+
+#include "cl_kernels.hip.h"
+
+namespace atexn {
+
+typedef unsigned long long cl_word;
+
+constexpr int kClSingleMaxCap = 64;    // channels per tile (the fallback keeps S x cap pairs in LDS)
+constexpr int kClSingleMaxSlabs = 64;  // slabs per instance: one lane each in the owner's fold
+constexpr int kClSingleMaxOwned = 4;   // channels one workgroup may own
+
+__device__ __forceinline__ cl_word cl_tagged(float v, unsigned tag) {
+  return static_cast<cl_word>(__builtin_bit_cast(unsigned, v)) | (static_cast<cl_word>(tag) << 32);
+}
+__device__ __forceinline__ cl_word cl_peek(const cl_word* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// A pair of tagged words as one 16-byte store (each aligned 8-byte half lands whole).
+__device__ __forceinline__ void cl_publish(cl_word* pair, float a, float b, unsigned tag) {
+  typedef cl_word w2 __attribute__((ext_vector_type(2)));
+  w2 v;
+  v.x = cl_tagged(a, tag);
+  v.y = cl_tagged(b, ~tag);
+  *reinterpret_cast<w2*>(pair) = v;
+}
+// The same, written through to memory (readers on other XCDs).
+__device__ __forceinline__ void cl_publish_device(cl_word* pair, float a, float b, unsigned tag) {
+  __hip_atomic_store(pair, cl_tagged(a, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(pair + 1, cl_tagged(b, ~tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One wave waits for the pair at `pair` (per lane; lanes with want == false wait for nothing):
+// true once every wanted lane has read both words with this call's tag, false after max_polls
+// rounds.  All 64 lanes of the wave must call it; the result is the same in all of them.
+__device__ __forceinline__ bool cl_wait_pair(const cl_word* pair, bool want, unsigned tag, int max_polls,
+                                             float& a, float& b) {
+  a = b = 0.f;
+  for (int poll = 0; poll < max_polls; ++poll) {
+    bool ready = true;
+    if (want) {
+      const cl_word w0 = cl_peek(pair);
+      const cl_word w1 = cl_peek(pair + 1);
+      ready = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
+      a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
+      b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
+    }
+    if (__all(ready)) return true;
+  }
+  return false;
+}
+
+// (mean, m2) of an instance from its slabs' (mean, m2), one slab per lane of a wave (lanes
+// >= S hold nothing): Chan's merge of all slabs at once, as cl_fold_stats does it.
+__device__ __forceinline__ void cl_fold_lanes_stats(float pm, float pq, int lane, int S, float n_full,
+                                                    float n_last, float inv_d, float& mean, float& m2) {
+#pragma clang fp contract(off)
+  const bool in = lane < S;
+  const float w = lane == S - 1 ? n_last : n_full;
+  mean = group_sum<kWave>(in ? pm * w : 0.f) * inv_d;
+  const float d = pm - mean;
+  m2 = group_sum<kWave>(in ? pq + w * (d * d) : 0.f);
+}
+
+// Geometry of slab l of the calling workgroup's instance and channel tile (the fallback walks
+// every slab with it).
+__device__ __forceinline__ ClGeom cl_geom_of_slab(const ClGeom& g, int l, int64_t D, int64_t slab_len) {
+  ClGeom h = g;
+  h.s = l;
+  h.p0 = static_cast<int64_t>(l) * slab_len;
+  h.p1 = h.p0 + slab_len < D ? h.p0 + slab_len : D;
+  h.slab_n = static_cast<int>(h.p1 - h.p0 < (1 << 20) ? h.p1 - h.p0 : (1 << 20));
+  return h;
+}
+
+// ------------------------------------------------------------------------------ forward
+// tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std).
+// Grid (N, S, channel tiles) as for the two-stage kernels; tile of at most 64 channels.
+template <typename T, int V, int U, bool FULL>
+__global__ void __launch_bounds__(kClThreads, 2)
+cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const float* __restrict__ gamma,
+              const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
+              float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
+              float eps, unsigned tag, int max_polls) {
+  __shared__ float lds[V * kClThreads];
+  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
+  __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
+  __shared__ int sm_fail;
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  const int c_base = g.ct * cap;
+  const int cap_here = C - c_base < cap ? C - c_base : cap;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  const float n_full = static_cast<float>(slab_len);
+  const float n_last = static_cast<float>(D - static_cast<int64_t>(S - 1) * slab_len);
+  if (threadIdx.x == 0) sm_fail = 0;
+  Pack<T, V> raw[U];
+  bool ok[U];
+  cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
+  // what the gathering lanes of wave 0 need besides the finals
+  float gmc = 0.f, btc = 0.f;
+  if (wave == 0 && lane < cap_here) {
+    gmc = gamma[c_base + lane];
+    btc = beta[c_base + lane];
+  }
+  float mean[V], m2[V];
+  cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(g.p1 - g.p0), TPP, lds, mean, m2);
+  if (g.ch_ok && g.slot == 0) {
+    cl_word* o = tagged + ((g.n * S + g.s) * C + g.coff) * 2;
+#pragma unroll
+    for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, mean[i], m2[i], tag);
+  }
+  if (wave == 0) {
+    bool fail = false;
+    // the channels this workgroup owns: a lane per slab
+    for (int lc = g.s; lc < cap_here; lc += S) {
+      const int c = c_base + lc;
+      float pm, pq;
+      if (!cl_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls,
+                        pm, pq)) {
+        fail = true;
+        break;
+      }
+      float mu, q;
+      cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
+      if (lane == 0) {
+        const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
+        cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
+        mean_out[g.n * C + c] = mu;
+        rstd_out[g.n * C + c] = rs;
+      }
+    }
+    // the finals of this tile's channels: a lane per channel
+    if (!fail) {
+      float fm, frs;
+      const bool want = lane < cap_here;
+      if (cl_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, fm, frs)) {
+        if (want) {
+          sm_mean[lane] = fm;
+          sm_sc[lane] = gmc * frs;
+          sm_bt[lane] = btc;
+        }
+      } else {
+        fail = true;
+      }
+    }
+    if (fail && lane == 0) sm_fail = 1;
+  }
+  __syncthreads();
+  if (sm_fail) {
+    // On its own: the partials of every slab of the instance, computed as their workgroups
+    // compute them, folded as their owners fold them.  The slabs pass through the registers of
+    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).
+    for (int l = 0; l < S; ++l) {
+      const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
+      cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
+      float mm[V], qq[V];
+      __syncthreads();  // the previous round's block sums have been read
+      cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
+      if (g.ch_ok && g.slot == 0) {
+        const int lc0 = g.coff - c_base;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          fb[(l * cap + lc0 + i) * 2] = mm[i];
+          fb[(l * cap + lc0 + i) * 2 + 1] = qq[i];
+        }
+      }
+    }
+    __syncthreads();
+    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
+      const int c = c_base + lc;
+      const float pm = lane < S ? fb[(lane * cap + lc) * 2] : 0.f;
+      const float pq = lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f;
+      float mu, q;
+      cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
+      if (lane == 0) {
+        const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
+        sm_mean[lc] = mu;
+        sm_sc[lc] = gamma[c] * rs;
+        sm_bt[lc] = beta[c];
+        if (lc % S == g.s) {  // an owner still serves its peers
+          cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
+          mean_out[g.n * C + c] = mu;
+          rstd_out[g.n * C + c] = rs;
+        }
+      }
+    }
+    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
+    __syncthreads();
+  }
+  if (g.ch_ok) {
+    ClFwdCoef<V, false> k;
+    k.load(g, tpp_shift, sm_mean, sm_sc, sm_bt);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        store_pack<T, V>(y + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u), k.template apply<T>(raw[u]));
+      }
+    }
+  }
+}
+
+// ----------------------------------------------------------------------------- backward
+// tagged: [N][S][C] pairs (sum dy * xh, sum dy) of the slabs; finals: [N][C] pairs of the
+// instances' sums, for the workgroups of the instance; finals_dev: the same pairs written
+// through to memory, for the workgroups of instance 0, which own the fold over the instances:
+// the owner of channel c there adds up the N pairs of c (a lane per instance) into dgamma[c]
+// and dbeta[c] after it has stored its dx.  N <= 64.
+template <typename T, int V, int U, bool FULL>
+__global__ void __launch_bounds__(kClThreads, 2)
+cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
+              const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
+              cl_word* finals, cl_word* finals_dev, T* __restrict__ dx, float* __restrict__ dgamma,
+              float* __restrict__ dbeta, int N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
+              unsigned tag, int max_polls) {
+  __shared__ float lds[2 * V * kClThreads];
+  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
+  __shared__ float sm_mu[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_ca[kClSingleMaxCap], sm_cb[kClSingleMaxCap];
+  __shared__ float inst[kClSingleMaxOwned][kWave][2];
+  __shared__ int sm_fail, sm_fail_dev;
+  const int CV = C / V;
+  const int TPP = 1 << tpp_shift;
+  const int cap = TPP * V;
+  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  const int c_base = g.ct * cap;
+  const int cap_here = C - c_base < cap ? C - c_base : cap;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = threadIdx.x / kWave;
+  const float inv_d = 1.0f / static_cast<float>(D);
+  if (threadIdx.x == 0) sm_fail = sm_fail_dev = 0;
+  Pack<T, V> rx[U], rd[U];
+  bool ok[U];
+  cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+  cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+  float mu[V], rs[V];
+#pragma unroll
+  for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
+  if (g.ch_ok) {
+    load_f32<V>(mean_in + g.n * C + g.coff, mu);
+    load_f32<V>(rstd_in + g.n * C + g.coff, rs);
+  }
+  // what the gathering lanes of wave 0 need besides the finals
+  float gmc = 0.f, muc = 0.f, rsc = 0.f;
+  if (wave == 0 && lane < cap_here) {
+    gmc = gamma[c_base + lane];
+    muc = mean_in[g.n * C + c_base + lane];
+    rsc = rstd_in[g.n * C + c_base + lane];
+  }
+  float acc[2 * V];
+  cl_resident_sums<T, V, U>(rx, rd, ok, mu, rs, TPP, lds, acc);
+  if (g.ch_ok && g.slot == 0) {
+    cl_word* o = tagged + ((g.n * S + g.s) * C + g.coff) * 2;
+#pragma unroll
+    for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, acc[i], acc[V + i], tag);
+  }
+  // constants of dx = sc * dy + (ca * (x - mu) + cb) from an instance's sums (b = sum dy * xh,
+  // a = sum dy), as cl_fold_sums derives them
+  auto constants = [&](int lc, float gm, float m, float r, float b, float a) {
+#pragma clang fp contract(off)
+    const float sc = gm * r;
+    sm_mu[lc] = m;
+    sm_sc[lc] = sc;
+    sm_ca[lc] = -(sc * r) * (b * inv_d);
+    sm_cb[lc] = -sc * (a * inv_d);
+  };
+  if (wave == 0) {
+    bool fail = false;
+    for (int lc = g.s; lc < cap_here; lc += S) {
+      const int c = c_base + lc;
+      float pb, pa;
+      if (!cl_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls,
+                        pb, pa)) {
+        fail = true;
+        break;
+      }
+      const float b = group_sum<kWave>(lane < S ? pb : 0.f);
+      const float a = group_sum<kWave>(lane < S ? pa : 0.f);
+      if (lane == 0) {
+        cl_publish(finals + (g.n * C + c) * 2, b, a, tag);
+        cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+      }
+    }
+    if (!fail) {
+      float fb_, fa_;
+      const bool want = lane < cap_here;
+      if (cl_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, fb_, fa_)) {
+        if (want) constants(lane, gmc, muc, rsc, fb_, fa_);
+      } else {
+        fail = true;
+      }
+    }
+    if (fail && lane == 0) sm_fail = 1;
+  }
+  __syncthreads();
+  // The sums of every slab of instance n2 for this workgroup's tile, as their workgroups compute
+  // them, into fb[slab][channel][2].  The slabs pass through the registers of the workgroup's own
+  // slab (x and dy are intact: dx aliases neither), which the caller loads again if it still
+  // needs it.
+  auto recompute_instance = [&](int64_t n2) {
+    float mu2[V], rs2[V];
+#pragma unroll
+    for (int i = 0; i < V; ++i) mu2[i] = rs2[i] = 0.f;
+    if (g.ch_ok) {
+      load_f32<V>(mean_in + n2 * C + g.coff, mu2);
+      load_f32<V>(rstd_in + n2 * C + g.coff, rs2);
+    }
+    for (int l = 0; l < S; ++l) {
+      const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
+      cl_load_slab<T, V, U, false, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
+      cl_load_slab<T, V, U, false, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
+      float a2[2 * V];
+      __syncthreads();  // the previous round's block sums have been read
+      cl_resident_sums<T, V, U>(rx, rd, ok, mu2, rs2, TPP, lds, a2);
+      if (g.ch_ok && g.slot == 0) {
+        const int lc0 = g.coff - c_base;
+#pragma unroll
+        for (int i = 0; i < V; ++i) {
+          fb[(l * cap + lc0 + i) * 2] = a2[i];
+          fb[(l * cap + lc0 + i) * 2 + 1] = a2[V + i];
+        }
+      }
+    }
+    __syncthreads();
+  };
+  if (sm_fail) {
+    recompute_instance(g.n);
+    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
+      const int c = c_base + lc;
+      const float b = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2] : 0.f);
+      const float a = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f);
+      if (lane == 0) {
+        constants(lc, gamma[c], mean_in[g.n * C + c], rstd_in[g.n * C + c], b, a);
+        if (lc % S == g.s) {  // an owner still serves its peers
+          cl_publish(finals + (g.n * C + c) * 2, b, a, tag);
+          cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+        }
+      }
+    }
+    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+    cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+    __syncthreads();
+  }
+  if (g.ch_ok) {
+    ClBwdCoef<V, false> k;
+    k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      if (ok[u]) {
+        store_pack<T, V>(dx + (g.n * D + g.p0) * C + cl_slab_offset(g, C, u),
+                         k.template apply<T>(rx[u], rd[u]));
+      }
+    }
+  }
+  // dgamma / dbeta: the owners of instance 0 add up the instances' sums, a lane per instance
+  if (g.n != 0 || g.s >= cap_here) return;  // uniform over the workgroup
+  if (wave == 0) {
+    bool fail = false;
+    for (int lc = g.s; lc < cap_here; lc += S) {
+      const int c = c_base + lc;
+      float pb, pa;
+      if (!cl_wait_pair(finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2, lane < N, tag,
+                        max_polls, pb, pa)) {
+        fail = true;
+        break;
+      }
+      const float b = group_sum<kWave>(lane < N ? pb : 0.f);
+      const float a = group_sum<kWave>(lane < N ? pa : 0.f);
+      if (lane == 0) {
+        dgamma[c] = b;
+        dbeta[c] = a;
+      }
+    }
+    if (fail && lane == 0) sm_fail_dev = 1;
+  }
+  __syncthreads();
+  if (sm_fail_dev) {
+    // every instance's sums for the owned channels, recomputed here
+    for (int n2 = 0; n2 < N; ++n2) {
+      recompute_instance(n2);
+      int k = 0;
+      for (int lc = g.s; lc < cap_here; lc += S, ++k) {
+        if (wave == 0) {
+          const float b = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2] : 0.f);
+          const float a = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f);
+          if (lane == 0) {
+            inst[k][n2][0] = b;
+            inst[k][n2][1] = a;
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (wave == 0) {
+      int k = 0;
+      for (int lc = g.s; lc < cap_here; lc += S, ++k) {
+        const float b = group_sum<kWave>(lane < N ? inst[k][lane][0] : 0.f);
+        const float a = group_sum<kWave>(lane < N ? inst[k][lane][1] : 0.f);
+        if (lane == 0) {
+          dgamma[c_base + lc] = b;
+          dbeta[c_base + lc] = a;
+        }
+      }
+    }
+  }
+}
+
+}  // namespace atexn

@@ -1,5 +1,6 @@
 // dtype dispatch, shared helper kernels, error state and tunables.
 #include <atomic>
+#include <chrono>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -37,6 +38,13 @@ const Tuning& tuning() {
   return t;
 }
 #endif
+
+unsigned next_call_tag() {
+  static std::atomic<unsigned> counter{
+      static_cast<unsigned>(std::chrono::steady_clock::now().time_since_epoch().count()) | 1u};
+  unsigned t = counter.fetch_add(1, std::memory_order_relaxed);
+  return t == 0 ? counter.fetch_add(1, std::memory_order_relaxed) : t;
+}
 
 int cu_count() {
   static std::atomic<int> cached[64];

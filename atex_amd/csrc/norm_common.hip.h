@@ -217,6 +217,29 @@ __device__ __forceinline__ T from_f32(float v) {
   return static_cast<T>(v);  // round-to-nearest-even for f16 / bf16
 }
 
+// Half storage: the conversion to float can ride on the multiply-add that consumes the value
+// (v_fma_mix_f32 takes a half operand as it is), which saves the separate v_cvt_f32_f16 per
+// element.  The compiler only forms it from an fma, and folds fma(x, 1, c) back into an add, so
+// the plain sums and differences below multiply by a 1.0f it cannot see through (mix_one()).
+// x * 1 is exact, so each result has the bits of the converted-then-added form.  Kernels whose
+// arithmetic trails their loads (a register-resident slab: every load is issued, then every
+// element is touched twice) are bound by these instruction counts, not by memory.
+__device__ __forceinline__ float mix_one() {
+  float one = 1.0f;
+  asm volatile("" : "+v"(one));
+  return one;
+}
+template <typename T>
+__device__ __forceinline__ float add_f32(float acc, T x, float one) {  // acc + float(x)
+  if constexpr (sizeof(T) == 2 && !__is_same(T, bf16_t)) return __builtin_fmaf(static_cast<float>(x), one, acc);
+  else return acc + to_f32(x);
+}
+template <typename T>
+__device__ __forceinline__ float sub_f32(T x, float m, float one) {  // float(x) - m
+  if constexpr (sizeof(T) == 2 && !__is_same(T, bf16_t)) return __builtin_fmaf(static_cast<float>(x), one, -m);
+  else return to_f32(x) - m;
+}
+
 // V consecutive fp32 values (gamma, beta, saved statistics, partial sums).
 template <int V>
 __device__ __forceinline__ void load_f32(const float* p, float (&out)[V]) {

@@ -58,6 +58,11 @@ struct Tuning {
   TuneInt cl_fold_cap{1};     // channels-last: no more slabs than a stage-2 fold takes from registers
   TuneInt cl_fused_split{1};  // channels-last single pass: narrower channel tiles so that an instance fits
   TuneInt cl_fused{1};        // channels-last: single-pass kernels when an instance fits a workgroup
+  // channels-last: statistics and their use in one launch (cl_single_kernels.hip.h) when every
+  // slab is register-resident and all workgroups fit the chip at once; and how many polls a wait
+  // for a peer's partials may take before a workgroup recomputes them itself (0: at once)
+  TuneInt cl_single{1};
+  TuneInt cl_single_polls{2000};
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
@@ -451,8 +456,19 @@ struct ClPlan {
   bool fused = false;  // one slab per instance and it fits the registers: single-pass kernels
   int fused_u = 0;     //   with fused_u (1, 2, 4, 8 or 16) pixels per thread
   size_t off_a = 0, off_fold = 0, ws_bytes = 0;
+  // One launch per direction (cl_single_kernels.hip.h): the workgroups of an instance exchange
+  // their slab partials while they run.  Needs every workgroup on the chip at once (two per CU),
+  // all workgroups of an instance on one XCD (the instance index is the fastest grid coordinate
+  // and workgroups are dealt to the 8 XCDs in turn: N a multiple of 8), at most 64 slabs and 64
+  // instances (a lane each in the folds) and tiles of at most 64 channels.  The launcher also
+  // wants y != x and a stream that is not being captured; the two-stage kernels stay the
+  // fallback, in the same workspace.
+  bool single = false;
+  size_t off_tagged = 0, off_finals = 0, off_finals_dev = 0;
 };
 constexpr int kClFoldAbove = 64;
+constexpr int kPlanXcds = 8;
+constexpr int kPlanClSingleMaxCap = 64, kPlanClSingleMaxSlabs = 64, kPlanClSingleMaxOwned = 4;
 // slab partials per lane that a stage-2 fold takes in one round trip (cl_kernels.hip.h: twice
 // kClFoldRegs)
 constexpr int kPlanClFoldRegs = 32;
@@ -580,6 +596,19 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
     p.fused_u = std::max(1, pow2_ceil(per_thread));
   }
   p.ws_bytes = p.off_fold + align256(sizeof(float) * 2 * size_t(N) * size_t(C));
+  const int cap_here = static_cast<int>(std::min<int64_t>(cap, C));
+  // (slabs of at most 8 vectors per thread: with 16 the forward kernel does not fit the registers
+  // of two workgroups per CU)
+  p.single = t.cl_single && V > 1 && C % V == 0 && p.U > 0 && p.U <= 8 && !p.fold && !p.fused && p.S >= 2 &&
+             p.S <= kPlanClSingleMaxSlabs && N % kPlanXcds == 0 && N <= 64 && p.n_work <= int64_t(cus) * 2 &&
+             cap <= kPlanClSingleMaxCap && div_up(cap_here, p.S) <= kPlanClSingleMaxOwned;
+  if (p.single) {
+    // tagged pairs: 16 bytes per (instance, slab, channel); finals: 16 bytes per (instance, channel), twice
+    p.off_tagged = 0;
+    p.off_finals = align256(size_t(16) * size_t(N) * size_t(p.S) * size_t(C));
+    p.off_finals_dev = p.off_finals + align256(size_t(16) * size_t(N) * size_t(C));
+    p.ws_bytes = std::max(p.ws_bytes, p.off_finals_dev + align256(size_t(16) * size_t(N) * size_t(C)));
+  }
   return p;
 }
 

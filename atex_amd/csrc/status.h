@@ -15,6 +15,12 @@ const char* last_error();
 // queried, so that the workspace queries stay usable on a host without a GPU.
 int cu_count();
 
+// A tag that no earlier call of this process has used (never 0): the single-launch
+// channels-last kernels mark the partial results they exchange with it, so that whatever an
+// earlier call left in the caller's workspace is never taken for data of this one.  A
+// process-wide atomic counter, started from the clock.
+unsigned next_call_tag();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ATEXN_REQUIRE(cond, ...)                                                  \

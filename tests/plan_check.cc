@@ -170,6 +170,20 @@ static void check_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) 
   }
   const size_t sect = sizeof(float) * size_t(N) * size_t(p.S) * size_t(C);
   EXPECT(p.off_fold >= 2 * sect && p.ws_bytes >= p.off_fold + sizeof(float) * 2 * size_t(N) * size_t(C), "workspace sections");
+  if (p.single) {
+    // what cl_fwd_single / cl_bwd_single assume: resident slabs of at most 8 vectors, whole
+    // channel vectors, a lane per slab and per instance, a tile's channels in LDS, every
+    // workgroup on the chip at once, the workgroups of an instance on one XCD
+    const int cap = p.TPP * V;
+    EXPECT(V > 1 && C % V == 0 && p.U >= 4 && p.U <= 8 && !p.fused && !p.fold, "single: U=%d", p.U);
+    EXPECT(p.S >= 2 && p.S <= 64 && N <= 64 && N % 8 == 0, "single: S=%d N=%lld", p.S, (long long)N);
+    EXPECT(cap <= 64 && div_up(std::min<int64_t>(cap, C), p.S) <= 4, "single: cap=%d S=%d", cap, p.S);
+    EXPECT(p.n_work <= int64_t(cus) * 2, "single: %lld workgroups on %d CUs", (long long)p.n_work, cus);
+    EXPECT(p.off_tagged % 256 == 0 && p.off_finals >= p.off_tagged + size_t(16) * N * p.S * C &&
+               p.off_finals_dev >= p.off_finals + size_t(16) * N * C &&
+               p.ws_bytes >= p.off_finals_dev + size_t(16) * N * C,
+           "single: workspace sections");
+  }
 }
 
 int main() {
@@ -193,7 +207,7 @@ int main() {
         }
       }
       // channels-last InstanceNorm
-      for (int64_t N : {1, 2, 8, 100, 16384, 70000}) {
+      for (int64_t N : {1, 2, 8, 16, 64, 100, 16384, 70000}) {
         for (int64_t C : {1, 3, 8, 16, 32, 64, 100, 256, 520, 2048, 4096, 100000, 1048576, 3000000, 600000000}) {
           for (int64_t D : {1, 2, 5, 32, 64, 100, 1000, 4096, 16384, 262144, 2097152, 16777216}) {
             if (double(N) * double(C) * double(D) > 4e12) continue;

@@ -8,6 +8,7 @@ spatial dim, both layouts, plus the non-typical spatial extents.
 import numpy as np
 import pytest
 
+from oracle import oracle as O
 from tests import util
 from tests.util import TOL, assert_close
 
@@ -288,3 +289,83 @@ def test_channels_last_slab_fold_paths(capi, coracle, N, C, S, dtype):
     slabs, whose partials a launch of its own folds in batches that end in a partial one.  The
     backward cases deal the dgamma / dbeta columns out in chunks of 1, 4, 16 and 64."""
     run_case(capi, coracle, N, C, S, dtype, False, 31)
+
+
+def _bits(t):
+    import torch
+
+    return t.view(torch.uint8)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (8, 32, 4096), (16, 64, 4000), (8, 128, 8192), (8, 24, 5000),
+                                   (32, 64, 4096), (8, 64, 2048), (8, 256, 4096)])
+def test_channels_last_single_launch(coracle, N, C, S, dtype):
+    """Register-resident slabs, every workgroup on the chip at once, N a multiple of 8: statistics
+    and their use run as ONE launch per direction whose workgroups exchange tagged partials while
+    they run.  Checked against the oracle, and three ways against itself through the benchmark
+    build of the library (which can switch the path off and set the poll limit):
+      * with a poll limit of 0 every workgroup gives up waiting at once and recomputes the other
+        slabs itself: the outputs must have the bits of the normal run (the fallback is the same
+        arithmetic), which is also what makes the results independent of timing;
+      * two runs in a row on the same workspace (stale tags of the first call in place) agree;
+      * the two-stage kernels (path switched off) meet the same oracle."""
+    import torch
+
+    capi = util.Capi(bench=True)
+    L = capi.L
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 91)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, m_ref.astype(np.float32), r_ref.astype(np.float32),
+                                            dtype, False)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    md = torch.from_numpy(m_ref.astype(np.float32)).cuda()
+    rd = torch.from_numpy(r_ref.astype(np.float32)).cuda()
+    tol = TOL[dtype]
+    buf = __import__("ctypes").create_string_buffer(256)
+    L.atexn_bench_describe_bwd(1, O.DTYPE_CODE[dtype], 1, N, C, S, buf, 256)
+    print(f"IN channels-last single launch N={N} C={C} spatial={S} {dtype}: {buf.value.decode()}", flush=True)
+    if b"cl_bwd_single" not in buf.value:
+        pytest.skip("this shape and dtype stay on the two-stage kernels")
+
+    def run():
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+        dx, dg, db = capi.in_bwd(dyd, xd, gd, md, rd, dtype, False)
+        torch.cuda.synchronize()
+        return y, m, r, dx, dg, db
+
+    def check(out, what):
+        y, m, r, dx, dg, db = out
+        assert_close(util.to_host(m), m_ref, tol["stat"], what + " mean")
+        assert_close(util.to_host(r), r_ref, tol["stat"], what + " inv_std")
+        assert_close(util.to_host(y), y_ref, tol["y"], what + " y")
+        scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), r_ref, dtype)
+        assert_close(util.to_host(dx), dx_ref, tol["dx"], what + " dx", scale=scale)
+        assert_close(util.to_host(dg), dg_ref, tol["dw"], what + " dgamma")
+        assert_close(util.to_host(db), db_ref, tol["dw"], what + " dbeta")
+
+    names = ("y", "mean", "inv_std", "dx", "dgamma", "dbeta")
+    try:
+        normal = run()
+        check(normal, "single launch")
+        again = run()
+        for n_, a, b in zip(names, normal, again):
+            assert torch.equal(_bits(a), _bits(b)), f"second run differs in {n_}"
+        assert L.atexn_set_tuning(b"cl_single_polls", 0) == 0
+        alone = run()
+        check(alone, "single launch, poll limit 0")
+        for n_, a, b in zip(names, normal, alone):
+            assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
+        assert L.atexn_set_tuning(b"cl_single_polls", 2000) == 0
+        assert L.atexn_set_tuning(b"cl_single", 0) == 0
+        check(run(), "two stages")
+    finally:
+        L.atexn_set_tuning(b"cl_single_polls", 2000)
+        L.atexn_set_tuning(b"cl_single", 1)
+
+
+def test_channels_last_single_launch_in_place_takes_two_stages(capi, coracle):
+    """y written over x (dx over dy) keeps a call off the single-launch kernels, whose fallback
+    reads other workgroups' parts of x: results as good as out of place."""
+    run_case(capi, coracle, 8, 64, 16384, "f16", False, 92, in_place=True)

@@ -266,6 +266,8 @@ def test_every_planning_parameter_is_settable_in_the_benchmark_build():
     assert L.atexn_bench_describe_bwd(0, 1, 0, 8192, 0, 1024, buf, 256) > 0
     assert b"rows_bwd_resident" in buf.value and b"alone=1" in buf.value
     assert L.atexn_bench_describe_bwd(1, 1, 1, 8, 64, 16384, buf, 256) > 0
+    assert b"cl_bwd_single" in buf.value and b"alone=0" in buf.value
+    assert L.atexn_bench_describe_bwd(1, 1, 1, 2, 32, 2097152, buf, 256) > 0
     assert b"cl_bwd_sums" in buf.value and b"alone=0" in buf.value
 
 
