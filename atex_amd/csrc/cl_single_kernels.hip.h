@@ -64,22 +64,26 @@ __device__ __forceinline__ void cl_publish_device(cl_word* pair, float a, float 
   __hip_atomic_store(pair + 1, cl_tagged(b, ~tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
-// One wave waits for the pair at `pair` (per lane; lanes with want == false wait for nothing):
-// true once every wanted lane has read both words with this call's tag, false after max_polls
-// rounds.  All 64 lanes of the wave must call it; the result is the same in all of them.
+// One round of a wave's wait for the pair at `pair` (per lane; lanes with want == false wait for
+// nothing): reads both words and tells whether every wanted lane found this call's tag in both.
+// All 64 lanes of the wave must call it; the result is the same in all of them.
+__device__ __forceinline__ bool cl_try_pair(const cl_word* pair, bool want, unsigned tag, float& a, float& b) {
+  bool ready = true;
+  if (want) {
+    const cl_word w0 = cl_peek(pair);
+    const cl_word w1 = cl_peek(pair + 1);
+    ready = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
+    a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
+    b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
+  }
+  return __all(ready);
+}
+// The wait itself: true once a round succeeds, false after max_polls rounds.
 __device__ __forceinline__ bool cl_wait_pair(const cl_word* pair, bool want, unsigned tag, int max_polls,
                                              float& a, float& b) {
   a = b = 0.f;
   for (int poll = 0; poll < max_polls; ++poll) {
-    bool ready = true;
-    if (want) {
-      const cl_word w0 = cl_peek(pair);
-      const cl_word w1 = cl_peek(pair + 1);
-      ready = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
-      a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
-      b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
-    }
-    if (__all(ready)) return true;
+    if (cl_try_pair(pair, want, tag, a, b)) return true;
   }
   return false;
 }
@@ -378,6 +382,14 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
     __syncthreads();
   }
+  // The owners of instance 0 also fold the instances' sums into dgamma / dbeta (below, after
+  // their dx is on its way).  The other instances' owners published their sums a hop ago: a first
+  // look now, whose round trip passes under the stores, usually finds them.
+  const bool folds_instances = g.n == 0 && g.s < cap_here;  // uniform over the workgroup
+  const cl_word* first_dev = finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c_base + g.s) * 2;
+  float eb = 0.f, ea = 0.f;
+  bool early = false;
+  if (folds_instances && wave == 0 && max_polls > 0) early = cl_try_pair(first_dev, lane < N, tag, eb, ea);
   if (g.ch_ok) {
     ClBwdCoef<V, false> k;
     k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);
@@ -390,13 +402,15 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     }
   }
   // dgamma / dbeta: the owners of instance 0 add up the instances' sums, a lane per instance
-  if (g.n != 0 || g.s >= cap_here) return;  // uniform over the workgroup
+  // (the first owned channel's may have arrived with the early look)
+  if (!folds_instances) return;
   if (wave == 0) {
     bool fail = false;
     for (int lc = g.s; lc < cap_here; lc += S) {
       const int c = c_base + lc;
-      float pb, pa;
-      if (!cl_wait_pair(finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2, lane < N, tag,
+      float pb = eb, pa = ea;
+      if (!(early && lc == g.s) &&
+          !cl_wait_pair(finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2, lane < N, tag,
                         max_polls, pb, pa)) {
         fail = true;
         break;

@@ -107,11 +107,14 @@ TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
 # what the same counter reads for the 64 MiB negation of --copy-calibration (FETCH_SIZE x 2.0,
 # WRITE_SIZE x 1.0).  Summaries: profiles/<case>_hbm_traffic.txt.  Cases without a run: None.
 MEASURED_TRAFFIC = {
-    "ln_bert": 52.78e6,                 # rows_bwd_resident
-    "in2d_nchw": 50.51e6,               # rows_bwd_resident (row-affine)
-    "in2d_nhwc": 33.99e6 + 52.59e6,     # cl_bwd_sums + cl_bwd_apply
-    "in3d_ndhwc": 537.01e6 + 805.34e6,  # cl_bwd_sums + cl_bwd_apply
-    "in3d_ncdhw": 536.84e6 + 805.38e6,  # split_bwd_sums + split_bwd_apply
+    "ln_bert": 52.79e6,                 # rows_bwd_resident
+    "ln_128_f16": 203.73e6,             # rows_bwd_resident
+    "ln_4096_f16": 412.22e6,            # rows_bwd_resident
+    "ln_12288_f16": 176.84e6,           # rows_bwd_resident (151.0 MB of rows + 25.2 MB of partial rows)
+    "in2d_nchw": 50.50e6,               # rows_bwd_resident (row-affine)
+    "in2d_nhwc": 51.67e6,               # cl_bwd_single
+    "in3d_ndhwc": 536.94e6 + 805.88e6,  # cl_bwd_sums + cl_bwd_apply
+    "in3d_ncdhw": 536.86e6 + 805.36e6,  # split_bwd_sums + split_bwd_apply
 }
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
@@ -578,8 +581,9 @@ def main():
     ap.add_argument("--no-targets", action="store_true",
                     help="default case only: skip the InstanceNorm target shapes and the other configurations")
     ap.add_argument("--cold-only", action="store_true",
-                    help="only the rotating-buffer (cold) legs: no hot-cache loop, no HIP-graph replay, no "
-                         "torch copy / add; what a rocprofv3 kernel trace of this file should average over")
+                    help="only the rotating-buffer (cold) legs: no hot-cache loop and no HIP-graph replay (and no "
+                         "torch copy / add for the targets and configurations of the default run); what a "
+                         "rocprofv3 kernel trace of this file should average over")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
                          "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
