@@ -66,3 +66,64 @@ def test_graph_replay_matches_eager(case):
         del junk
         for name, got, ref in zip(("y", "mean", "inv_std", "dx", "dgamma", "dbeta"), outs, eager):
             assert torch.equal(got, ref), f"replay {replay}: {name} differs from the eager result"
+
+
+def test_graph_capture_of_a_single_launch_shape(coracle):
+    """Channels-last shapes that run as one launch per direction in eager mode (the workgroups
+    exchange partials tagged with a per-call number) are recorded as the two-stage kernels when
+    the stream is being captured, since a replay would repeat the tag.  The replays must agree
+    with each other bit for bit and with the oracle; against the eager (single-launch) result only
+    the last bits of the statistics may differ (another order of the same additions)."""
+    import torch
+
+    from tests.util import TOL, assert_close
+
+    capi = util.Capi()
+    dtype, N, C, S = "f16", 8, 64, 4096
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 33)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
+    print(f"graph capture of IN channels-last N={N} C={C} spatial={S} {dtype}", flush=True)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+    dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
+    torch.cuda.synchronize()
+    eager = [t.clone() for t in (y, m, r, dx, dg, db)]
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, False)
+
+    graph = torch.cuda.CUDAGraph()
+    s = torch.cuda.Stream()
+    s.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(s):
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+        capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
+    torch.cuda.current_stream().wait_stream(s)
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph):
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
+        dx, dg, db = capi.in_bwd(dyd, xd, gd, eager[1], eager[2], dtype, False)
+    outs = (y, m, r, dx, dg, db)
+    first = None
+    tol = TOL[dtype]
+    for replay in range(3):
+        for t in outs:
+            t.fill_(float("nan"))
+        junk = torch.randn(1 << 20, device="cuda").sum()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        del junk
+        if first is None:
+            first = [t.clone() for t in outs]
+            assert_close(util.to_host(m), m_ref, tol["stat"], "mean")
+            assert_close(util.to_host(r), r_ref, tol["stat"], "inv_std")
+            assert_close(util.to_host(y), y_ref, tol["y"], "y")
+            scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), util.to_host(eager[2]), dtype)
+            assert_close(util.to_host(dx), dx_ref, tol["dx"], "dx", scale=scale)
+            assert_close(util.to_host(dg), dg_ref, tol["dw"], "dgamma")
+            assert_close(util.to_host(db), db_ref, tol["dw"], "dbeta")
+            assert_close(util.to_host(m), util.to_host(eager[1]), 1e-6, "mean vs eager")
+            assert_close(util.to_host(r), util.to_host(eager[2]), 1e-6, "inv_std vs eager")
+        else:
+            for name, got, ref in zip(("y", "mean", "inv_std", "dx", "dgamma", "dbeta"), outs, first):
+                assert torch.equal(got, ref), f"replay {replay}: {name} differs from the first replay"
