@@ -38,55 +38,9 @@
 
 namespace atexn {
 
-typedef unsigned long long cl_word;
-
 constexpr int kClSingleMaxCap = 64;    // channels per tile (the fallback keeps S x cap pairs in LDS)
 constexpr int kClSingleMaxSlabs = 64;  // slabs per instance: one lane each in the owner's fold
 constexpr int kClSingleMaxOwned = 4;   // channels one workgroup may own
-
-__device__ __forceinline__ cl_word cl_tagged(float v, unsigned tag) {
-  return static_cast<cl_word>(__builtin_bit_cast(unsigned, v)) | (static_cast<cl_word>(tag) << 32);
-}
-__device__ __forceinline__ cl_word cl_peek(const cl_word* p) {
-  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-// A pair of tagged words as one 16-byte store (each aligned 8-byte half lands whole).
-__device__ __forceinline__ void cl_publish(cl_word* pair, float a, float b, unsigned tag) {
-  typedef cl_word w2 __attribute__((ext_vector_type(2)));
-  w2 v;
-  v.x = cl_tagged(a, tag);
-  v.y = cl_tagged(b, ~tag);
-  *reinterpret_cast<w2*>(pair) = v;
-}
-// The same, written through to memory (readers on other XCDs).
-__device__ __forceinline__ void cl_publish_device(cl_word* pair, float a, float b, unsigned tag) {
-  __hip_atomic_store(pair, cl_tagged(a, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  __hip_atomic_store(pair + 1, cl_tagged(b, ~tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-// One round of a wave's wait for the pair at `pair` (per lane; lanes with want == false wait for
-// nothing): reads both words and tells whether every wanted lane found this call's tag in both.
-// All 64 lanes of the wave must call it; the result is the same in all of them.
-__device__ __forceinline__ bool cl_try_pair(const cl_word* pair, bool want, unsigned tag, float& a, float& b) {
-  bool ready = true;
-  if (want) {
-    const cl_word w0 = cl_peek(pair);
-    const cl_word w1 = cl_peek(pair + 1);
-    ready = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
-    a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
-    b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
-  }
-  return __all(ready);
-}
-// The wait itself: true once a round succeeds, false after max_polls rounds.
-__device__ __forceinline__ bool cl_wait_pair(const cl_word* pair, bool want, unsigned tag, int max_polls,
-                                             float& a, float& b) {
-  a = b = 0.f;
-  for (int poll = 0; poll < max_polls; ++poll) {
-    if (cl_try_pair(pair, want, tag, a, b)) return true;
-  }
-  return false;
-}
 
 // (mean, m2) of an instance from its slabs' (mean, m2), one slab per lane of a wave (lanes
 // >= S hold nothing): Chan's merge of all slabs at once, as cl_fold_stats does it.

@@ -363,6 +363,61 @@ __device__ __forceinline__ float group_sum(float v) {
   return v;
 }
 
+// ---------------------------------------------------- values exchanged between workgroups
+// Workgroups of one launch that hand each other partial results through memory while they run
+// (the single-launch channels-last kernels, the channel-first backward's fold over the batch)
+// write every value as an 8-byte word (value, tag) with one store.  The tag is a number that
+// no earlier call of the process has used, so a word either still carries an older call's tag
+// or is complete: no separate flag, no fence, nothing to clear between calls.  Values travel in
+// pairs; the second word carries the complemented tag, so 64 bits of arbitrary memory would
+// have to match before garbage in a fresh workspace could pass for data.  Readers poll with
+// device-scope loads, which never return a stale cache line, a bounded number of times.
+typedef unsigned long long cl_word;
+
+__device__ __forceinline__ cl_word cl_tagged(float v, unsigned tag) {
+  return static_cast<cl_word>(__builtin_bit_cast(unsigned, v)) | (static_cast<cl_word>(tag) << 32);
+}
+__device__ __forceinline__ cl_word cl_peek(const cl_word* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// A pair of tagged words as one 16-byte store (each aligned 8-byte half lands whole).
+__device__ __forceinline__ void cl_publish(cl_word* pair, float a, float b, unsigned tag) {
+  typedef cl_word w2 __attribute__((ext_vector_type(2)));
+  w2 v;
+  v.x = cl_tagged(a, tag);
+  v.y = cl_tagged(b, ~tag);
+  *reinterpret_cast<w2*>(pair) = v;
+}
+// The same, written through to memory (readers on other XCDs).
+__device__ __forceinline__ void cl_publish_device(cl_word* pair, float a, float b, unsigned tag) {
+  __hip_atomic_store(pair, cl_tagged(a, tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(pair + 1, cl_tagged(b, ~tag), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// One round of a wave's wait for the pair at `pair` (per lane; lanes with want == false wait for
+// nothing): reads both words and tells whether every wanted lane found this call's tag in both.
+// All 64 lanes of the wave must call it; the result is the same in all of them.
+__device__ __forceinline__ bool cl_try_pair(const cl_word* pair, bool want, unsigned tag, float& a, float& b) {
+  bool ready = true;
+  if (want) {
+    const cl_word w0 = cl_peek(pair);
+    const cl_word w1 = cl_peek(pair + 1);
+    ready = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
+    a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
+    b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
+  }
+  return __all(ready);
+}
+// The wait itself: true once a round succeeds, false after max_polls rounds.
+__device__ __forceinline__ bool cl_wait_pair(const cl_word* pair, bool want, unsigned tag, int max_polls,
+                                             float& a, float& b) {
+  a = b = 0.f;
+  for (int poll = 0; poll < max_polls; ++poll) {
+    if (cl_try_pair(pair, want, tag, a, b)) return true;
+  }
+  return false;
+}
+
 // Loops over strided indices are written in batches of B whose loads are all issued before
 // the first is consumed: the compiler does not move a load above the bounds check of the
 // iteration before it, so a plain loop would pay one memory latency per iteration.

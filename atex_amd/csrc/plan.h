@@ -63,6 +63,8 @@ struct Tuning {
   // for a peer's partials may take before a workgroup recomputes them itself (0: at once)
   TuneInt cl_single{1};
   TuneInt cl_single_polls{2000};
+  TuneInt affine_fold{1};      // channel-first backward, a workgroup per plane: dgamma / dbeta folded over the batch in the row kernel
+  TuneInt affine_fold_polls{2000};  //   polls before a workgroup recomputes its peers' plane sums (0: at once)
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
@@ -90,6 +92,7 @@ inline int bwd_stage_mask() {
 #endif
 }
 
+constexpr int kPlanXcdCount = 8;  // workgroups are dealt to the XCDs of an MI355X in turn
 enum class RowsKind { kFwd, kBwdCols /*LayerNorm: per-column dgamma/dbeta*/, kBwdAffine };
 
 inline int64_t div_up(int64_t a, int64_t b) { return (a + b - 1) / b; }
@@ -120,6 +123,12 @@ struct RowsPlan {
   // workspace sections (bytes from the start of the workspace)
   size_t off_part = 0, off_pairs = 0, ws_bytes = 0;
   int part_rows = 0;  // G of the column reduction
+  // Channel-first backward with a workgroup per plane: the fold of the plane sums over the batch
+  // runs inside the row kernel (tagged pairs at off_tagged, 16 bytes per plane) instead of as a
+  // col_reduce launch.  Needs the planes of a channel on one XCD (C and the grid multiples of the
+  // XCD count), at most 64 instances; the launcher also wants dx != dy and no stream capture.
+  bool affine_fold = false;
+  size_t off_tagged = 0;
 };
 
 // Longest row, in vectors, that the register-resident kernels take: forward 8 vectors per
@@ -343,6 +352,12 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.part_rows = static_cast<int>(n_rows / C);
       p.off_part = 0;
       p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
+      p.affine_fold = t.affine_fold && p.tpr == 0 && C % kPlanXcdCount == 0 && p.grid % kPlanXcdCount == 0 &&
+                      p.part_rows >= 2 && p.part_rows <= 64;
+      if (p.affine_fold) {
+        p.off_tagged = p.ws_bytes;
+        p.ws_bytes += align256(size_t(16) * size_t(n_rows));
+      }
     }
     return p;
   }
@@ -467,7 +482,6 @@ struct ClPlan {
   size_t off_tagged = 0, off_finals = 0, off_finals_dev = 0;
 };
 constexpr int kClFoldAbove = 64;
-constexpr int kPlanXcds = 8;
 constexpr int kPlanClSingleMaxCap = 64, kPlanClSingleMaxSlabs = 64, kPlanClSingleMaxOwned = 4;
 // slab partials per lane that a stage-2 fold takes in one round trip (cl_kernels.hip.h: twice
 // kClFoldRegs)
@@ -600,7 +614,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   // (slabs of at most 8 vectors per thread: with 16 the forward kernel does not fit the registers
   // of two workgroups per CU)
   p.single = t.cl_single && V > 1 && C % V == 0 && p.U > 0 && p.U <= 8 && !p.fold && !p.fused && p.S >= 2 &&
-             p.S <= kPlanClSingleMaxSlabs && N % kPlanXcds == 0 && N <= 64 && p.n_work <= int64_t(cus) * 2 &&
+             p.S <= kPlanClSingleMaxSlabs && N % kPlanXcdCount == 0 && N <= 64 && p.n_work <= int64_t(cus) * 2 &&
              cap <= kPlanClSingleMaxCap && div_up(cap_here, p.S) <= kPlanClSingleMaxOwned;
   if (p.single) {
     // tagged pairs: 16 bytes per (instance, slab, channel); finals: 16 bytes per (instance, channel), twice

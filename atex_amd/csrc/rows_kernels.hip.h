@@ -391,13 +391,32 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // N * 2 * C floats and the same second kernel folds it over n.
 // dx may alias dy (a thread reads its elements of a row before it writes them), not x.
 // RB / EXACT / prefetch as in the forward kernel.
+// Channel-first InstanceNorm with a workgroup per plane: the fold of the per-plane sums over the
+// batch (dgamma[c] = sum over n of the plane sums of (n, c)) can run inside the row kernel instead
+// of as a launch of its own.  Every workgroup publishes the two sums of its plane as a tagged
+// pair as soon as it has them, before it computes and stores dx; the workgroup that handled plane
+// (0, c) afterwards waits (a lane per instance, a bounded number of polls) for the N pairs of
+// channel c and adds them up.  The host asks for it only when the planes of a channel are all
+// handled on one XCD (C and the grid multiples of the XCD count: plane n * C + c goes to
+// workgroup (n * C + c) mod grid), so that plain stores are visible to the device-scope polls,
+// when N <= 64, dx != dy and the stream is not being captured.  A workgroup whose wait runs out
+// recomputes the sums of the N planes itself, with the code the row loop uses (same bits).
+struct AffineFold {
+  cl_word* tagged = nullptr;  // [N * C] pairs (sum dy * xh, sum dy); nullptr: col_reduce follows
+  float* dgamma = nullptr;
+  float* dbeta = nullptr;
+  unsigned tag = 0;
+  int max_polls = 0;
+  int N = 0;
+};
+
 template <typename T, int V, int TPR, int VPT, int RB, bool EXACT, bool ROW_AFFINE,
           bool RAGGED = false>
 __global__ void __launch_bounds__((resident_bwd_max_threads<TPR, !ROW_AFFINE, RB, VPT>()))
 rows_bwd_resident(const T* dy, const T* __restrict__ x,
                   const float* __restrict__ gamma, const float* __restrict__ mean_in,
                   const float* __restrict__ rstd_in, T* dx,
-                  float* __restrict__ part, int64_t n_rows, int d_elems, int C) {
+                  float* __restrict__ part, int64_t n_rows, int d_elems, int C, AffineFold fold) {
   using M = RowMap<TPR>;
   constexpr int NE = V * VPT;
   static_assert(!(RAGGED && (EXACT || V == 1)), "ragged rows use the non-exact vector variants");
@@ -486,14 +505,10 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
   // kernel, a vector slot past the row holds the row's last vector again, and is masked out of
   // the row sums only; dx of it is stored like every other (the same bits as its owner's).
   constexpr bool DUP_SLOTS = !EXACT && TPR == 0;
-  auto process = [&](Batch& cur, int64_t row0, int it) {
-    bool row_ok[RB];
-#pragma unroll
-    for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
-    // stage 1: convert once; xh = (x - mean) * r, gv = dy * gamma; row sums and the
-    // column accumulators.  Elements outside the row are 0 and add nothing.
-    float xh[RB][NE], gv[RB][NE];
-    float s1[RB], s2[RB];
+  // stage 1: convert once; xh = (x - mean) * r, gv = dy * gamma; row sums and the
+  // column accumulators.  Elements outside the row are 0 and add nothing.
+  auto row_sums = [&](Batch& cur, const bool (&row_ok)[RB], float (&xh)[RB][NE], float (&gv)[RB][NE],
+                      float (&s1)[RB], float (&s2)[RB], int it) {
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
       float a1 = 0.f, a2 = 0.f;
@@ -550,6 +565,14 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
         s2[r] = t.y;
       }
     }
+  };
+  auto process = [&](Batch& cur, int64_t row0, int it) {
+    bool row_ok[RB];
+#pragma unroll
+    for (int r = 0; r < RB; ++r) row_ok[r] = EXACT || row0 + r * rpb + slot < n_rows;
+    float xh[RB][NE], gv[RB][NE];
+    float s1[RB], s2[RB];
+    row_sums(cur, row_ok, xh, gv, s1, s2, it);
     // stage 2: dx = scale * gv + (A * xh + B), A = -scale * s2 / D, B = -scale * s1 / D
 #pragma unroll
     for (int r = 0; r < RB; ++r) {
@@ -558,10 +581,14 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       if constexpr (ROW_AFFINE) {
         scale *= cur.gm[r];
         if (row_ok[r] && lane_r == 0) {
-          const int64_t n = row / C;
-          const int c = static_cast<int>(row % C);
-          part[(n * 2 + 0) * C + c] = s2[r];
-          part[(n * 2 + 1) * C + c] = s1[r];
+          if (TPR == 0 && fold.tagged != nullptr) {
+            cl_publish(fold.tagged + row * 2, s2[r], s1[r], fold.tag);
+          } else {
+            const int64_t n = row / C;
+            const int c = static_cast<int>(row % C);
+            part[(n * 2 + 0) * C + c] = s2[r];
+            part[(n * 2 + 1) * C + c] = s1[r];
+          }
         }
       }
       const float ca = -scale * (s2[r] * inv_d), cb = -scale * (s1[r] * inv_d);
@@ -621,6 +648,60 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
     }
   }
 
+  if constexpr (ROW_AFFINE && TPR == 0) {
+    if (fold.tagged != nullptr) {
+      // dgamma / dbeta of the channels whose first plane this workgroup handled
+      __shared__ int fold_failed;
+      __shared__ float inst[kWave][2];
+      const int lane = threadIdx.x & (kWave - 1);
+      const int wave = threadIdx.x / kWave;
+      const int N = fold.N;
+      int it = 0;
+      for (int64_t c = blockIdx.x; c < C && c < n_rows; c += gridDim.x) {
+        if (wave == 0) {
+          float pb, pa;
+          const bool ok = cl_wait_pair(fold.tagged + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2,
+                                       lane < N, fold.tag, fold.max_polls, pb, pa);
+          if (ok) {
+            const float b = group_sum<kWave>(lane < N ? pb : 0.f);
+            const float a = group_sum<kWave>(lane < N ? pa : 0.f);
+            if (lane == 0) {
+              fold.dgamma[c] = b;
+              fold.dbeta[c] = a;
+            }
+          }
+          if (lane == 0) fold_failed = ok ? 0 : 1;
+        }
+        __syncthreads();
+        if (fold_failed) {  // uniform: the planes of channel c, summed here as their workgroups sum them
+          for (int n = 0; n < N; ++n) {
+            Batch t;
+            load_batch(static_cast<int64_t>(n) * C + c, t);
+            bool row_ok[RB];
+#pragma unroll
+            for (int r = 0; r < RB; ++r) row_ok[r] = true;
+            float xh[RB][NE], gv[RB][NE];
+            float s1[RB], s2[RB];
+            row_sums(t, row_ok, xh, gv, s1, s2, it++);
+            if (threadIdx.x == 0) {
+              inst[n][0] = s2[0];
+              inst[n][1] = s1[0];
+            }
+          }
+          __syncthreads();
+          if (wave == 0) {
+            const float b = group_sum<kWave>(lane < N ? inst[lane < N ? lane : 0][0] : 0.f);
+            const float a = group_sum<kWave>(lane < N ? inst[lane < N ? lane : 0][1] : 0.f);
+            if (lane == 0) {
+              fold.dgamma[c] = b;
+              fold.dbeta[c] = a;
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
   if constexpr (!ROW_AFFINE) {
     float* prow = part + static_cast<int64_t>(blockIdx.x) * 2 * D;
     if constexpr (TPR == 0) {

@@ -15,12 +15,23 @@ namespace atexn {
 static_assert(kFoldLdsBytes == kPlanFoldLdsBytes && kFoldMaxWaves == kPlanFoldMaxWaves,
               "the planner sizes the fold's LDS with the kernels' constants");
 
+// The in-kernel fold over the batch tags what it exchanges with a number taken per call, which a
+// graph replay would repeat: callers that capture get the col_reduce launch.
+inline bool rows_stream_is_capturing(hipStream_t st) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return true;
+  }
+  return status != hipStreamCaptureStatusNone;
+}
+
 template <typename T, int V, bool AFF>
 using FwdResidentFn = void (*)(const T*, const float*, const float*, T*, float*, float*, int64_t,
                                int, int, float);
 template <typename T, int V, bool AFF>
 using BwdResidentFn = void (*)(const T*, const T*, const float*, const float*, const float*, T*,
-                               float*, int64_t, int, int);
+                               float*, int64_t, int, int, AffineFold);
 
 // Row batching (RB > 1) exists for the vector path and rows of at most one wave; the
 // predicate-free EXACT variants exist for the vector path.
@@ -310,10 +321,25 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
   if (p.resident) {
     auto fn = pick_bwd_resident<T, V, AFF>(p.tpr, p.vpt, p.rb, p.exact, p.ragged);
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
+    AffineFold fold;
+    if (AFF && p.affine_fold && static_cast<const void*>(dx) != static_cast<const void*>(dy) &&
+        !rows_stream_is_capturing(st)) {
+      // the plane sums are folded over the batch inside the row kernel: no col_reduce
+      fold.tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_tagged);
+      fold.dgamma = dgamma;
+      fold.dbeta = dbeta;
+      fold.tag = next_call_tag();
+      fold.max_polls = tuning().affine_fold_polls;
+      fold.N = p.part_rows;
+      fn<<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
+                                                static_cast<int>(D), C, fold);
+      ATEXN_CHECK_LAUNCH("rows_bwd_resident");
+      return ATEXN_OK;
+    }
     const int stages = bwd_stage_mask();
     if (stages & 1) {
       fn<<<p.grid, p.threads, p.fold_lds, st>>>(dy, x, gamma, mean, rstd, dx, part, n_rows,
-                                                static_cast<int>(D), C);
+                                                static_cast<int>(D), C, fold);
       ATEXN_CHECK_LAUNCH("rows_bwd_resident");
     }
     if (!(stages & 2)) return ATEXN_OK;

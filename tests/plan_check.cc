@@ -128,6 +128,15 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
     } else if (kind == RowsKind::kBwdAffine) {
       EXPECT(n_rows % C == 0 && p.part_rows == n_rows / C, "affine part rows");
       EXPECT(p.ws_bytes >= sizeof(float) * 2 * size_t(n_rows), "affine workspace");
+      if (p.affine_fold) {
+        // what the in-kernel fold over the batch assumes: a workgroup per plane, a lane per
+        // instance, the planes of a channel handled on one XCD, its tagged pairs in the workspace
+        EXPECT(p.tpr == 0 && p.rb == 1 && p.part_rows >= 2 && p.part_rows <= 64, "affine fold: tpr=%d N=%d", p.tpr, p.part_rows);
+        EXPECT(C % 8 == 0 && p.grid % 8 == 0, "affine fold: C=%d grid=%d", C, p.grid);
+        EXPECT(p.off_tagged % 256 == 0 && p.off_tagged >= sizeof(float) * 2 * size_t(n_rows) &&
+                   p.ws_bytes >= p.off_tagged + size_t(16) * size_t(n_rows),
+               "affine fold: workspace");
+      }
     }
   } else {
     EXPECT(!layer_norm, "LayerNorm rows beyond the resident limit go to the tiles");
@@ -198,7 +207,7 @@ int main() {
         }
       }
       // channel-first InstanceNorm: rows = N * C planes
-      for (int64_t N : {1, 2, 8, 100}) {
+      for (int64_t N : {1, 2, 8, 64, 100}) {
         for (int C : {1, 3, 32, 64, 100, 1024}) {
           for (int64_t D = 1; D <= 3000000; D += (D < 2100 ? 1 : (D < 70000 ? 211 : 65537))) {
             check_rows(RowsKind::kFwd, false, vec, N * C, D, C, cus);

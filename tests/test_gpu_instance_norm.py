@@ -369,3 +369,64 @@ def test_channels_last_single_launch_in_place_takes_two_stages(capi, coracle):
     """y written over x (dx over dy) keeps a call off the single-launch kernels, whose fallback
     reads other workgroups' parts of x: results as good as out of place."""
     run_case(capi, coracle, 8, 64, 16384, "f16", False, 92, in_place=True)
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (8, 32, 4096), (16, 64, 3000), (64, 8, 32768), (2, 16, 5001),
+                                   (24, 40, 2048)])
+def test_channel_first_backward_folds_the_batch_in_the_row_kernel(coracle, N, C, S, dtype):
+    """Channel-first planes with a workgroup each, C a multiple of 8, at most 64 instances: the
+    backward's row kernel publishes its plane sums as tagged pairs and the workgroups of instance
+    0 add them up over the batch into dgamma / dbeta, instead of a col_reduce launch.  Checked
+    against the oracle and, through the benchmark build, against itself with the poll limit
+    forced to 0 (every folding workgroup recomputes the plane sums of its channel itself: same
+    bits), twice on the same workspace, and with the fold switched off (col_reduce again)."""
+    import ctypes
+
+    import torch
+
+    capi = util.Capi(bench=True)
+    L = capi.L
+    buf = ctypes.create_string_buffer(384)
+    L.atexn_bench_describe_bwd(1, O.DTYPE_CODE[dtype], 0, N, C, S, buf, 384)
+    print(f"IN channel-first N={N} C={C} spatial={S} {dtype}: {buf.value.decode()}", flush=True)
+    if b"folded over the batch in the kernel" not in buf.value:
+        pytest.skip("this shape and dtype keep the col_reduce launch")
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, True, 93)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, True)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, m_ref.astype(np.float32), r_ref.astype(np.float32),
+                                            dtype, True)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd = torch.from_numpy(gamma).cuda()
+    md = torch.from_numpy(m_ref.astype(np.float32)).cuda()
+    rd = torch.from_numpy(r_ref.astype(np.float32)).cuda()
+    tol = TOL[dtype]
+
+    def run():
+        out = capi.in_bwd(dyd, xd, gd, md, rd, dtype, True)
+        torch.cuda.synchronize()
+        return out
+
+    def check(out, what):
+        dx, dg, db = out
+        scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), r_ref, dtype)
+        assert_close(util.to_host(dx), dx_ref, tol["dx"], what + " dx", scale=scale)
+        assert_close(util.to_host(dg), dg_ref, tol["dw"], what + " dgamma")
+        assert_close(util.to_host(db), db_ref, tol["dw"], what + " dbeta")
+
+    try:
+        normal = run()
+        check(normal, "fold in the kernel")
+        again = run()
+        for n_, a, b in zip(("dx", "dgamma", "dbeta"), normal, again):
+            assert torch.equal(_bits(a), _bits(b)), f"second run differs in {n_}"
+        assert L.atexn_set_tuning(b"affine_fold_polls", 0) == 0
+        alone = run()
+        for n_, a, b in zip(("dx", "dgamma", "dbeta"), normal, alone):
+            assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
+        assert L.atexn_set_tuning(b"affine_fold_polls", 2000) == 0
+        assert L.atexn_set_tuning(b"affine_fold", 0) == 0
+        check(run(), "col_reduce")
+    finally:
+        L.atexn_set_tuning(b"affine_fold_polls", 2000)
+        L.atexn_set_tuning(b"affine_fold", 1)
