@@ -42,6 +42,12 @@ def test_concurrent_threads_and_streams():
         "ln_long": ((6, 70000), 70000),
         "in_cl": ((4, 64 * 64, 64), 64),
         "in_cf": ((4, 64, 64 * 64), 64),
+        # batches of 8: the channels-last kernels whose workgroups exchange partial results while
+        # they run (all of them must be on the chip, which two such launches at once contend for:
+        # a wait that runs out makes a workgroup recompute its peers' share, to the same bits) and
+        # the channel-first backward that folds its plane sums over the batch in the row kernel
+        "in_cl_single": ((8, 128 * 128, 64), 64),
+        "in_cf_fold": ((8, 64, 128 * 128), 64),
     }
     data = {}
     for key, (shape, P) in jobs.items():
@@ -53,7 +59,7 @@ def test_concurrent_threads_and_streams():
     torch.cuda.synchronize()
 
     def kind_of(key):
-        return "ln" if key.startswith("ln") else key
+        return "ln" if key.startswith("ln") else key[:5]
 
     # single-threaded results on the default stream
     ref = {}
@@ -61,7 +67,7 @@ def test_concurrent_threads_and_streams():
         _work(capi, torch, kind_of(key), x, dy, gamma, beta, torch.cuda.current_stream(), ref, key, 1)
         assert not isinstance(ref[key], Exception), ref[key]
 
-    print("concurrent threads: 4 jobs x 2 threads each, own streams", flush=True)
+    print(f"concurrent threads: {len(data)} jobs x 2 threads each, own streams", flush=True)
     out = {}
     threads = []
     for key, (x, dy, gamma, beta) in data.items():

@@ -158,3 +158,41 @@ def test_rows_kept_in_lds_random(coracle, seed):
         finally:
             assert capi.L.atexn_set_tuning(b"staged_rows", 1) == 0
     _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
+
+
+@pytest.mark.parametrize("seed", range(max(1, N_SEEDS // 2)))
+def test_exchange_paths_random(coracle, seed):
+    """Shapes drawn for the kernels whose workgroups hand each other partial results while they
+    run: channels-last with batches that are multiples of 8 (one launch per direction) and
+    channel-first planes with C a multiple of 8 (plane sums folded over the batch in the row
+    kernel), at random sizes around their limits, misaligned tensors and in-place calls (which
+    must take the other kernels) included.  Against the oracle."""
+    import torch
+
+    capi = util.Capi()
+    rng = np.random.Generator(np.random.PCG64(11000 + seed))
+    cf = bool(seed % 2)
+    N = int(8 * rng.integers(1, 5)) if rng.integers(0, 4) else int(rng.integers(2, 65))
+    C = int(8 * rng.integers(1, 17))
+    budget = 4_000_000
+    hi = max(600, budget // (N * C))
+    S = int(rng.integers(max(300, hi // 8), hi))
+    if cf and rng.integers(0, 2):
+        S = S // 8 * 8  # whole vectors per plane
+    dtype = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
+    mis = bool(rng.integers(0, 3) == 0)
+    in_place = bool(rng.integers(0, 4) == 0)
+    print(f"IN exchange random seed={seed} N={N} C={C} spatial={S} dtype={dtype} channel_first={cf} "
+          f"misaligned={mis} in_place={in_place}", flush=True)
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, cf, 500 + seed)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, cf)
+    wrap = util.misalign if mis else (lambda t: t)
+    xd, dyd = wrap(util.to_device(x, dtype)), wrap(util.to_device(dy, dtype))
+    gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
+    x_keep = xd.clone() if in_place else xd
+    y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, cf, y=xd if in_place else None)
+    torch.cuda.synchronize()
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, cf)
+    dx, dg, db = capi.in_bwd(dyd, x_keep, gd, m, r, dtype, cf, dx=dyd if in_place else None)
+    torch.cuda.synchronize()
+    _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
