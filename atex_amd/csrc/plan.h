@@ -126,7 +126,8 @@ struct RowsPlan {
   // Channel-first backward with a workgroup per plane: the fold of the plane sums over the batch
   // runs inside the row kernel (tagged pairs at off_tagged, 16 bytes per plane) instead of as a
   // col_reduce launch.  Needs the planes of a channel on one XCD (C and the grid multiples of the
-  // XCD count), at most 64 instances; the launcher also wants dx != dy and no stream capture.
+  // XCD count), the grid a multiple of C or C of the grid, at most 64 instances; the launcher
+  // also wants dx != dy and no stream capture.
   bool affine_fold = false;
   size_t off_tagged = 0;
 };
@@ -352,8 +353,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.part_rows = static_cast<int>(n_rows / C);
       p.off_part = 0;
       p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
+      // (grid a multiple of C or C of the grid: the workgroup that folds a channel is then the
+      // last-started of those that handle its planes, and waits for none that starts after it)
       p.affine_fold = t.affine_fold && p.tpr == 0 && C % kPlanXcdCount == 0 && p.grid % kPlanXcdCount == 0 &&
-                      p.part_rows >= 2 && p.part_rows <= 64;
+                      (p.grid % C == 0 || C % p.grid == 0) && p.part_rows >= 2 && p.part_rows <= 64;
       if (p.affine_fold) {
         p.off_tagged = p.ws_bytes;
         p.ws_bytes += align256(size_t(16) * size_t(n_rows));

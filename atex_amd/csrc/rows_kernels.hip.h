@@ -650,14 +650,19 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
 
   if constexpr (ROW_AFFINE && TPR == 0) {
     if (fold.tagged != nullptr) {
-      // dgamma / dbeta of the channels whose first plane this workgroup handled
+      // dgamma / dbeta of channel c are folded by workgroup G-1 - (C-1-c) % G: the workgroups
+      // that start last, so that every plane they wait for belongs to a workgroup that has been
+      // started already (a grid larger than the chip holds at once would otherwise leave its
+      // first workgroups waiting in the places that their peers need), and one whose index is
+      // congruent to c modulo the XCD count (C and G are multiples of it), as the indices of
+      // the workgroups that publish the planes of channel c are.
       __shared__ int fold_failed;
       __shared__ float inst[kWave][2];
       const int lane = threadIdx.x & (kWave - 1);
       const int wave = threadIdx.x / kWave;
       const int N = fold.N;
       int it = 0;
-      for (int64_t c = blockIdx.x; c < C && c < n_rows; c += gridDim.x) {
+      for (int64_t c = static_cast<int64_t>(C) - static_cast<int64_t>(gridDim.x) + blockIdx.x; c >= 0; c -= gridDim.x) {
         if (wave == 0) {
           float pb, pa;
           const bool ok = cl_wait_pair(fold.tagged + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2,

@@ -136,6 +136,18 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
         EXPECT(p.off_tagged % 256 == 0 && p.off_tagged >= sizeof(float) * 2 * size_t(n_rows) &&
                    p.ws_bytes >= p.off_tagged + size_t(16) * size_t(n_rows),
                "affine fold: workspace");
+        // channel c is folded by workgroup G-1 - (C-1-c) % G (rows_bwd_resident): on the XCD of
+        // every workgroup that handles a plane of c, and started after all of them
+        const int64_t G = p.grid;
+        bool placed = true;
+        for (int64_t c = 0; c < C && placed; ++c) {
+          const int64_t folder = G - 1 - (C - 1 - c) % G;
+          for (int64_t n = 0; n < p.part_rows; ++n) {
+            const int64_t w = (n * C + c) % G;
+            if (w > folder || w % 8 != folder % 8) placed = false;
+          }
+        }
+        EXPECT(placed, "affine fold: C=%d grid=%d: a folding workgroup waits for a later one or another XCD's", C, p.grid);
       }
     }
   } else {

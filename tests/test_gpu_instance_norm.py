@@ -373,11 +373,12 @@ def test_channels_last_single_launch_in_place_takes_two_stages(capi, coracle):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (8, 32, 4096), (16, 64, 3000), (64, 8, 32768), (2, 16, 5001),
-                                   (24, 40, 2048)])
+                                   (24, 40, 2048), (8, 512, 8192)])
 def test_channel_first_backward_folds_the_batch_in_the_row_kernel(coracle, N, C, S, dtype):
     """Channel-first planes with a workgroup each, C a multiple of 8, at most 64 instances: the
-    backward's row kernel publishes its plane sums as tagged pairs and the workgroups of instance
-    0 add them up over the batch into dgamma / dbeta, instead of a col_reduce launch.  Checked
+    backward's row kernel publishes its plane sums as tagged pairs and the last workgroups of the
+    grid add them up over the batch into dgamma / dbeta, instead of a col_reduce launch
+    ((8, 512, 8192) has more workgroups than the chip holds at once).  Checked
     against the oracle and, through the benchmark build, against itself with the poll limit
     forced to 0 (every folding workgroup recomputes the plane sums of its channel itself: same
     bits), twice on the same workspace, and with the fold switched off (col_reduce again)."""
@@ -430,3 +431,34 @@ def test_channel_first_backward_folds_the_batch_in_the_row_kernel(coracle, N, C,
     finally:
         L.atexn_set_tuning(b"affine_fold_polls", 2000)
         L.atexn_set_tuning(b"affine_fold", 1)
+
+
+def test_channel_first_backward_fold_with_more_workgroups_than_fit():
+    """[8, 256, 32^3] fp16 channel-first: 1024 workgroups of 512 threads with 8 vectors per thread
+    do not fit the chip at once.  The workgroups that fold the batch are the last of the grid, so
+    they wait only for workgroups already started.  Checked against the same call with the fold
+    switched off (col_reduce): dx to the bit, dgamma / dbeta to the summation-order tolerance."""
+    import torch
+
+    capi = util.Capi(bench=True)
+    L = capi.L
+    N, C, S = 8, 256, 32768
+    gen = torch.Generator(device="cuda").manual_seed(97)
+    x = (torch.randn(N, C, S, device="cuda", generator=gen) * 1.5 + 0.25).half()
+    dy = torch.randn(N, C, S, device="cuda", generator=gen).half()
+    gamma = torch.randn(C, device="cuda", generator=gen) * 0.5 + 1.0
+    beta = torch.zeros(C, device="cuda")
+    _, mean, rstd = capi.in_fwd(x, gamma, beta, EPS, "f16", True)
+    try:
+        folded = capi.in_bwd(dy, x, gamma, mean, rstd, "f16", True)
+        torch.cuda.synchronize()
+        assert L.atexn_set_tuning(b"affine_fold", 0) == 0
+        plain = capi.in_bwd(dy, x, gamma, mean, rstd, "f16", True)
+        torch.cuda.synchronize()
+    finally:
+        L.atexn_set_tuning(b"affine_fold", 1)
+    assert torch.equal(_bits(folded[0]), _bits(plain[0])), "dx differs"
+    for name, a, b in (("dgamma", folded[1], plain[1]), ("dbeta", folded[2], plain[2])):
+        err = (a.double() - b.double()).abs().max().item()
+        bound = 1e-5 * b.double().abs().max().item() + 1e-3
+        assert err <= bound, f"{name}: {err} > {bound}"
