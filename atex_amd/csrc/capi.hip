@@ -150,7 +150,7 @@ int atexn_abi_version(void) { return kAbiVersion; }
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "plane_single") || !strcmp(name, "plane_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -212,6 +212,11 @@ int atexn_set_tuning(const char* name, int value) {
     t.affine_fold = value;
   } else if (!strcmp(name, "affine_fold_polls")) {
     t.affine_fold_polls = value;
+  } else if (!strcmp(name, "plane_single")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "plane_single must be 0 or 1");
+    t.plane_single = value;
+  } else if (!strcmp(name, "plane_single_polls")) {
+    t.plane_single_polls = value;
   } else if (!strcmp(name, "cl_single")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_single must be 0 or 1");
     t.cl_single = value;
@@ -263,7 +268,12 @@ int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C
     } else {
       const RowsPlan p = plan_rows(kind, r.V, rows, D, affine ? static_cast<int>(C) : 0, cus);
       const char* k = p.acc_lds ? "rows_bwd_lds" : p.staged ? "rows_bwd_staged" : p.resident ? "rows_bwd_resident" : "";
-      if (k[0] && p.affine_fold)
+      const char* two = p.staged ? "rows_bwd_staged" : "split_bwd_sums + split_bwd_apply";
+      if (p.plane_single)
+        n = snprintf(out, out_bytes, "plane_bwd_single (S=%d chunks of %d vectors, grid %d x %d threads; %s when dx == dy or under capture)%s; alone=0",
+                     p.ps_S, p.ps_chunk_vec, p.ps_grid, kPlanPlaneThreads, two,
+                     p.ps_fold ? ", plane sums folded over the batch in the kernel" : " + col_reduce");
+      else if (k[0] && p.affine_fold)
         n = snprintf(out, out_bytes, "%s (grid %d x %d threads, vpt=%d), plane sums folded over the batch in the kernel (col_reduce follows instead when dx == dy or under capture); alone=0",
                      k, p.grid, p.threads, p.vpt);
       else if (k[0])

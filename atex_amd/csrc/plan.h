@@ -65,6 +65,10 @@ struct Tuning {
   TuneInt cl_single_polls{2000};
   TuneInt affine_fold{1};      // channel-first backward, a workgroup per plane: dgamma / dbeta folded over the batch in the row kernel
   TuneInt affine_fold_polls{2000};  //   polls before a workgroup recomputes its peers' plane sums (0: at once)
+  // channel-first planes too long for a workgroup: the chunks of a plane on the workgroups of one
+  // XCD, statistics exchanged while they run, one pass (plane_single_kernels.hip.h); and its polls
+  TuneInt plane_single{1};
+  TuneInt plane_single_polls{2000};
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,
   // smaller-register threads) before switching to 4; forward <= 2048, backward <= 1536.
@@ -130,7 +134,23 @@ struct RowsPlan {
   // also wants dx != dy and no stream capture.
   bool affine_fold = false;
   size_t off_tagged = 0;
+  // Channel-first planes beyond the resident and staged kernels, one launch and one pass
+  // (plane_single_kernels.hip.h): ps_S chunks of ps_chunk_vec vectors per plane, each on a
+  // 512-thread workgroup with at most 8 vectors per thread; workgroup b of the ps_grid takes chunk
+  // (b / 8) % ps_S of plane ((b / 8) / ps_S) * 8 + b % 8.  Needs whole vectors (D % V == 0) and no
+  // more chunks than an XCD holds such workgroups (two per CU).  The split kernels stay the
+  // fallback (y == x, stream capture) in the same workspace; tagged pairs at off_ps_tagged.
+  bool plane_single = false;
+  int ps_S = 0, ps_chunk_vec = 0, ps_grid = 0;
+  bool ps_full = false;  // every thread of every workgroup holds 8 vectors
+  size_t off_ps_tagged = 0;
+  // backward: the planes' sums folded over the batch inside the kernel (tagged pairs per plane at
+  // off_ps_fold) instead of by a col_reduce launch: the planes of a channel must share an XCD (C a
+  // multiple of the XCD count, or a single instance), at most 64 instances
+  bool ps_fold = false;
+  size_t off_ps_fold = 0;
 };
+constexpr int kPlanPlaneThreads = 512, kPlanPlaneVpt = 8, kPlanPlaneMaxChunks = 64;
 
 // Longest row, in vectors, that the register-resident kernels take: forward 8 vectors per
 // thread at 512 threads, backward 4 (it holds x and dy, and LayerNorm also gamma and the
@@ -217,6 +237,35 @@ inline SmallPlan plan_small(RowsKind kind, int V, int64_t n_rows, int64_t D, int
   return p;
 }
 
+// Adds the one-launch plan for channel-first planes (RowsPlan::plane_single) to a plan whose other
+// workspace sections end at `bytes`, when the shape qualifies.
+inline void plan_plane_single(RowsPlan& p, RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus,
+                              size_t& bytes) {
+  const Tuning& t = tuning();
+  const int64_t n_vec = div_up(D, V);
+  if (t.plane_single && C > 0 && V > 1 && D % V == 0 && kind != RowsKind::kBwdCols) {
+    const int64_t per_wg = int64_t(kPlanPlaneThreads) * kPlanPlaneVpt;
+    const int64_t S2 = div_up(n_vec, per_wg);
+    const int64_t slots = int64_t(cus / kPlanXcdCount) * 2;
+    const int64_t grid = round_up(n_rows, kPlanXcdCount) * S2;
+    if (S2 >= 2 && S2 <= std::min<int64_t>(kPlanPlaneMaxChunks, slots) && grid < (int64_t(1) << 31)) {
+      p.plane_single = true;
+      p.ps_S = static_cast<int>(S2);
+      p.ps_chunk_vec = static_cast<int>(div_up(n_vec, S2));
+      p.ps_grid = static_cast<int>(grid);
+      p.ps_full = n_vec % S2 == 0 && p.ps_chunk_vec == per_wg;
+      p.off_ps_tagged = bytes;
+      bytes += align256(size_t(16) * size_t(n_rows) * size_t(S2));
+      if (kind == RowsKind::kBwdAffine && t.affine_fold && p.part_rows <= 64 &&
+          (C % kPlanXcdCount == 0 || p.part_rows == 1)) {
+        p.ps_fold = true;
+        p.off_ps_fold = bytes;
+        bytes += align256(size_t(16) * size_t(n_rows));
+      }
+    }
+  }
+}
+
 // V: vector width in elements (see route_rows).  C: the channel count of a channel-first input
 // (row r takes gamma[r % C]), 0 for LayerNorm.
 inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C, int cus) {
@@ -255,6 +304,10 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       p.off_part = 0;
       p.ws_bytes = align256(sizeof(float) * 2 * size_t(n_rows));
     }
+    // (the one-launch kernels over the workgroups of an XCD, where they apply, are faster:
+    // [16, 64, 256, 256] fp16 44.7 / 86.1 us staged, 41.9 / 74.8 us so; the staged kernels then
+    // serve y == x, stream capture and ragged planes)
+    plan_plane_single(p, kind, V, n_rows, D, C, cus, p.ws_bytes);
     return p;
   }
   if (p.resident) {
@@ -381,6 +434,7 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
     p.off_part = bytes;
     bytes += align256(sizeof(float) * 2 * size_t(n_rows));
   }
+  plan_plane_single(p, kind, V, n_rows, D, C, cus, bytes);
   p.ws_bytes = bytes;
   return p;
 }

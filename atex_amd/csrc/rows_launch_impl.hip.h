@@ -4,6 +4,7 @@
 
 #include "plan.h"
 #include "rows_kernels.hip.h"
+#include "plane_single_kernels.hip.h"
 #include "small_kernels.hip.h"
 #include "tiles_kernels.hip.h"
 
@@ -162,6 +163,19 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
                                      eps);
     ATEXN_CHECK_LAUNCH("rows_fwd_resident");
     return ATEXN_OK;
+  }
+  if constexpr (AFF && V > 1) {
+    if (p.plane_single && static_cast<const void*>(y) != static_cast<const void*>(x) && !rows_stream_is_capturing(st)) {
+      static_assert(kPlaneThreads == kPlanPlaneThreads && kPlaneMaxChunks == kPlanPlaneMaxChunks && kPlaneXcds == kPlanXcdCount,
+                    "plan_rows sizes the plane_*_single launches");
+      cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
+      const int n_vec = static_cast<int>(D / V);
+      auto fn = p.ps_full ? plane_fwd_single<T, V, kPlanPlaneVpt, true> : plane_fwd_single<T, V, kPlanPlaneVpt, false>;
+      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(x, tagged, gamma, beta, y, mean, rstd, n_rows, n_vec, p.ps_S,
+                                              p.ps_chunk_vec, C, eps, next_call_tag(), tuning().plane_single_polls);
+      ATEXN_CHECK_LAUNCH("plane_fwd_single");
+      return ATEXN_OK;
+    }
   }
   if constexpr (AFF && V > 1) {
     if (p.staged) {
@@ -344,6 +358,20 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     }
     if (!(stages & 2)) return ATEXN_OK;
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+  }
+  if constexpr (AFF && V > 1) {
+    if (p.plane_single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && !rows_stream_is_capturing(st)) {
+      cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
+      const int n_vec = static_cast<int>(D / V);
+      auto fn = p.ps_full ? plane_bwd_single<T, V, kPlanPlaneVpt, true> : plane_bwd_single<T, V, kPlanPlaneVpt, false>;
+      PlaneFold pf{nullptr, dgamma, dbeta, p.part_rows};
+      if (p.ps_fold) pf.tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_fold);
+      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, dx, part, n_rows, n_vec, p.ps_S,
+                                              p.ps_chunk_vec, C, next_call_tag(), tuning().plane_single_polls, pf);
+      ATEXN_CHECK_LAUNCH("plane_bwd_single");
+      if (p.ps_fold) return ATEXN_OK;
+      return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
+    }
   }
   if constexpr (AFF && V > 1) {
     if (p.staged) {

@@ -70,6 +70,34 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
   }
   const RowsPlan p = plan_rows(kind, r.V, n_rows, D, layer_norm ? 0 : C, cus);
   EXPECT(p.ragged == (D % r.V != 0), "ragged");
+  // the one-launch plan for channel-first planes, where a plan carries one (`before`: bytes of the
+  // workspace sections that precede its tagged pairs)
+  auto check_plane_single = [&](size_t before) {
+  if (p.plane_single) {
+    // what plane_fwd_single / plane_bwd_single assume: whole vectors, chunks of at most 8
+    // vectors per thread of 512, no more chunks than lanes in a wave or than an XCD holds such
+    // workgroups, a grid of whole planes per XCD, the tagged pairs behind the other sections
+    const int64_t n_vec = D / r.V;
+    EXPECT(D % r.V == 0 && r.V > 1 && C > 0, "plane single: D=%lld V=%d", (long long)D, r.V);
+    EXPECT(p.ps_S >= 2 && p.ps_S <= 64 && p.ps_S <= cus / 8 * 2, "plane single: S=%d cus=%d", p.ps_S, cus);
+    EXPECT(p.ps_chunk_vec >= 1 && p.ps_chunk_vec <= 512 * 8, "plane single: chunk of %d vectors", p.ps_chunk_vec);
+    EXPECT(int64_t(p.ps_S - 1) * p.ps_chunk_vec < n_vec && n_vec <= int64_t(p.ps_S) * p.ps_chunk_vec,
+           "plane single: S=%d chunk=%d n_vec=%lld", p.ps_S, p.ps_chunk_vec, (long long)n_vec);
+    EXPECT(p.ps_full == (n_vec == int64_t(p.ps_S) * 4096), "plane single: full=%d", int(p.ps_full));
+    EXPECT(int64_t(p.ps_grid) == (n_rows + 7) / 8 * 8 * p.ps_S, "plane single: grid=%d", p.ps_grid);
+    EXPECT(p.off_ps_tagged % 256 == 0 && p.off_ps_tagged >= before &&
+               p.ws_bytes >= p.off_ps_tagged + size_t(16) * size_t(n_rows) * size_t(p.ps_S),
+           "plane single: workspace");
+    if (kind == RowsKind::kBwdAffine) EXPECT(p.off_ps_tagged >= p.off_part + sizeof(float) * 2 * size_t(n_rows), "plane single: tagged pairs over the plane sums");
+    if (p.ps_fold) {
+      EXPECT(kind == RowsKind::kBwdAffine && p.part_rows >= 1 && p.part_rows <= 64 && (C % 8 == 0 || p.part_rows == 1),
+             "plane fold: N=%d C=%d", p.part_rows, C);
+      EXPECT(p.off_ps_fold % 256 == 0 && p.off_ps_fold >= p.off_ps_tagged + size_t(16) * size_t(n_rows) * size_t(p.ps_S) &&
+                 p.ws_bytes >= p.off_ps_fold + size_t(16) * size_t(n_rows),
+             "plane fold: workspace");
+    }
+  }
+  };
   if (p.staged) {
     // the row staged in registers (8 vectors per thread) and LDS, 512 threads
     EXPECT(!p.resident && r.V > 1 && kind != RowsKind::kBwdCols && n_vec > resident_limit(kind), "staged with n_vec=%lld", (long long)n_vec);
@@ -77,6 +105,7 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
     EXPECT(p.fold_lds == size_t(p.nv_lds) * 512 * (kind == RowsKind::kFwd ? 16 : 32) && p.fold_lds + 512 <= 160 * 1024, "staged LDS bytes %zu", p.fold_lds);
     EXPECT(p.grid >= 1 && p.grid <= n_rows && int64_t(p.grid) * int64_t(p.fold_lds + 512) <= int64_t(cus) * 160 * 1024, "staged grid=%d", p.grid);
     if (kind == RowsKind::kBwdAffine) EXPECT(p.part_rows == n_rows / C && p.ws_bytes >= sizeof(float) * 2 * size_t(n_rows), "staged partial rows");
+    check_plane_single(kind == RowsKind::kBwdAffine ? sizeof(float) * 2 * size_t(n_rows) : 0);
     return;
   }
   if (p.resident) {
@@ -157,6 +186,7 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
     EXPECT(p.chunk % (256 * r.V) == 0, "chunk granularity");
     EXPECT(p.split_grid >= 1 && int64_t(p.split_grid) <= n_rows * p.S, "split_grid");
     EXPECT(p.ws_bytes >= sizeof(float) * 2 * size_t(n_rows) * size_t(p.S), "pairs workspace");
+    check_plane_single(sizeof(float) * 2 * size_t(n_rows) * size_t(p.S));
     if (kind == RowsKind::kBwdAffine) EXPECT(p.ws_bytes >= p.off_part + sizeof(float) * 2 * size_t(n_rows), "part workspace");
   }
 }

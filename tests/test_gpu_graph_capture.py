@@ -17,7 +17,22 @@ EPS = 1e-3
 def test_graph_replay_matches_eager(case):
     import torch
 
-    capi = util.Capi()
+    # (the staged case through the benchmark build with the kernels that would take these planes
+    # in eager mode, but not under capture, switched off: eager and replay then run the same ones)
+    staged = case == "in_channel_first_staged"
+    capi = util.Capi(bench=staged)
+    if staged:
+        assert capi.L.atexn_set_tuning(b"plane_single", 0) == 0
+    try:
+        _replay_matches_eager(capi, case)
+    finally:
+        if staged:
+            assert capi.L.atexn_set_tuning(b"plane_single", 1) == 0
+
+
+def _replay_matches_eager(capi, case):
+    import torch
+
     dtype = "f16"
     if case.startswith("ln"):
         N, D = {"ln_resident": (512, 1024), "ln_tiles": (6, 70001), "ln_small": (5000, 10),
@@ -68,9 +83,11 @@ def test_graph_replay_matches_eager(case):
             assert torch.equal(got, ref), f"replay {replay}: {name} differs from the eager result"
 
 
-def test_graph_capture_of_a_single_launch_shape(coracle):
-    """Channels-last shapes that run as one launch per direction in eager mode (the workgroups
-    exchange partials tagged with a per-call number) are recorded as the two-stage kernels when
+@pytest.mark.parametrize("N,C,S,cf", [(8, 64, 4096, False), (2, 4, 262144, True)])
+def test_graph_capture_of_a_single_launch_shape(coracle, N, C, S, cf):
+    """Shapes that run as one launch per direction in eager mode, with workgroups that exchange
+    partials tagged with a per-call number (channels-last instances over the workgroups of an XCD;
+    channel-first planes too long for one workgroup), are recorded as the two-stage kernels when
     the stream is being captured, since a replay would repeat the tag.  The replays must agree
     with each other bit for bit and with the oracle; against the eager (single-launch) result only
     the last bits of the statistics may differ (another order of the same additions)."""
@@ -79,29 +96,29 @@ def test_graph_capture_of_a_single_launch_shape(coracle):
     from tests.util import TOL, assert_close
 
     capi = util.Capi()
-    dtype, N, C, S = "f16", 8, 64, 4096
-    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, False, 33)
-    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, False)
-    print(f"graph capture of IN channels-last N={N} C={C} spatial={S} {dtype}", flush=True)
+    dtype = "f16"
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, cf, 33)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, cf)
+    print(f"graph capture of IN channel_first={cf} N={N} C={C} spatial={S} {dtype}", flush=True)
     xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
     gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
-    y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
-    dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
+    y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, cf)
+    dx, dg, db = capi.in_bwd(dyd, xd, gd, m, r, dtype, cf)
     torch.cuda.synchronize()
     eager = [t.clone() for t in (y, m, r, dx, dg, db)]
-    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, False)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, util.to_host(m), util.to_host(r), dtype, cf)
 
     graph = torch.cuda.CUDAGraph()
     s = torch.cuda.Stream()
     s.wait_stream(torch.cuda.current_stream())
     with torch.cuda.stream(s):
-        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
-        capi.in_bwd(dyd, xd, gd, m, r, dtype, False)
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, cf)
+        capi.in_bwd(dyd, xd, gd, m, r, dtype, cf)
     torch.cuda.current_stream().wait_stream(s)
     torch.cuda.synchronize()
     with torch.cuda.graph(graph):
-        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, False)
-        dx, dg, db = capi.in_bwd(dyd, xd, gd, eager[1], eager[2], dtype, False)
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, cf)
+        dx, dg, db = capi.in_bwd(dyd, xd, gd, eager[1], eager[2], dtype, cf)
     outs = (y, m, r, dx, dg, db)
     first = None
     tol = TOL[dtype]

@@ -256,14 +256,18 @@ def test_channel_first_planes_staged_on_chip(coracle, N, C, S, dtype, in_place):
     LDS make a single pass (forward up to 27 vectors per thread of 512, backward, which stages x
     and dy, up to 17): the limits of both directions for 16-bit and float32 planes, one
     element past them (two-stage kernels again), ragged planes, in place, and more planes than
-    workgroups.  (The planner stages rows only when there are enough of them to fill the chip;
-    the benchmark build's tuning hook lifts that condition here.)"""
+    workgroups.  (The planner stages rows only when there are enough of them to fill the chip, and
+    prefers the kernels that spread a plane over the workgroups of an XCD to these unless the call
+    is in place or being captured; the benchmark build's tuning hook lifts the first condition
+    and switches the other kernels off here.)"""
     capi = util.Capi(bench=True)
     assert capi.L.atexn_set_tuning(b"staged_rows", 2) == 0
+    assert capi.L.atexn_set_tuning(b"plane_single", 0) == 0
     try:
         run_case(capi, coracle, N, C, S, dtype, True, 37, in_place=in_place)
     finally:
         assert capi.L.atexn_set_tuning(b"staged_rows", 1) == 0
+        assert capi.L.atexn_set_tuning(b"plane_single", 1) == 0
 
 
 @pytest.mark.parametrize("dtype", ["f16", "f32"])
@@ -462,3 +466,76 @@ def test_channel_first_backward_fold_with_more_workgroups_than_fit():
         err = (a.double() - b.double()).abs().max().item()
         bound = 1e-5 * b.double().abs().max().item() + 1e-3
         assert err <= bound, f"{name}: {err} > {bound}"
+
+
+@pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
+@pytest.mark.parametrize("N,C,S", [(2, 8, 40000), (1, 3, 100000), (2, 4, 262144), (3, 5, 65544), (1, 16, 2097152),
+                                   (2, 9, 32776), (1, 1, 1048576)])
+def test_channel_first_planes_across_workgroups(coracle, N, C, S, dtype):
+    """Channel-first planes too long for one workgroup (and too few, or too long, for the kernels
+    that stage a plane in LDS): the chunks of a plane go to consecutive workgroups of one XCD, which
+    keep them in registers and exchange their statistics while they run, so x (and dy) is read
+    once.  Checked against the oracle, and through the benchmark build against itself with the
+    poll limit forced to 0 (every workgroup recomputes the statistics of its plane's other chunks
+    itself: same bits), twice on the same workspace, and with the path switched off (the two-stage
+    kernels).  (1, 3, ...) and (2, 9, ...) leave XCDs with fewer planes than others."""
+    import ctypes
+
+    import torch
+
+    capi = util.Capi(bench=True)
+    L = capi.L
+    buf = ctypes.create_string_buffer(384)
+    L.atexn_bench_describe_bwd(1, O.DTYPE_CODE[dtype], 0, N, C, S, buf, 384)
+    print(f"IN channel-first N={N} C={C} spatial={S} {dtype}: {buf.value.decode()}", flush=True)
+    if b"plane_bwd_single" not in buf.value:
+        pytest.skip("this shape and dtype take other kernels")
+    x, gamma, beta, dy = util.in_inputs(N, C, S, dtype, True, 95)
+    y_ref, m_ref, r_ref = coracle.in_fwd(x, gamma, beta, EPS, dtype, True)
+    dx_ref, dg_ref, db_ref = coracle.in_bwd(dy, x, gamma, m_ref.astype(np.float32), r_ref.astype(np.float32),
+                                            dtype, True)
+    xd, dyd = util.to_device(x, dtype), util.to_device(dy, dtype)
+    gd, bd = torch.from_numpy(gamma).cuda(), torch.from_numpy(beta).cuda()
+    md = torch.from_numpy(m_ref.astype(np.float32)).cuda()
+    rd = torch.from_numpy(r_ref.astype(np.float32)).cuda()
+    tol = TOL[dtype]
+
+    def run():
+        y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, True)
+        dx, dg, db = capi.in_bwd(dyd, xd, gd, md, rd, dtype, True)
+        torch.cuda.synchronize()
+        return y, m, r, dx, dg, db
+
+    def check(out, what):
+        y, m, r, dx, dg, db = out
+        assert_close(util.to_host(m), m_ref, tol["stat"], what + " mean")
+        assert_close(util.to_host(r), r_ref, tol["stat"], what + " inv_std")
+        assert_close(util.to_host(y), y_ref, tol["y"], what + " y")
+        scale = util.dx_scale(dy, np.sqrt(np.mean(gamma.astype(np.float64) ** 2)), r_ref, dtype)
+        assert_close(util.to_host(dx), dx_ref, tol["dx"], what + " dx", scale=scale)
+        assert_close(util.to_host(dg), dg_ref, tol["dw"], what + " dgamma")
+        assert_close(util.to_host(db), db_ref, tol["dw"], what + " dbeta")
+
+    names = ("y", "mean", "inv_std", "dx", "dgamma", "dbeta")
+    try:
+        normal = run()
+        check(normal, "one launch")
+        again = run()
+        for n_, a, b in zip(names, normal, again):
+            assert torch.equal(_bits(a), _bits(b)), f"second run differs in {n_}"
+        assert L.atexn_set_tuning(b"plane_single_polls", 0) == 0
+        alone = run()
+        for n_, a, b in zip(names, normal, alone):
+            assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
+        assert L.atexn_set_tuning(b"plane_single_polls", 2000) == 0
+        assert L.atexn_set_tuning(b"plane_single", 0) == 0
+        check(run(), "two stages")
+    finally:
+        L.atexn_set_tuning(b"plane_single_polls", 2000)
+        L.atexn_set_tuning(b"plane_single", 1)
+
+
+def test_channel_first_planes_across_workgroups_in_place(capi, coracle):
+    """y written over x (dx over dy) keeps such a call on the two-stage kernels (the one-launch
+    kernels' fallback reads other workgroups' chunks of x): results as good as out of place."""
+    run_case(capi, coracle, 2, 4, 262144, "f16", True, 96, in_place=True)

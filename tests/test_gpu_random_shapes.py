@@ -149,6 +149,7 @@ def test_rows_kept_in_lds_random(coracle, seed):
         gd, bd = wrap(torch.from_numpy(gamma).cuda()), wrap(torch.from_numpy(beta).cuda())
         x_keep = xd.clone() if in_place else xd
         assert capi.L.atexn_set_tuning(b"staged_rows", 2) == 0
+        assert capi.L.atexn_set_tuning(b"plane_single", 0) == 0  # (they would take what is not in place)
         try:
             y, m, r = capi.in_fwd(xd, gd, bd, EPS, dtype, True, y=xd if in_place else None)
             torch.cuda.synchronize()
@@ -157,28 +158,40 @@ def test_rows_kept_in_lds_random(coracle, seed):
             torch.cuda.synchronize()
         finally:
             assert capi.L.atexn_set_tuning(b"staged_rows", 1) == 0
+            assert capi.L.atexn_set_tuning(b"plane_single", 1) == 0
     _check((y, m, r, dx, dg, db), (y_ref, m_ref, r_ref, dx_ref, dg_ref, db_ref), dy, gamma, util.to_host(r), dtype)
 
 
 @pytest.mark.parametrize("seed", range(max(1, N_SEEDS // 2)))
 def test_exchange_paths_random(coracle, seed):
     """Shapes drawn for the kernels whose workgroups hand each other partial results while they
-    run: channels-last with batches that are multiples of 8 (one launch per direction) and
+    run: channels-last with batches that are multiples of 8 (one launch per direction),
     channel-first planes with C a multiple of 8 (plane sums folded over the batch in the row
-    kernel), at random sizes around their limits, misaligned tensors and in-place calls (which
-    must take the other kernels) included.  Against the oracle."""
+    kernel) and channel-first planes too long for a workgroup (a plane's chunks on consecutive
+    workgroups of an XCD), at random sizes around their limits, misaligned tensors and in-place
+    calls (which must take the other kernels) included.  Against the oracle."""
     import torch
 
     capi = util.Capi()
     rng = np.random.Generator(np.random.PCG64(11000 + seed))
-    cf = bool(seed % 2)
-    N = int(8 * rng.integers(1, 5)) if rng.integers(0, 4) else int(rng.integers(2, 65))
-    C = int(8 * rng.integers(1, 17))
-    budget = 4_000_000
-    hi = max(600, budget // (N * C))
-    S = int(rng.integers(max(300, hi // 8), hi))
-    if cf and rng.integers(0, 2):
-        S = S // 8 * 8  # whole vectors per plane
+    family = seed % 3
+    cf = family != 0
+    if family == 2:
+        N = int(rng.integers(1, 4))
+        C = int(rng.choice([1, 2, 3, 5, 8, 16]))
+        S = int(rng.integers(32769, max(32770, 3_000_000 // (N * C))))
+        if rng.integers(0, 4):
+            S = S // 8 * 8  # whole vectors per plane: otherwise the two-stage kernels
+        if rng.integers(0, 4) == 0:
+            S = int(rng.integers(1, 9)) * 32768  # every workgroup's registers full
+    else:
+        N = int(8 * rng.integers(1, 5)) if rng.integers(0, 4) else int(rng.integers(2, 65))
+        C = int(8 * rng.integers(1, 17))
+        budget = 4_000_000
+        hi = max(600, budget // (N * C))
+        S = int(rng.integers(max(300, hi // 8), hi))
+        if cf and rng.integers(0, 2):
+            S = S // 8 * 8  # whole vectors per plane
     dtype = ["f32", "f16", "bf16"][int(rng.integers(0, 3))]
     mis = bool(rng.integers(0, 3) == 0)
     in_place = bool(rng.integers(0, 4) == 0)

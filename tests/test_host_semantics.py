@@ -252,16 +252,21 @@ def test_every_planning_parameter_is_settable_in_the_benchmark_build():
     for name, default in names:
         rc = L.atexn_set_tuning(name.encode(), int(default))
         assert rc == 0, (name, default, L.atexn_last_error())
-    # a plan follows its parameter: planes staged on chip need no statistics workspace
+    # a plan follows its parameter: planes staged on chip need no workspace, planes spread over
+    # the workgroups of an XCD need 16 bytes per chunk, the two-stage kernels 8
     rows = (1, 0, 16, 64, 65536)  # dtype f16, channel-first, N, C, D
-    assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
-    assert L.atexn_set_tuning(b"staged_rows", 0) == 0
+    default = L.atexn_instance_norm_fwd_workspace_bytes(*rows)
+    assert default == 16 * 16 * 64 * 2 == _capi.lib().atexn_instance_norm_fwd_workspace_bytes(*rows)
+    assert L.atexn_set_tuning(b"plane_single", 0) == 0
     try:
+        assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
+        assert L.atexn_set_tuning(b"staged_rows", 0) == 0
         assert L.atexn_instance_norm_fwd_workspace_bytes(*rows) > 0
         # ... and the product library, loaded beside it, is not affected
-        assert _capi.lib().atexn_instance_norm_fwd_workspace_bytes(*rows) == 0
+        assert _capi.lib().atexn_instance_norm_fwd_workspace_bytes(*rows) == default
     finally:
         assert L.atexn_set_tuning(b"staged_rows", 1) == 0
+        assert L.atexn_set_tuning(b"plane_single", 1) == 0
     buf = ctypes.create_string_buffer(256)
     assert L.atexn_bench_describe_bwd(0, 1, 0, 8192, 0, 1024, buf, 256) > 0
     assert b"rows_bwd_resident" in buf.value and b"alone=1" in buf.value
@@ -269,6 +274,8 @@ def test_every_planning_parameter_is_settable_in_the_benchmark_build():
     assert b"cl_bwd_single" in buf.value and b"alone=0" in buf.value
     assert L.atexn_bench_describe_bwd(1, 1, 1, 2, 32, 2097152, buf, 256) > 0
     assert b"cl_bwd_sums" in buf.value and b"alone=0" in buf.value
+    assert L.atexn_bench_describe_bwd(1, 1, 0, 2, 32, 2097152, buf, 256) > 0
+    assert b"plane_bwd_single (S=64" in buf.value and b"folded over the batch" in buf.value
 
 
 def test_workspace_queries_without_gpu(L):
