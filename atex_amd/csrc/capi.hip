@@ -217,6 +217,8 @@ int atexn_set_tuning(const char* name, int value) {
     t.plane_single = value;
   } else if (!strcmp(name, "plane_single_polls")) {
     t.plane_single_polls = value;
+  } else if (!strcmp(name, "plane_nt_min_mb")) {
+    t.plane_nt_min_mb = value;
   } else if (!strcmp(name, "cl_single")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_single must be 0 or 1");
     t.cl_single = value;

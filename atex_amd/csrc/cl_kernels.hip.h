@@ -1058,8 +1058,8 @@ cl_bwd_fused(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
   const ClGeom g = cl_geom<RG>(tpp_shift, CV, C, V, D, D);
   Pack<T, V> rx[U], rd[U];
   bool ok[U];
-  cl_load_slab<T, V, U>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-  cl_load_slab<T, V, U>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+  cl_load_slab<T, V, U, true>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+  cl_load_slab<T, V, U, true>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   float mu[V], rs[V], sc[V];
   load_f32<V>(mean_in + g.n * C + g.coff, mu);
   load_f32<V>(rstd_in + g.n * C + g.coff, rs);

@@ -226,8 +226,8 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   if (threadIdx.x == 0) sm_fail = sm_fail_dev = 0;
   Pack<T, V> rx[U], rd[U];
   bool ok[U];
-  cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-  cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+  cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+  cl_load_slab<T, V, U, true, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
   float mu[V], rs[V];
 #pragma unroll
   for (int i = 0; i < V; ++i) mu[i] = rs[i] = 0.f;
@@ -302,8 +302,8 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     }
     for (int l = 0; l < S; ++l) {
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
-      cl_load_slab<T, V, U, false, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
-      cl_load_slab<T, V, U, false, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
+      cl_load_slab<T, V, U, true, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
+      cl_load_slab<T, V, U, true, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
       float a2[2 * V];
       __syncthreads();  // the previous round's block sums have been read
       cl_resident_sums<T, V, U>(rx, rd, ok, mu2, rs2, TPP, lds, a2);
@@ -332,8 +332,8 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
         }
       }
     }
-    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-    cl_load_slab<T, V, U, false, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+    cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
+    cl_load_slab<T, V, U, true, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
     __syncthreads();
   }
   // The owners of instance 0 also fold the instances' sums into dgamma / dbeta (below, after

@@ -492,8 +492,8 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       if constexpr (ROW_AFFINE) t.gm[r] = gamma[static_cast<int>(row % C)];
 #pragma unroll
       for (int k = 0; k < VPT; ++k) {
-        t.px[r][k] = load_pack<T, V>(xr + col[k]);
-        t.pd[r][k] = load_pack<T, V>(dyr + col[k]);
+        t.px[r][k] = load_pack_last<T, V>(xr + col[k]);
+        t.pd[r][k] = load_pack_last<T, V>(dyr + col[k]);
       }
     }
   };
@@ -909,8 +909,8 @@ rows_bwd_lds(const T* dy, const T* __restrict__ x, const float* __restrict__ gam
     const T* dyr = dy + row * D;
 #pragma unroll
     for (int k = 0; k < VPT; ++k) {
-      qx[k] = load_pack<T, V>(xr + col[k]);
-      qd[k] = load_pack<T, V>(dyr + col[k]);
+      qx[k] = load_pack_last<T, V>(xr + col[k]);
+      qd[k] = load_pack_last<T, V>(dyr + col[k]);
     }
   };
   Pack<T, V> px[VPT], pd[VPT];
@@ -1231,8 +1231,8 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
     Pack<T, V> rx[R], rd[R];
 #pragma unroll
     for (int j = 0; j < R; ++j) {
-      rx[j] = load_pack<T, V>(xr + rs[j].col);
-      rd[j] = load_pack<T, V>(dyr + rs[j].col);
+      rx[j] = load_pack_last<T, V>(xr + rs[j].col);
+      rd[j] = load_pack_last<T, V>(dyr + rs[j].col);
     }
     float a1 = 0.f, a2 = 0.f;
     auto add = [&](const Pack<T, V>& px, const Pack<T, V>& pd, const StagedSlot<V>& sl) {
@@ -1250,8 +1250,8 @@ rows_bwd_staged(const T* dy, const T* __restrict__ x, const float* __restrict__ 
 #pragma unroll
       for (int u = 0; u < B; ++u) {
         sl[u] = lds_slot(j0 + u < nv_lds ? j0 + u : nv_lds - 1);
-        px[u] = load_pack<T, V>(xr + sl[u].col);
-        pd[u] = load_pack<T, V>(dyr + sl[u].col);
+        px[u] = load_pack_last<T, V>(xr + sl[u].col);
+        pd[u] = load_pack_last<T, V>(dyr + sl[u].col);
       }
       batch_loaded<T, V, B>(px, pd);
 #pragma unroll

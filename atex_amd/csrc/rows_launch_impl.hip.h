@@ -170,7 +170,9 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
                     "plan_rows sizes the plane_*_single launches");
       cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
       const int n_vec = static_cast<int>(D / V);
-      auto fn = p.ps_full ? plane_fwd_single<T, V, kPlanPlaneVpt, true> : plane_fwd_single<T, V, kPlanPlaneVpt, false>;
+      const bool nt = n_rows * D * int64_t(sizeof(T)) >= int64_t(tuning().plane_nt_min_mb) << 20;
+      auto fn = p.ps_full ? (nt ? plane_fwd_single<T, V, kPlanPlaneVpt, true, true> : plane_fwd_single<T, V, kPlanPlaneVpt, true, false>)
+                          : (nt ? plane_fwd_single<T, V, kPlanPlaneVpt, false, true> : plane_fwd_single<T, V, kPlanPlaneVpt, false, false>);
       fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(x, tagged, gamma, beta, y, mean, rstd, n_rows, n_vec, p.ps_S,
                                               p.ps_chunk_vec, C, eps, next_call_tag(), tuning().plane_single_polls);
       ATEXN_CHECK_LAUNCH("plane_fwd_single");

@@ -130,8 +130,8 @@ small_bwd(const T* dy, const T* __restrict__ x, const float* __restrict__ gamma,
     Pack<T, V> px[NV], pd[NV];
 #pragma unroll
     for (int j = 0; j < NV; ++j) {
-      px[j] = load_pack<T, V>(xr + g.off[j]);
-      pd[j] = load_pack<T, V>(dr + g.off[j]);
+      px[j] = load_pack_last<T, V>(xr + g.off[j]);
+      pd[j] = load_pack_last<T, V>(dr + g.off[j]);
     }
     const float mean = mean_in[row], rstd = rstd_in[row];
     float gs = 1.f;
