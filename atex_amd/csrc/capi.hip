@@ -150,7 +150,7 @@ int atexn_abi_version(void) { return kAbiVersion; }
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "plane_single") || !strcmp(name, "plane_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "cl_single_xm") || !strcmp(name, "plane_single") || !strcmp(name, "plane_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -222,6 +222,9 @@ int atexn_set_tuning(const char* name, int value) {
   } else if (!strcmp(name, "cl_single")) {
     ATEXN_REQUIRE(value == 0 || value == 1, "cl_single must be 0 or 1");
     t.cl_single = value;
+  } else if (!strcmp(name, "cl_single_xm")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "cl_single_xm must be 0 or 1");
+    t.cl_single_xm = value;
   } else if (!strcmp(name, "cl_single_polls")) {
     t.cl_single_polls = value;
   } else if (!strcmp(name, "cl_fold_cap")) {
@@ -251,8 +254,8 @@ int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C
       n = snprintf(out, out_bytes, "cl_bwd_fused (u=%d, grid %lld x %d)%s; alone=0", p.fused_u, (long long)N,
                    p.CT, N > 1 ? " + col_reduce" : "");
     else if (p.single)
-      n = snprintf(out, out_bytes, "cl_bwd_single (S=%d slabs, tiles=%d, U=%d; two stages when dx == dy or under capture); alone=0",
-                   p.S, p.CT, p.U);
+      n = snprintf(out, out_bytes, "cl_bwd_single (S=%d slabs, tiles=%d, U=%d%s; two stages when dx == dy or under capture)%s; alone=0",
+                   p.S, p.CT, p.U, p.single_xm ? ", XCD-major grid" : "", p.single_xm && !p.xm_fold && N > 1 ? " + col_reduce" : "");
     else
       n = snprintf(out, out_bytes, "cl_bwd_sums + %scl_bwd_apply (S=%d slabs, tiles=%d, U=%d); alone=0",
                    p.fold ? "col_reduce + " : "", p.S, p.CT, p.U);

@@ -53,13 +53,14 @@ struct ClGeom {
   int slab_n;      // p1 - p0 (resident slabs only: they have at most 16 * 256 pixels)
 };
 
+// Geometry of the thread for instance n, slab s, channel tile ct.
 template <bool RG>
-__device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, int64_t D,
-                                          int64_t slab_len) {
+__device__ __forceinline__ ClGeom cl_geom_at(int64_t n, int s, int ct, int tpp_shift, int CV, int C, int V,
+                                             int64_t D, int64_t slab_len) {
   ClGeom g;
-  g.n = blockIdx.x;
-  g.s = static_cast<int>(blockIdx.y);
-  g.ct = static_cast<int>(blockIdx.z);
+  g.n = n;
+  g.s = s;
+  g.ct = ct;
   const int t = static_cast<int>(threadIdx.x);
   g.cvi = (g.ct << tpp_shift) | (t & ((1 << tpp_shift) - 1));
   g.slot = t >> tpp_shift;
@@ -79,6 +80,13 @@ __device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, i
   g.p1 = g.p0 + slab_len < D ? g.p0 + slab_len : D;
   g.slab_n = static_cast<int>(g.p1 - g.p0 < (1 << 20) ? g.p1 - g.p0 : (1 << 20));
   return g;
+}
+// The same for a launch whose grid is (N, S, channel tiles).
+template <bool RG>
+__device__ __forceinline__ ClGeom cl_geom(int tpp_shift, int CV, int C, int V, int64_t D,
+                                          int64_t slab_len) {
+  return cl_geom_at<RG>(blockIdx.x, static_cast<int>(blockIdx.y), static_cast<int>(blockIdx.z), tpp_shift, CV, C,
+                        V, D, slab_len);
 }
 
 // v + v of the lane whose id differs in bit M: VALU cross-lane forms where the ISA has

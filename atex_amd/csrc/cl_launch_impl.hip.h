@@ -99,10 +99,12 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
       const unsigned tag = next_call_tag();
       const int polls = tuning().cl_single_polls;
+      const dim3 sgrid = p.single_xm ? dim3(static_cast<unsigned>(p.xm_grid), 1, 1) : grid;
+      const int xm_tiles = p.single_xm ? p.CT : 0;
 #define ATEXN_CL_FWD_SINGLE(U_, FULL_)                                                          \
-  cl_fwd_single<T, V, U_, FULL_><<<grid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, \
-                                                              rstd, D, Ci, p.S, p.tpp_shift,     \
-                                                              p.slab_len, eps, tag, polls)
+  cl_fwd_single<T, V, U_, FULL_><<<sgrid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, \
+                                                               rstd, N, D, Ci, p.S, p.tpp_shift,  \
+                                                               p.slab_len, eps, tag, polls, xm_tiles)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_FWD_SINGLE(4, true);
         else ATEXN_CL_FWD_SINGLE(8, true);
@@ -214,10 +216,20 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       const unsigned tag = next_call_tag();
       const int polls = tuning().cl_single_polls;
       const int Ni = static_cast<int>(N);
+      // XCD-major grid: no fold over the instances in the kernel; a single instance's sums are
+      // dgamma / dbeta, else per-instance rows for col_reduce
+      const dim3 sgrid = p.single_xm ? dim3(static_cast<unsigned>(p.xm_grid), 1, 1) : grid;
+      const int xm_tiles = p.single_xm ? p.CT : 0;
+      float* xpart = reinterpret_cast<float*>(w + p.off_xm_part);
+      float* o0 = N == 1 ? dgamma : xpart;
+      float* o1 = N == 1 ? dbeta : xpart + C;
+      const int64_t o_stride = N == 1 ? 0 : 2 * C;
+      if (p.single_xm && !p.xm_fold) finals_dev = nullptr;
 #define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
-  cl_bwd_single<T, V, U_, FULL_><<<grid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, \
-                                                              finals_dev, dx, dgamma, dbeta, Ni, D, Ci, \
-                                                              p.S, p.tpp_shift, p.slab_len, tag, polls)
+  cl_bwd_single<T, V, U_, FULL_><<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, \
+                                                               finals_dev, dx, dgamma, dbeta, Ni, D, Ci, \
+                                                               p.S, p.tpp_shift, p.slab_len, tag, polls, \
+                                                               xm_tiles, o0, o1, o_stride)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_BWD_SINGLE(4, true);
         else ATEXN_CL_BWD_SINGLE(8, true);
@@ -227,6 +239,7 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       }
 #undef ATEXN_CL_BWD_SINGLE
       ATEXN_CHECK_LAUNCH("cl_bwd_single");
+      if (p.single_xm && !p.xm_fold && N > 1) return launch_col_reduce(xpart, dgamma, dbeta, static_cast<int>(N), C, st);
       return ATEXN_OK;
     }
     if (C % V != 0) {

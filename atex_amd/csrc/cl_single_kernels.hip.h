@@ -65,15 +65,41 @@ __device__ __forceinline__ ClGeom cl_geom_of_slab(const ClGeom& g, int l, int64_
   return h;
 }
 
+// Which (instance, slab, channel tile) the calling workgroup takes.  xm_tiles == 0: the grid is
+// (N, S, channel tiles), every workgroup of the launch is on the chip at once and N is a multiple
+// of the XCD count, which puts an instance's workgroups on one XCD.  xm_tiles > 0 (the number of
+// channel tiles): a one-dimensional, XCD-major grid for any N and any number of workgroups:
+// workgroups are dealt to the 8 XCDs in turn and each XCD starts its workgroups in index order, so
+// workgroup b takes slab (b / 8) % S of unit ((b / 8) / S) * 8 + b % 8, a unit being an (instance,
+// channel tile) pair: the S workgroups of a unit are consecutive workgroups of one XCD, resident
+// together when S is at most what an XCD holds, and wait only for each other.  False: the
+// workgroup has nothing to do (the grid is padded to whole units per XCD).
+constexpr int kClSingleXcds = 8;
+__device__ __forceinline__ bool cl_single_place(int64_t N, int S, int xm_tiles, int64_t& n, int& s, int& ct) {
+  if (xm_tiles == 0) {
+    n = blockIdx.x;
+    s = static_cast<int>(blockIdx.y);
+    ct = static_cast<int>(blockIdx.z);
+    return true;
+  }
+  const unsigned b = blockIdx.x;
+  const unsigned xcd = b % kClSingleXcds, j = b / kClSingleXcds;
+  const int64_t unit = static_cast<int64_t>(j / static_cast<unsigned>(S)) * kClSingleXcds + xcd;
+  s = static_cast<int>(j % static_cast<unsigned>(S));
+  n = unit / xm_tiles;
+  ct = static_cast<int>(unit % xm_tiles);
+  return unit < N * xm_tiles;
+}
+
 // ------------------------------------------------------------------------------ forward
 // tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std).
-// Grid (N, S, channel tiles) as for the two-stage kernels; tile of at most 64 channels.
+// Grid: see cl_single_place; tile of at most 64 channels.
 template <typename T, int V, int U, bool FULL>
 __global__ void __launch_bounds__(kClThreads, 2)
 cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const float* __restrict__ gamma,
               const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
-              float* __restrict__ rstd_out, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
-              float eps, unsigned tag, int max_polls) {
+              float* __restrict__ rstd_out, int64_t N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
+              float eps, unsigned tag, int max_polls, int xm_tiles) {
   __shared__ float lds[V * kClThreads];
   __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
   __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
@@ -81,7 +107,10 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
   const int CV = C / V;
   const int TPP = 1 << tpp_shift;
   const int cap = TPP * V;
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  int64_t n_;
+  int s_, ct_;
+  if (!cl_single_place(N, S, xm_tiles, n_, s_, ct_)) return;
+  const ClGeom g = cl_geom_at<false>(n_, s_, ct_, tpp_shift, CV, C, V, D, slab_len);
   const int c_base = g.ct * cap;
   const int cap_here = C - c_base < cap ? C - c_base : cap;
   const int lane = threadIdx.x & (kWave - 1);
@@ -201,14 +230,18 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
 // instances' sums, for the workgroups of the instance; finals_dev: the same pairs written
 // through to memory, for the workgroups of instance 0, which own the fold over the instances:
 // the owner of channel c there adds up the N pairs of c (a lane per instance) into dgamma[c]
-// and dbeta[c] after it has stored its dx.  N <= 64.
+// and dbeta[c] after it has stored its dx.  N <= 64.  finals_dev == nullptr (the XCD-major grid,
+// whose workgroups are not all on the chip together): the owners leave the instances' sums at
+// o0[n * o_stride + c] (sum dy * xh) and o1[n * o_stride + c] (sum dy) instead: dgamma / dbeta
+// themselves for a single instance, partial rows for a col_reduce launch otherwise.
 template <typename T, int V, int U, bool FULL>
 __global__ void __launch_bounds__(kClThreads, 2)
 cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
               const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
               cl_word* finals, cl_word* finals_dev, T* __restrict__ dx, float* __restrict__ dgamma,
               float* __restrict__ dbeta, int N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
-              unsigned tag, int max_polls) {
+              unsigned tag, int max_polls, int xm_tiles, float* __restrict__ o0, float* __restrict__ o1,
+              int64_t o_stride) {
   __shared__ float lds[2 * V * kClThreads];
   __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
   __shared__ float sm_mu[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_ca[kClSingleMaxCap], sm_cb[kClSingleMaxCap];
@@ -217,7 +250,10 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   const int CV = C / V;
   const int TPP = 1 << tpp_shift;
   const int cap = TPP * V;
-  const ClGeom g = cl_geom<false>(tpp_shift, CV, C, V, D, slab_len);
+  int64_t n_;
+  int s_, ct_;
+  if (!cl_single_place(N, S, xm_tiles, n_, s_, ct_)) return;
+  const ClGeom g = cl_geom_at<false>(n_, s_, ct_, tpp_shift, CV, C, V, D, slab_len);
   const int c_base = g.ct * cap;
   const int cap_here = C - c_base < cap ? C - c_base : cap;
   const int lane = threadIdx.x & (kWave - 1);
@@ -273,7 +309,12 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       const float a = group_sum<kWave>(lane < S ? pa : 0.f);
       if (lane == 0) {
         cl_publish(finals + (g.n * C + c) * 2, b, a, tag);
-        cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+        if (finals_dev != nullptr) {
+          cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+        } else {
+          o0[g.n * o_stride + c] = b;
+          o1[g.n * o_stride + c] = a;
+        }
       }
     }
     if (!fail) {
@@ -328,7 +369,12 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
         constants(lc, gamma[c], mean_in[g.n * C + c], rstd_in[g.n * C + c], b, a);
         if (lc % S == g.s) {  // an owner still serves its peers
           cl_publish(finals + (g.n * C + c) * 2, b, a, tag);
-          cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+          if (finals_dev != nullptr) {
+            cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
+          } else {
+            o0[g.n * o_stride + c] = b;
+            o1[g.n * o_stride + c] = a;
+          }
         }
       }
     }
@@ -339,11 +385,13 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   // The owners of instance 0 also fold the instances' sums into dgamma / dbeta (below, after
   // their dx is on its way).  The other instances' owners published their sums a hop ago: a first
   // look now, whose round trip passes under the stores, usually finds them.
-  const bool folds_instances = g.n == 0 && g.s < cap_here;  // uniform over the workgroup
-  const cl_word* first_dev = finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c_base + g.s) * 2;
+  const bool folds_instances = finals_dev != nullptr && g.n == 0 && g.s < cap_here;  // uniform over the workgroup
   float eb = 0.f, ea = 0.f;
   bool early = false;
-  if (folds_instances && wave == 0 && max_polls > 0) early = cl_try_pair(first_dev, lane < N, tag, eb, ea);
+  if (folds_instances && wave == 0 && max_polls > 0) {
+    early = cl_try_pair(finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c_base + g.s) * 2, lane < N, tag,
+                        eb, ea);
+  }
   if (g.ch_ok) {
     ClBwdCoef<V, false> k;
     k.load(g, tpp_shift, sm_mu, sm_sc, sm_ca, sm_cb);

@@ -62,6 +62,7 @@ struct Tuning {
   // slab is register-resident and all workgroups fit the chip at once; and how many polls a wait
   // for a peer's partials may take before a workgroup recomputes them itself (0: at once)
   TuneInt cl_single{1};
+  TuneInt cl_single_xm{1};  //   also on the XCD-major grid (any batch size, any number of workgroups)
   TuneInt cl_single_polls{2000};
   TuneInt affine_fold{1};      // channel-first backward, a workgroup per plane: dgamma / dbeta folded over the batch in the row kernel
   TuneInt affine_fold_polls{2000};  //   polls before a workgroup recomputes its peers' plane sums (0: at once)
@@ -538,6 +539,17 @@ struct ClPlan {
   // fallback, in the same workspace.
   bool single = false;
   size_t off_tagged = 0, off_finals = 0, off_finals_dev = 0;
+  // The same kernels on a one-dimensional XCD-major grid (cl_single_place) for launches that do
+  // not meet the conditions on N and on the number of workgroups: any batch size, any number of
+  // instances; an instance's slabs must fit one XCD (two workgroups per CU).  The backward then
+  // leaves per-instance sums at off_xm_part for a col_reduce launch (N > 1).
+  bool single_xm = false;
+  int xm_grid = 0;
+  size_t off_xm_part = 0;
+  // ... unless every workgroup of the XCD-major grid is on the chip at once after all (whole
+  // units per XCD, N <= 64): the fold over the instances then runs in the kernel as on the
+  // other grid
+  bool xm_fold = false;
 };
 constexpr int kClFoldAbove = 64;
 constexpr int kPlanClSingleMaxCap = 64, kPlanClSingleMaxSlabs = 64, kPlanClSingleMaxOwned = 4;
@@ -565,7 +577,8 @@ inline int cl_dparam_chunk_shift(int64_t rows, int64_t W2, int64_t n_blocks) {
   return best_shift;
 }
 
-inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
+// force_S > 0: that many slabs per instance instead of the count the rules below arrive at.
+inline ClPlan plan_cl_with(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus, int64_t force_S) {
   const Tuning& t = tuning();
   ClPlan p;
   p.V = V;
@@ -643,6 +656,7 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
       }
     }
   }
+  if (force_S > 0 && !single_pass) S = std::min<int64_t>(force_S, std::min<int64_t>(max_s, s_cap));
   p.slab_len = round_up(div_up(D, S), ppb);
   p.S = static_cast<int>(div_up(D, p.slab_len));
   p.n_work = N * p.S * p.CT;
@@ -671,17 +685,45 @@ inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus)
   const int cap_here = static_cast<int>(std::min<int64_t>(cap, C));
   // (slabs of at most 8 vectors per thread: with 16 the forward kernel does not fit the registers
   // of two workgroups per CU)
-  p.single = t.cl_single && V > 1 && C % V == 0 && p.U > 0 && p.U <= 8 && !p.fold && !p.fused && p.S >= 2 &&
-             p.S <= kPlanClSingleMaxSlabs && N % kPlanXcdCount == 0 && N <= 64 && p.n_work <= int64_t(cus) * 2 &&
-             cap <= kPlanClSingleMaxCap && div_up(cap_here, p.S) <= kPlanClSingleMaxOwned;
+  const bool single_ok = t.cl_single && V > 1 && C % V == 0 && p.U > 0 && p.U <= 8 && !p.fold && !p.fused &&
+                         p.S >= 2 && p.S <= kPlanClSingleMaxSlabs && cap <= kPlanClSingleMaxCap &&
+                         div_up(cap_here, p.S) <= kPlanClSingleMaxOwned;
+  p.single = single_ok && N % kPlanXcdCount == 0 && N <= 64 && p.n_work <= int64_t(cus) * 2;
+  const int64_t xm_grid = round_up(N * p.CT, kPlanXcdCount) * p.S;
+  p.single_xm = single_ok && !p.single && t.cl_single_xm && p.S <= cus / kPlanXcdCount * 2 &&
+                xm_grid < (int64_t(1) << 31);
+  if (p.single_xm) {
+    p.single = true;
+    p.xm_grid = static_cast<int>(xm_grid);
+    p.xm_fold = N > 1 && N <= 64 && div_up(N * p.CT, kPlanXcdCount) * p.S <= cus / kPlanXcdCount * 2;
+  }
   if (p.single) {
     // tagged pairs: 16 bytes per (instance, slab, channel); finals: 16 bytes per (instance, channel), twice
     p.off_tagged = 0;
     p.off_finals = align256(size_t(16) * size_t(N) * size_t(p.S) * size_t(C));
     p.off_finals_dev = p.off_finals + align256(size_t(16) * size_t(N) * size_t(C));
     p.ws_bytes = std::max(p.ws_bytes, p.off_finals_dev + align256(size_t(16) * size_t(N) * size_t(C)));
+    if (p.single_xm) {  // (the finals_dev section is not used; the per-instance sums take its place)
+      p.off_xm_part = p.off_finals_dev;
+    }
   }
   return p;
+}
+
+inline ClPlan plan_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) {
+  const ClPlan p = plan_cl_with(bwd, V, N, C, D, cus, 0);
+  const Tuning& t = tuning();
+  if (p.single || p.fused || !t.cl_single || !t.cl_single_xm || V == 1) return p;
+  // The slab count above suits the two-stage kernels (fewer, longer slabs when there are many
+  // instances).  One launch and one pass over x (and dy) is worth more where it is possible:
+  // with slabs of at most 8 vectors per thread, if an instance then has no more slabs than the
+  // single-launch kernels take.  (A call that cannot use them, in place or under capture, runs
+  // the two-stage kernels on these slabs.)
+  const int ppb = 256 / p.TPP;
+  const int64_t s_x = div_up(D, int64_t(ppb) * 8);
+  if (s_x < 2 || s_x > kPlanClSingleMaxSlabs) return p;
+  const ClPlan q = plan_cl_with(bwd, V, N, C, D, cus, s_x);
+  return q.single ? q : p;
 }
 
 }  // namespace atexn

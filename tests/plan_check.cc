@@ -227,9 +227,23 @@ static void check_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) 
     // workgroup on the chip at once, the workgroups of an instance on one XCD
     const int cap = p.TPP * V;
     EXPECT(V > 1 && C % V == 0 && p.U >= 4 && p.U <= 8 && !p.fused && !p.fold, "single: U=%d", p.U);
-    EXPECT(p.S >= 2 && p.S <= 64 && N <= 64 && N % 8 == 0, "single: S=%d N=%lld", p.S, (long long)N);
+    EXPECT(p.S >= 2 && p.S <= 64, "single: S=%d", p.S);
     EXPECT(cap <= 64 && div_up(std::min<int64_t>(cap, C), p.S) <= 4, "single: cap=%d S=%d", cap, p.S);
-    EXPECT(p.n_work <= int64_t(cus) * 2, "single: %lld workgroups on %d CUs", (long long)p.n_work, cus);
+    if (!p.single_xm) {
+      // the (N, S, tiles) grid: every workgroup resident, an instance per XCD, a lane per instance
+      EXPECT(N <= 64 && N % 8 == 0, "single: N=%lld", (long long)N);
+      EXPECT(p.n_work <= int64_t(cus) * 2, "single: %lld workgroups on %d CUs", (long long)p.n_work, cus);
+    } else {
+      // the XCD-major grid: an instance's slabs fit one XCD, whole units per XCD, the
+      // per-instance sums of the backward where the written-through finals would be
+      EXPECT(p.S <= cus / 8 * 2, "single, XCD-major: S=%d on %d CUs", p.S, cus);
+      EXPECT(int64_t(p.xm_grid) == (N * p.CT + 7) / 8 * 8 * p.S, "single, XCD-major: grid=%d", p.xm_grid);
+      EXPECT(p.off_xm_part >= p.off_finals + size_t(16) * N * C && p.ws_bytes >= p.off_xm_part + sizeof(float) * 2 * N * C,
+             "single, XCD-major: per-instance sums");
+      if (p.xm_fold) {
+        EXPECT(N > 1 && N <= 64 && (N * p.CT + 7) / 8 * p.S <= cus / 8 * 2, "single, XCD-major, fold in the kernel: N=%lld", (long long)N);
+      }
+    }
     EXPECT(p.off_tagged % 256 == 0 && p.off_finals >= p.off_tagged + size_t(16) * N * p.S * C &&
                p.off_finals_dev >= p.off_finals + size_t(16) * N * C &&
                p.ws_bytes >= p.off_finals_dev + size_t(16) * N * C,

@@ -48,6 +48,8 @@ def test_concurrent_threads_and_streams():
         # the channel-first backward that folds its plane sums over the batch in the row kernel
         "in_cl_single": ((8, 128 * 128, 64), 64),
         "in_cf_fold": ((8, 64, 128 * 128), 64),
+        # the same channels-last kernels on the XCD-major grid (a batch that is no multiple of 8)
+        "in_cl_xm": ((5, 64 * 64, 64), 64),
         # channel-first planes spread over the workgroups of an XCD (16 chunks each)
         "in_cf_planes": ((2, 8, 64 * 64 * 128), 8),
     }

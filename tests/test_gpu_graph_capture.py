@@ -17,17 +17,18 @@ EPS = 1e-3
 def test_graph_replay_matches_eager(case):
     import torch
 
-    # (the staged case through the benchmark build with the kernels that would take these planes
-    # in eager mode, but not under capture, switched off: eager and replay then run the same ones)
-    staged = case == "in_channel_first_staged"
-    capi = util.Capi(bench=staged)
-    if staged:
-        assert capi.L.atexn_set_tuning(b"plane_single", 0) == 0
+    # (two cases through the benchmark build with the kernels that would take their shapes in
+    # eager mode, but not under capture, switched off: eager and replay then run the same ones;
+    # test_graph_capture_of_a_single_launch_shape covers what happens otherwise)
+    switch = {"in_channel_first_staged": b"plane_single", "in_channels_last": b"cl_single"}.get(case)
+    capi = util.Capi(bench=switch is not None)
+    if switch:
+        assert capi.L.atexn_set_tuning(switch, 0) == 0
     try:
         _replay_matches_eager(capi, case)
     finally:
-        if staged:
-            assert capi.L.atexn_set_tuning(b"plane_single", 1) == 0
+        if switch:
+            assert capi.L.atexn_set_tuning(switch, 1) == 0
 
 
 def _replay_matches_eager(capi, case):

@@ -303,11 +303,17 @@ def _bits(t):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (8, 32, 4096), (16, 64, 4000), (8, 128, 8192), (8, 24, 5000),
-                                   (32, 64, 4096), (8, 64, 2048), (8, 256, 4096)])
+                                   (32, 64, 4096), (8, 64, 2048), (8, 256, 4096),
+                                   # the XCD-major grid: batches that are no multiples of 8, more
+                                   # workgroups than the chip holds, a single instance, many instances
+                                   (4, 64, 16384), (16, 64, 16384), (2, 128, 4096), (1, 64, 8192), (3, 24, 5000),
+                                   (100, 64, 2048), (5, 256, 4096)])
 def test_channels_last_single_launch(coracle, N, C, S, dtype):
-    """Register-resident slabs, every workgroup on the chip at once, N a multiple of 8: statistics
-    and their use run as ONE launch per direction whose workgroups exchange tagged partials while
-    they run.  Checked against the oracle, and three ways against itself through the benchmark
+    """Register-resident slabs whose instance fits one XCD: statistics and their use run as ONE
+    launch per direction whose workgroups exchange tagged partials while they run (every
+    workgroup on the chip at once and N a multiple of 8: the (N, slabs, tiles) grid, dgamma / dbeta
+    folded over the instances in the kernel; otherwise the XCD-major grid and a col_reduce over the
+    instances).  Checked against the oracle, and three ways against itself through the benchmark
     build of the library (which can switch the path off and set the poll limit):
       * with a poll limit of 0 every workgroup gives up waiting at once and recomputes the other
         slabs itself: the outputs must have the bits of the normal run (the fallback is the same
