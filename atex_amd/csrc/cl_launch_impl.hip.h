@@ -12,17 +12,6 @@ static_assert(kPlanClSingleMaxCap == kClSingleMaxCap && kPlanClSingleMaxSlabs ==
                   kPlanClSingleMaxOwned == kClSingleMaxOwned,
               "the planner and the single-launch kernels must agree on their limits");
 
-// The single-launch kernels tag what they exchange with a number taken per call, which a graph
-// replay would repeat: callers that capture get the two-stage kernels.
-inline bool stream_is_capturing(hipStream_t st) {
-  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
-    (void)hipGetLastError();
-    return true;
-  }
-  return status != hipStreamCaptureStatusNone;
-}
-
 static_assert(kPlanClFoldRegs == 2 * kClFoldRegs, "the planner and the kernels must agree on the fold's register limit");
 
 // Whether every register-resident slab of the plan holds exactly U pixels per pixel slot and
@@ -93,7 +82,7 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       ATEXN_CHECK_LAUNCH("cl_fwd_fused");
       return ATEXN_OK;
     }
-    if (p.single && static_cast<const void*>(y) != static_cast<const void*>(x) && !stream_is_capturing(st)) {
+    if (p.single && static_cast<const void*>(y) != static_cast<const void*>(x) && exchange_allowed(st)) {
       char* w = static_cast<char*>(ws);
       cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
       cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
@@ -208,7 +197,7 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       if (N > 1) return launch_col_reduce(part, dgamma, dbeta, static_cast<int>(N), C, st);
       return ATEXN_OK;
     }
-    if (p.single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && !stream_is_capturing(st)) {
+    if (p.single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && exchange_allowed(st)) {
       char* w = static_cast<char*>(ws);
       cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
       cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);

@@ -1,6 +1,7 @@
 // dtype dispatch, shared helper kernels, error state and tunables.
 #include <atomic>
 #include <chrono>
+#include <cstdlib>
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
@@ -44,6 +45,20 @@ unsigned next_call_tag() {
       static_cast<unsigned>(std::chrono::steady_clock::now().time_since_epoch().count()) | 1u};
   unsigned t = counter.fetch_add(1, std::memory_order_relaxed);
   return t == 0 ? counter.fetch_add(1, std::memory_order_relaxed) : t;
+}
+
+bool exchange_allowed(void* st) {
+  static const bool disabled = [] {
+    const char* v = std::getenv("ATEXN_NO_EXCHANGE");
+    return v != nullptr && v[0] != '\0' && !(v[0] == '0' && v[1] == '\0');
+  }();
+  if (disabled) return false;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(static_cast<hipStream_t>(st), &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return false;
+  }
+  return status == hipStreamCaptureStatusNone;
 }
 
 int cu_count() {

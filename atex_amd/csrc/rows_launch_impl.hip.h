@@ -16,17 +16,6 @@ namespace atexn {
 static_assert(kFoldLdsBytes == kPlanFoldLdsBytes && kFoldMaxWaves == kPlanFoldMaxWaves,
               "the planner sizes the fold's LDS with the kernels' constants");
 
-// The in-kernel fold over the batch tags what it exchanges with a number taken per call, which a
-// graph replay would repeat: callers that capture get the col_reduce launch.
-inline bool rows_stream_is_capturing(hipStream_t st) {
-  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
-  if (hipStreamIsCapturing(st, &status) != hipSuccess) {
-    (void)hipGetLastError();
-    return true;
-  }
-  return status != hipStreamCaptureStatusNone;
-}
-
 template <typename T, int V, bool AFF>
 using FwdResidentFn = void (*)(const T*, const float*, const float*, T*, float*, float*, int64_t,
                                int, int, float);
@@ -165,7 +154,7 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
     return ATEXN_OK;
   }
   if constexpr (AFF && V > 1) {
-    if (p.plane_single && static_cast<const void*>(y) != static_cast<const void*>(x) && !rows_stream_is_capturing(st)) {
+    if (p.plane_single && static_cast<const void*>(y) != static_cast<const void*>(x) && exchange_allowed(st)) {
       static_assert(kPlaneThreads == kPlanPlaneThreads && kPlaneMaxChunks == kPlanPlaneMaxChunks && kPlaneXcds == kPlanXcdCount,
                     "plan_rows sizes the plane_*_single launches");
       cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
@@ -339,7 +328,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     if (!fn) return set_error(ATEXN_LAUNCH_ERROR, "no resident backward kernel for tpr=%d vpt=%d", p.tpr, p.vpt);
     AffineFold fold;
     if (AFF && p.affine_fold && static_cast<const void*>(dx) != static_cast<const void*>(dy) &&
-        !rows_stream_is_capturing(st)) {
+        exchange_allowed(st)) {
       // the plane sums are folded over the batch inside the row kernel: no col_reduce
       fold.tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_tagged);
       fold.dgamma = dgamma;
@@ -362,7 +351,7 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);
   }
   if constexpr (AFF && V > 1) {
-    if (p.plane_single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && !rows_stream_is_capturing(st)) {
+    if (p.plane_single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && exchange_allowed(st)) {
       cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
       const int n_vec = static_cast<int>(D / V);
       auto fn = p.ps_full ? plane_bwd_single<T, V, kPlanPlaneVpt, true> : plane_bwd_single<T, V, kPlanPlaneVpt, false>;

@@ -21,6 +21,15 @@ int cu_count();
 // process-wide atomic counter, started from the clock.
 unsigned next_call_tag();
 
+// Whether a call on stream `st` may take the kernels whose workgroups exchange partial results
+// while they run.  Not while the stream is being captured (a graph replay would repeat the call's
+// tag), and not in a process started with ATEXN_NO_EXCHANGE set to anything but "0": those
+// kernels need the workgroups of one instance / plane on the chip together, which a process that
+// keeps other kernels resident on the same GPU (communication kernels overlapped with compute)
+// may never give them; every wait then runs out and every workgroup recomputes its peers' share.
+// The results are the same; the time is not.  The variable is read once, at the first call.
+bool exchange_allowed(void* st);
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ATEXN_REQUIRE(cond, ...)                                                  \

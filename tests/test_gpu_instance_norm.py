@@ -545,3 +545,56 @@ def test_channel_first_planes_across_workgroups_in_place(capi, coracle):
     """y written over x (dx over dy) keeps such a call on the two-stage kernels (the one-launch
     kernels' fallback reads other workgroups' chunks of x): results as good as out of place."""
     run_case(capi, coracle, 2, 4, 262144, "f16", True, 96, in_place=True)
+
+
+_DIGEST_SCRIPT = r"""
+import hashlib, sys
+import torch
+sys.path.insert(0, sys.argv[1])
+from tests import util
+capi = util.Capi(bench=sys.argv[2] == "bench")
+if sys.argv[2] == "bench":
+    for name in (b"cl_single", b"plane_single", b"affine_fold"):
+        assert capi.L.atexn_set_tuning(name, 0) == 0
+h = hashlib.sha256()
+for N, C, S, cf in ((8, 64, 16384, False), (16, 32, 4096, False), (2, 4, 262144, True), (8, 64, 16384, True)):
+    gen = torch.Generator(device="cuda").manual_seed(1234 + N + S)
+    shape = (N, C, S) if cf else (N, S, C)
+    x = (torch.randn(shape, device="cuda", generator=gen) + 0.5).half()
+    dy = torch.randn(shape, device="cuda", generator=gen).half()
+    gamma = torch.rand(C, device="cuda", generator=gen) + 0.5
+    beta = torch.randn(C, device="cuda", generator=gen)
+    y, m, r = capi.in_fwd(x, gamma, beta, 1e-3, "f16", cf)
+    dx, dg, db = capi.in_bwd(dy, x, gamma, m, r, "f16", cf)
+    torch.cuda.synchronize()
+    for t in (y, m, r, dx, dg, db):
+        h.update(t.contiguous().view(torch.uint8).cpu().numpy().tobytes())
+print("DIGEST", h.hexdigest())
+"""
+
+
+def test_exchange_kernels_can_be_switched_off_for_a_process():
+    """ATEXN_NO_EXCHANGE=1 in the environment keeps every call of a process on the kernels that
+    need no workgroups resident together (for processes that keep other kernels on the GPU all
+    the time).  A child process with the variable set, calling the product library, must produce
+    the bits that the benchmark build produces with those kernels switched off by its tuning hook
+    (a second child, so that both see the same seeded inputs from a fresh process)."""
+    import os
+    import subprocess
+    import sys
+
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+    def digest(flavour, extra_env):
+        env = dict(os.environ, **extra_env)
+        out = subprocess.run([sys.executable, "-c", _DIGEST_SCRIPT, root, flavour], env=env, capture_output=True,
+                             text=True, timeout=300)
+        assert out.returncode == 0, out.stderr[-2000:]
+        lines = [ln for ln in out.stdout.splitlines() if ln.startswith("DIGEST ")]
+        assert len(lines) == 1, out.stdout[-2000:]
+        return lines[0]
+
+    print("child processes: product library with ATEXN_NO_EXCHANGE=1, benchmark build with the switches off", flush=True)
+    off_by_env = digest("product", {"ATEXN_NO_EXCHANGE": "1"})
+    off_by_hook = digest("bench", {"ATEXN_NO_EXCHANGE": "0"})
+    assert off_by_env == off_by_hook
