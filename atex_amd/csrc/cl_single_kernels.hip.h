@@ -1,5 +1,6 @@
-// Channels-last InstanceNorm in ONE launch per direction, for launches whose slabs are all
-// register-resident and whose workgroups are all on the chip at once (two per CU).
+// Channels-last InstanceNorm in ONE launch per direction, for instances that can be cut into at
+// most 64 register-resident slabs: the workgroups of one instance must be on the chip together,
+// on one XCD (cl_single_place below has the two grids that see to that).
 //
 // The two-stage kernels (cl_kernels.hip.h) read x (and dy) twice and pay a kernel boundary
 // between the statistics and their use.  Here a workgroup keeps its slab in registers and the
@@ -18,10 +19,9 @@
 // The second word of a pair carries the complemented tag, so that 64 bits of arbitrary memory
 // contents would have to match before garbage in a fresh workspace is taken for data.  Readers
 // use device-scope loads, which go past the vector and L2 caches' stale lines; writers use plain
-// stores, which reach the L2 of their XCD: every workgroup of an instance runs on the same XCD
-// (the host only takes this path when the instance index, the fastest grid coordinate, is
-// congruent to the workgroup id modulo the eight XCDs), and that L2 is where those loads look.
-// A hop costs about 2 us, against about 3.5 us for the kernel boundary and the second read.
+// stores, which reach the L2 of their XCD: every workgroup of an instance runs on the same XCD,
+// and that L2 is where those loads look.  A hop costs about 2 us, against about 3.5 us for the
+// kernel boundary and the second read.
 //
 // Nothing here can hang: every wait is a bounded number of polls.  A workgroup whose wait runs
 // out (its peers are not resident: another kernel holds the CUs; or the placement assumption
