@@ -90,10 +90,15 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       const int polls = tuning().cl_single_polls;
       const dim3 sgrid = p.single_xm ? dim3(static_cast<unsigned>(p.xm_grid), 1, 1) : grid;
       const int xm_tiles = p.single_xm ? p.CT : 0;
+      // more instances than the chip holds at once: the kernel compiled for more workgroups per CU
+      // (16-bit data; the float32 kernel needs fewer registers to begin with and gains nothing)
+      const bool occ = p.single_xm && !p.xm_resident && sizeof(T) == 2 && tuning().cl_single_occ;
 #define ATEXN_CL_FWD_SINGLE(U_, FULL_)                                                          \
-  cl_fwd_single<T, V, U_, FULL_><<<sgrid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, \
-                                                               rstd, N, D, Ci, p.S, p.tpp_shift,  \
-                                                               p.slab_len, eps, tag, polls, xm_tiles)
+  do {                                                                                          \
+    auto fn = occ ? cl_fwd_single<T, V, U_, FULL_, true> : cl_fwd_single<T, V, U_, FULL_, false>; \
+    fn<<<sgrid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, rstd, N, D, Ci, p.S, \
+                                     p.tpp_shift, p.slab_len, eps, tag, polls, xm_tiles);       \
+  } while (0)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_FWD_SINGLE(4, true);
         else ATEXN_CL_FWD_SINGLE(8, true);
@@ -214,11 +219,17 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       float* o1 = N == 1 ? dbeta : xpart + C;
       const int64_t o_stride = N == 1 ? 0 : 2 * C;
       if (p.single_xm && !p.xm_fold) finals_dev = nullptr;
+      // (the backward only with at most 32 slabs per instance: with 64, three workgroups per CU
+      // are one and a half instances per XCD and the registers moved to scratch memory cost as
+      // much: [16, 128^2, 64] fp16 25.4 -> 26.4 us, [128, 64^2, 64] 49.6 -> 43.9 us)
+      const bool occ = p.single_xm && !p.xm_resident && p.S <= 32 && tuning().cl_single_occ;
 #define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
-  cl_bwd_single<T, V, U_, FULL_><<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, \
-                                                               finals_dev, dx, dgamma, dbeta, Ni, D, Ci, \
-                                                               p.S, p.tpp_shift, p.slab_len, tag, polls, \
-                                                               xm_tiles, o0, o1, o_stride)
+  do {                                                                                          \
+    auto fn = occ ? cl_bwd_single<T, V, U_, FULL_, true> : cl_bwd_single<T, V, U_, FULL_, false>; \
+    fn<<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, finals_dev, dx, dgamma, \
+                                     dbeta, Ni, D, Ci, p.S, p.tpp_shift, p.slab_len, tag, polls, \
+                                     xm_tiles, o0, o1, o_stride);                               \
+  } while (0)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_BWD_SINGLE(4, true);
         else ATEXN_CL_BWD_SINGLE(8, true);

@@ -94,14 +94,19 @@ __device__ __forceinline__ bool cl_single_place(int64_t N, int S, int xm_tiles, 
 // ------------------------------------------------------------------------------ forward
 // tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std).
 // Grid: see cl_single_place; tile of at most 64 channels.
-template <typename T, int V, int U, bool FULL>
-__global__ void __launch_bounds__(kClThreads, 2)
+// OCC: compiled for four workgroups per CU instead of two (128 VGPRs, a few values in scratch
+// memory): an XCD then has the workgroups of two instances in flight, one loading while the
+// other waits for its exchange.  Pays on the XCD-major grid with more instances than the chip
+// holds at once ([16, 128^2, 64] fp16 forward 18.3 -> 14.7 us, [64, 128^2, 64] 68.1 -> 59.3 us);
+// a launch that fits the chip anyway loses a little (config 3: 9.97 -> 10.4 us) and keeps OCC off.
+template <typename T, int V, int U, bool FULL, bool OCC>
+__global__ void __launch_bounds__(kClThreads, OCC ? 4 : 2)
 cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const float* __restrict__ gamma,
               const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
               float* __restrict__ rstd_out, int64_t N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
               float eps, unsigned tag, int max_polls, int xm_tiles) {
   __shared__ float lds[V * kClThreads];
-  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
+  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap];
   __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
   __shared__ int sm_fail;
   const int CV = C / V;
@@ -175,38 +180,47 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
   if (sm_fail) {
     // On its own: the partials of every slab of the instance, computed as their workgroups
     // compute them, folded as their owners fold them.  The slabs pass through the registers of
-    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).
-    for (int l = 0; l < S; ++l) {
-      const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
-      cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
-      float mm[V], qq[V];
-      __syncthreads();  // the previous round's block sums have been read
-      cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
-      if (g.ch_ok && g.slot == 0) {
-        const int lc0 = g.coff - c_base;
+    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).  Two
+    // rounds, each for half of the tile's channels: fb holds S x cap / 2 pairs (the LDS this
+    // kernel asks for decides how many workgroups a CU takes, and this path hardly ever runs).
+    const int hw = cap / 2;
+    for (int hf = 0; hf < 2; ++hf) {
+      for (int l = 0; l < S; ++l) {
+        const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
+        cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
+        float mm[V], qq[V];
+        __syncthreads();  // the previous round's block sums (and fold) have been read
+        cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
+        if (g.ch_ok && g.slot == 0) {
+          const int lc0 = g.coff - c_base;
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          fb[(l * cap + lc0 + i) * 2] = mm[i];
-          fb[(l * cap + lc0 + i) * 2 + 1] = qq[i];
+          for (int i = 0; i < V; ++i) {
+            const int lh = lc0 + i - hf * hw;
+            if (lh >= 0 && lh < hw) {
+              fb[(l * hw + lh) * 2] = mm[i];
+              fb[(l * hw + lh) * 2 + 1] = qq[i];
+            }
+          }
         }
       }
-    }
-    __syncthreads();
-    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
-      const int c = c_base + lc;
-      const float pm = lane < S ? fb[(lane * cap + lc) * 2] : 0.f;
-      const float pq = lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f;
-      float mu, q;
-      cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
-      if (lane == 0) {
-        const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
-        sm_mean[lc] = mu;
-        sm_sc[lc] = gamma[c] * rs;
-        sm_bt[lc] = beta[c];
-        if (lc % S == g.s) {  // an owner still serves its peers
-          cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
-          mean_out[g.n * C + c] = mu;
-          rstd_out[g.n * C + c] = rs;
+      __syncthreads();
+      for (int lc = hf * hw + wave; lc < cap_here && lc < (hf + 1) * hw; lc += kClThreads / kWave) {
+        const int c = c_base + lc;
+        const int lh = lc - hf * hw;
+        const float pm = lane < S ? fb[(lane * hw + lh) * 2] : 0.f;
+        const float pq = lane < S ? fb[(lane * hw + lh) * 2 + 1] : 0.f;
+        float mu, q;
+        cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
+        if (lane == 0) {
+          const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
+          sm_mean[lc] = mu;
+          sm_sc[lc] = gamma[c] * rs;
+          sm_bt[lc] = beta[c];
+          if (lc % S == g.s) {  // an owner still serves its peers
+            cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
+            mean_out[g.n * C + c] = mu;
+            rstd_out[g.n * C + c] = rs;
+          }
         }
       }
     }
@@ -234,8 +248,8 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
 // whose workgroups are not all on the chip together): the owners leave the instances' sums at
 // o0[n * o_stride + c] (sum dy * xh) and o1[n * o_stride + c] (sum dy) instead: dgamma / dbeta
 // themselves for a single instance, partial rows for a col_reduce launch otherwise.
-template <typename T, int V, int U, bool FULL>
-__global__ void __launch_bounds__(kClThreads, 2)
+template <typename T, int V, int U, bool FULL, bool OCC>
+__global__ void __launch_bounds__(kClThreads, OCC ? 3 : 2)
 cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
               const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
               cl_word* finals, cl_word* finals_dev, T* __restrict__ dx, float* __restrict__ dgamma,

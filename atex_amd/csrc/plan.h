@@ -63,6 +63,7 @@ struct Tuning {
   // for a peer's partials may take before a workgroup recomputes them itself (0: at once)
   TuneInt cl_single{1};
   TuneInt cl_single_xm{1};  //   also on the XCD-major grid (any batch size, any number of workgroups)
+  TuneInt cl_single_occ{1};  //   on that grid, when the launch does not fit the chip: the kernels compiled for more workgroups per CU
   TuneInt cl_single_polls{2000};
   TuneInt affine_fold{1};      // channel-first backward, a workgroup per plane: dgamma / dbeta folded over the batch in the row kernel
   TuneInt affine_fold_polls{2000};  //   polls before a workgroup recomputes its peers' plane sums (0: at once)
@@ -550,6 +551,7 @@ struct ClPlan {
   // units per XCD, N <= 64): the fold over the instances then runs in the kernel as on the
   // other grid
   bool xm_fold = false;
+  bool xm_resident = false;  // every workgroup of the XCD-major grid on the chip at once
 };
 constexpr int kClFoldAbove = 64;
 constexpr int kPlanClSingleMaxCap = 64, kPlanClSingleMaxSlabs = 64, kPlanClSingleMaxOwned = 4;
@@ -695,7 +697,8 @@ inline ClPlan plan_cl_with(bool bwd, int V, int64_t N, int64_t C, int64_t D, int
   if (p.single_xm) {
     p.single = true;
     p.xm_grid = static_cast<int>(xm_grid);
-    p.xm_fold = N > 1 && N <= 64 && div_up(N * p.CT, kPlanXcdCount) * p.S <= cus / kPlanXcdCount * 2;
+    p.xm_resident = div_up(N * p.CT, kPlanXcdCount) * p.S <= cus / kPlanXcdCount * 2;
+    p.xm_fold = N > 1 && N <= 64 && p.xm_resident;
   }
   if (p.single) {
     // tagged pairs: 16 bytes per (instance, slab, channel); finals: 16 bytes per (instance, channel), twice

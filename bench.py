@@ -94,10 +94,14 @@ CASES = {
     "ln_8192x12288_f32": ("ln", "f32", (8192, 12288)),
     # 1024 channel-first planes of 256 x 256: staged in registers + LDS, single pass
     "in_16x64x256x256_cf": ("in", "f16", (16, 64, 256 * 256, True)),
+    # more instances than the chip holds workgroups for at once: the channels-last single-launch
+    # kernels on their XCD-major grid
+    "in_16x128x128x64_cl": ("in", "f16", (16, 64, 128 * 128, False)),
+    "in_64x128x128x64_cl": ("in", "f16", (64, 64, 128 * 128, False)),
 }
 # cases that `--case all` leaves out (single-purpose sweeps and the reference's benchmark table)
 SWEEP_ONLY_CASES = frozenset(
-    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "in_16x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
+    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "in_16x", "in_64x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
 DEFAULT_CASE = "ln_bert"
 # the two shapes the throughput target is stated on, reported on the default run's line
 TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
