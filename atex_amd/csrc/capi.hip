@@ -282,8 +282,8 @@ int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C
                      p.ps_S, p.ps_chunk_vec, p.ps_grid, kPlanPlaneThreads, two,
                      p.ps_fold ? ", plane sums folded over the batch in the kernel" : " + col_reduce");
       else if (k[0] && p.affine_fold)
-        n = snprintf(out, out_bytes, "%s (grid %d x %d threads, vpt=%d), plane sums folded over the batch in the kernel (col_reduce follows instead when dx == dy or under capture); alone=0",
-                     k, p.grid, p.threads, p.vpt);
+        n = snprintf(out, out_bytes, "%s (grid %d x %d threads, tpr=%d vpt=%d rb=%d), plane sums folded over the batch in the kernel (col_reduce follows instead when dx == dy or under capture); alone=0",
+                     k, p.grid, p.threads, p.tpr, p.vpt, p.rb);
       else if (k[0])
         n = snprintf(out, out_bytes, "%s (grid %d x %d threads, tpr=%d vpt=%d rb=%d) + col_reduce over %d partial rows; alone=1",
                      k, p.grid, p.threads, p.tpr, p.vpt, p.rb, p.part_rows);

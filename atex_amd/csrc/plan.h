@@ -153,6 +153,7 @@ struct RowsPlan {
   bool ps_fold = false;
   size_t off_ps_fold = 0;
 };
+constexpr int kPlanAffineFoldMaxStep = 64, kPlanAffineFoldMaxPairs = 1024;
 constexpr int kPlanPlaneThreads = 512, kPlanPlaneVpt = 8, kPlanPlaneMaxChunks = 64;
 
 // Longest row, in vectors, that the register-resident kernels take: forward 8 vectors per
@@ -413,6 +414,15 @@ inline RowsPlan plan_rows(RowsKind kind, int V, int64_t n_rows, int64_t D, int C
       // last-started of those that handle its planes, and waits for none that starts after it)
       p.affine_fold = t.affine_fold && p.tpr == 0 && C % kPlanXcdCount == 0 && p.grid % kPlanXcdCount == 0 &&
                       (p.grid % C == 0 || C % p.grid == 0) && p.part_rows >= 2 && p.part_rows <= 64;
+      if (p.tpr != 0) {
+        // lane groups per plane: q consecutive planes per workgroup and step; the same conditions
+        // on C / q channel groups, and the fallback's LDS (instances x q pairs)
+        const int q = p.rpb * p.rb;
+        const int64_t cg = C / q;
+        p.affine_fold = t.affine_fold && V > 1 && C % q == 0 && cg % kPlanXcdCount == 0 && p.grid % kPlanXcdCount == 0 &&
+                        (p.grid % cg == 0 || cg % p.grid == 0) && p.part_rows >= 2 && p.part_rows <= 64 &&
+                        q <= kPlanAffineFoldMaxStep && int64_t(p.part_rows) * q <= kPlanAffineFoldMaxPairs;
+      }
       if (p.affine_fold) {
         p.off_tagged = p.ws_bytes;
         p.ws_bytes += align256(size_t(16) * size_t(n_rows));

@@ -394,13 +394,17 @@ rows_fwd_resident(const T* x, const float* __restrict__ gamma, const float* __re
 // Channel-first InstanceNorm with a workgroup per plane: the fold of the per-plane sums over the
 // batch (dgamma[c] = sum over n of the plane sums of (n, c)) can run inside the row kernel instead
 // of as a launch of its own.  Every workgroup publishes the two sums of its plane as a tagged
-// pair as soon as it has them, before it computes and stores dx; the workgroup that handled plane
-// (0, c) afterwards waits (a lane per instance, a bounded number of polls) for the N pairs of
-// channel c and adds them up.  The host asks for it only when the planes of a channel are all
-// handled on one XCD (C and the grid multiples of the XCD count: plane n * C + c goes to
-// workgroup (n * C + c) mod grid), so that plain stores are visible to the device-scope polls,
-// when N <= 64, dx != dy and the stream is not being captured.  A workgroup whose wait runs out
-// recomputes the sums of the N planes itself, with the code the row loop uses (same bits).
+// pair as soon as it has them, before it computes and stores dx; after its own planes, one of the
+// last workgroups of the grid waits (a lane per instance, a bounded number of polls) for the N
+// pairs of channel c and adds them up.  The host asks for it only when the planes of a channel are
+// all handled on one XCD, the folding workgroup's (a workgroup per plane: C and the grid multiples
+// of the XCD count, plane n * C + c goes to workgroup (n * C + c) mod grid; q planes per workgroup
+// and step: C / q and the grid multiples of it), so that plain stores are visible to the
+// device-scope polls, when N <= 64, dx != dy and the stream is not being captured.  A workgroup
+// whose wait runs out recomputes the sums of the N planes itself, with the code the row loop uses
+// (same bits).
+constexpr int kAffineFoldMaxStep = 64;     // planes per workgroup and step (lane groups per plane)
+constexpr int kAffineFoldMaxPairs = 1024;  // instances x planes per step that the fallback keeps in LDS
 struct AffineFold {
   cl_word* tagged = nullptr;  // [N * C] pairs (sum dy * xh, sum dy); nullptr: col_reduce follows
   float* dgamma = nullptr;
@@ -581,7 +585,7 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
       if constexpr (ROW_AFFINE) {
         scale *= cur.gm[r];
         if (row_ok[r] && lane_r == 0) {
-          if (TPR == 0 && fold.tagged != nullptr) {
+          if (fold.tagged != nullptr) {
             cl_publish(fold.tagged + row * 2, s2[r], s1[r], fold.tag);
           } else {
             const int64_t n = row / C;
@@ -700,6 +704,77 @@ rows_bwd_resident(const T* dy, const T* __restrict__ x,
             if (lane == 0) {
               fold.dgamma[c] = b;
               fold.dbeta[c] = a;
+            }
+          }
+        }
+        __syncthreads();
+      }
+    }
+  }
+  if constexpr (ROW_AFFINE && TPR != 0) {
+    if (fold.tagged != nullptr) {
+      // Lane groups per plane: a workgroup takes q = rpb * RB consecutive planes per step, i.e.
+      // the channels j * q .. j * q + q - 1 of an instance (C is a multiple of q), and so does the
+      // fold: channel group j belongs to workgroup G-1 - (C/q-1-j) % G, which is started after
+      // every workgroup that handles planes of the group and sits on their XCD (C / q and G
+      // multiples of the XCD count and one of the other).  A wave per channel, a lane per instance.
+      __shared__ int fold_fail[kAffineFoldMaxStep];
+      __shared__ float inst[kAffineFoldMaxPairs][2];
+      const int lane = threadIdx.x & (kWave - 1);
+      const int wave = threadIdx.x / kWave;
+      const int N = fold.N;
+      const int q = rpb * RB;
+      const int64_t groups = C / q;
+      int it = 0;
+      for (int64_t j = groups - static_cast<int64_t>(gridDim.x) + blockIdx.x; j >= 0; j -= gridDim.x) {
+        const int c0 = static_cast<int>(j) * q;
+        if (static_cast<int>(threadIdx.x) < q) fold_fail[threadIdx.x] = 0;
+        __syncthreads();
+        for (int i = wave; i < q; i += n_waves) {
+          float pb, pa;
+          const bool ok = cl_wait_pair(fold.tagged + (static_cast<int64_t>(lane < N ? lane : 0) * C + c0 + i) * 2,
+                                       lane < N, fold.tag, fold.max_polls, pb, pa);
+          if (ok) {
+            const float b = group_sum<kWave>(lane < N ? pb : 0.f);
+            const float a = group_sum<kWave>(lane < N ? pa : 0.f);
+            if (lane == 0) {
+              fold.dgamma[c0 + i] = b;
+              fold.dbeta[c0 + i] = a;
+            }
+          } else if (lane == 0) {
+            fold_fail[i] = 1;
+          }
+        }
+        __syncthreads();
+        bool failed = false;
+        for (int i = 0; i < q; ++i) failed = failed || fold_fail[i] != 0;
+        if (failed) {  // uniform: the planes of these channels, summed here as their workgroups sum them
+          for (int n = 0; n < N; ++n) {
+            Batch t;
+            load_batch(static_cast<int64_t>(n) * C + c0, t);
+            bool row_ok[RB];
+#pragma unroll
+            for (int r = 0; r < RB; ++r) row_ok[r] = true;
+            float xh[RB][NE], gv[RB][NE];
+            float s1[RB], s2[RB];
+            row_sums(t, row_ok, xh, gv, s1, s2, it++);
+            if (lane_r == 0) {
+#pragma unroll
+              for (int r = 0; r < RB; ++r) {
+                inst[n * q + r * rpb + slot][0] = s2[r];
+                inst[n * q + r * rpb + slot][1] = s1[r];
+              }
+            }
+          }
+          __syncthreads();
+          for (int i = wave; i < q; i += n_waves) {
+            if (fold_fail[i]) {
+              const float b = group_sum<kWave>(lane < N ? inst[(lane < N ? lane : 0) * q + i][0] : 0.f);
+              const float a = group_sum<kWave>(lane < N ? inst[(lane < N ? lane : 0) * q + i][1] : 0.f);
+              if (lane == 0) {
+                fold.dgamma[c0 + i] = b;
+                fold.dbeta[c0 + i] = a;
+              }
             }
           }
         }

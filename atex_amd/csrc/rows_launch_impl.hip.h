@@ -13,6 +13,8 @@
 
 namespace atexn {
 
+static_assert(kAffineFoldMaxStep == kPlanAffineFoldMaxStep && kAffineFoldMaxPairs == kPlanAffineFoldMaxPairs,
+              "the planner admits the in-kernel batch fold with the kernels' limits");
 static_assert(kFoldLdsBytes == kPlanFoldLdsBytes && kFoldMaxWaves == kPlanFoldMaxWaves,
               "the planner sizes the fold's LDS with the kernels' constants");
 

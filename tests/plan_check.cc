@@ -158,25 +158,30 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
       EXPECT(n_rows % C == 0 && p.part_rows == n_rows / C, "affine part rows");
       EXPECT(p.ws_bytes >= sizeof(float) * 2 * size_t(n_rows), "affine workspace");
       if (p.affine_fold) {
-        // what the in-kernel fold over the batch assumes: a workgroup per plane, a lane per
-        // instance, the planes of a channel handled on one XCD, its tagged pairs in the workspace
-        EXPECT(p.tpr == 0 && p.rb == 1 && p.part_rows >= 2 && p.part_rows <= 64, "affine fold: tpr=%d N=%d", p.tpr, p.part_rows);
-        EXPECT(C % 8 == 0 && p.grid % 8 == 0, "affine fold: C=%d grid=%d", C, p.grid);
+        // what the in-kernel fold over the batch assumes: q consecutive planes per workgroup and
+        // step (1 with a workgroup per plane), a lane per instance, the planes of a channel group
+        // handled on one XCD, its tagged pairs in the workspace
+        const int64_t q = p.tpr == 0 ? 1 : int64_t(p.rpb) * p.rb;
+        EXPECT((p.tpr == 0 ? p.rb == 1 : r.V > 1) && p.part_rows >= 2 && p.part_rows <= 64, "affine fold: tpr=%d N=%d", p.tpr, p.part_rows);
+        EXPECT(C % q == 0 && (C / q) % 8 == 0 && p.grid % 8 == 0 && q <= 64 && p.part_rows * q <= 1024,
+               "affine fold: C=%d q=%lld grid=%d", C, (long long)q, p.grid);
         EXPECT(p.off_tagged % 256 == 0 && p.off_tagged >= sizeof(float) * 2 * size_t(n_rows) &&
                    p.ws_bytes >= p.off_tagged + size_t(16) * size_t(n_rows),
                "affine fold: workspace");
-        // channel c is folded by workgroup G-1 - (C-1-c) % G (rows_bwd_resident): on the XCD of
-        // every workgroup that handles a plane of c, and started after all of them
-        const int64_t G = p.grid;
+        // channel group j (channels j * q ...) is folded by workgroup G-1 - (C/q-1-j) % G
+        // (rows_bwd_resident): on the XCD of every workgroup that handles a plane of the group,
+        // and started after all of them.  Step t of the row loop (planes t * q ...) runs on
+        // workgroup t % G.
+        const int64_t G = p.grid, cg = C / q;
         bool placed = true;
-        for (int64_t c = 0; c < C && placed; ++c) {
-          const int64_t folder = G - 1 - (C - 1 - c) % G;
+        for (int64_t j = 0; j < cg && placed; ++j) {
+          const int64_t folder = G - 1 - (cg - 1 - j) % G;
           for (int64_t n = 0; n < p.part_rows; ++n) {
-            const int64_t w = (n * C + c) % G;
+            const int64_t w = (n * cg + j) % G;
             if (w > folder || w % 8 != folder % 8) placed = false;
           }
         }
-        EXPECT(placed, "affine fold: C=%d grid=%d: a folding workgroup waits for a later one or another XCD's", C, p.grid);
+        EXPECT(placed, "affine fold: C=%d q=%lld grid=%d: a folding workgroup waits for a later one or another XCD's", C, (long long)q, p.grid);
       }
     }
   } else {

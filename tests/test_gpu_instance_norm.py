@@ -383,11 +383,15 @@ def test_channels_last_single_launch_in_place_takes_two_stages(capi, coracle):
 
 @pytest.mark.parametrize("dtype", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("N,C,S", [(8, 64, 16384), (8, 32, 4096), (16, 64, 3000), (64, 8, 32768), (2, 16, 5001),
-                                   (24, 40, 2048), (8, 512, 8192)])
+                                   (24, 40, 2048), (8, 512, 8192),
+                                   # lane groups per plane, several planes per workgroup and step
+                                   (32, 128, 784), (2, 320, 216), (8, 512, 100), (64, 64, 196), (4, 256, 1000),
+                                   (16, 1024, 64), (3, 128, 49)])
 def test_channel_first_backward_folds_the_batch_in_the_row_kernel(coracle, N, C, S, dtype):
-    """Channel-first planes with a workgroup each, C a multiple of 8, at most 64 instances: the
-    backward's row kernel publishes its plane sums as tagged pairs and the last workgroups of the
-    grid add them up over the batch into dgamma / dbeta, instead of a col_reduce launch
+    """Channel-first planes with a workgroup each (or a group of lanes each, a workgroup then taking
+    several consecutive planes per step), the planes of a channel on one XCD, at most 64 instances:
+    the backward's row kernel publishes its plane sums as tagged pairs and the last workgroups of
+    the grid add them up over the batch into dgamma / dbeta, instead of a col_reduce launch
     ((8, 512, 8192) has more workgroups than the chip holds at once).  Checked
     against the oracle and, through the benchmark build, against itself with the poll limit
     forced to 0 (every folding workgroup recomputes the plane sums of its channel itself: same
