@@ -25,10 +25,11 @@
 //
 // Nothing here can hang: every wait is a bounded number of polls.  A workgroup whose wait runs
 // out (its peers are not resident: another kernel holds the CUs; or the placement assumption
-// does not hold on this device) recomputes, with the same code and therefore to the same bits,
-// the pairs of every chunk of its plane from x (and dy) itself.  That is why the host keeps
-// callers that pass y == x (dx == dy) on the two-stage kernels: a peer may already have
-// overwritten its chunk by then.
+// does not hold on this device) computes, with the same code and therefore to the same bits,
+// the pairs that have not arrived from x (and dy) itself, and publishes them: whoever gives up
+// first does the missing chunks for everybody.  That is why the host keeps callers that pass
+// y == x (dx == dy) on the two-stage kernels: a peer may already have overwritten its chunk by
+// then.
 //
 // Counterpart in the reference: the two-kernel channel-first path for large planes
 // (fused_instance_norm_op.cu:1311-1455 forward, 1168-1309 backward), which reads its inputs
@@ -153,16 +154,46 @@ __device__ __forceinline__ void plane_merge_stats(float pm, float pq, int lane, 
   m2 = group_sum<kWave>(in ? pq + w * (d * d) : 0.f);
 }
 
+// Start of a workgroup's fallback: wave 0 looks once, a lane per chunk, at the pairs of the plane
+// at `pairs`, keeps those that have arrived in fb and notes which have (have[l]); the fallback
+// then computes, and publishes for its peers, only the others.  (When the workgroups of a plane
+// cannot be resident together, the first ones to give up thus do the missing chunks once, and
+// the late ones find everything there, instead of every workgroup redoing the whole plane.)
+// Contains a barrier; have / fb are valid for every thread afterwards.
+__device__ __forceinline__ void plane_look(const cl_word* pairs, int S, unsigned tag, int (&have)[kPlaneMaxChunks],
+                                           float (&fb)[kPlaneMaxChunks][2]) {
+  __syncthreads();  // whatever read have / fb before is done
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    bool ok = false;
+    float a = 0.f, b = 0.f;
+    if (lane < S) {
+      const cl_word w0 = cl_peek(pairs + 2 * lane);
+      const cl_word w1 = cl_peek(pairs + 2 * lane + 1);
+      ok = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
+      a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
+      b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
+    }
+    have[lane] = ok ? 1 : 0;
+    fb[lane][0] = a;
+    fb[lane][1] = b;
+  }
+  __syncthreads();
+}
+
 // ------------------------------------------------------------------------------ forward
 // tagged: [n_rows][S] pairs (mean, m2) of the chunks.  n_vec = D / V, chunk_vec <= U * 512.
+// (FULL: built for four workgroups per CU, 64 VGPRs, which the path that every launch takes needs
+// anyway; the fallback then keeps a few values in scratch memory)
 template <typename T, int V, int U, bool FULL, bool NT>
-__global__ void __launch_bounds__(kPlaneThreads, 4)
+__global__ void __launch_bounds__(kPlaneThreads, FULL ? 8 : 4)
 plane_fwd_single(const T* __restrict__ x, cl_word* tagged, const float* __restrict__ gamma,
                  const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
                  float* __restrict__ rstd_out, int64_t n_rows, int n_vec, int S, int chunk_vec, int C, float eps,
                  unsigned tag, int max_polls) {
   __shared__ Wf wf_buf[2][16];
   __shared__ float fb[kPlaneMaxChunks][2];
+  __shared__ int have[kPlaneMaxChunks];
   __shared__ float sm_mean, sm_rstd;
   __shared__ int sm_fail;
   const PlaneGeom g = plane_geom(n_rows, S);
@@ -199,16 +230,21 @@ plane_fwd_single(const T* __restrict__ x, cl_word* tagged, const float* __restri
   }
   __syncthreads();
   if (sm_fail) {
-    // On its own: the pair of every chunk of the plane, computed as its workgroup computes it.
-    // The chunks pass through the registers of the workgroup's own chunk, which is loaded again
-    // at the end (x is intact: y != x).
+    // On its own: the pair of every chunk of the plane that has not arrived, computed as its
+    // workgroup computes it (and published: the workgroup may turn up late, its peers may be
+    // looking).  The chunks pass through the registers of the workgroup's own chunk, which is
+    // loaded again at the end (x is intact: y != x).
+    plane_look(tagged + g.row * S * 2, S, tag, have, fb);
+    int it = 1;
     for (int l = 0; l < S; ++l) {
+      if (have[l]) continue;  // uniform
       const int n_l = plane_chunk_vectors(l, S, n_vec, chunk_vec);
       plane_load<T, V, U, FULL, NT>(xr + static_cast<int64_t>(l) * chunk_vec * V, n_l, raw);
-      const Wf w = plane_chunk_stats<T, V, U, FULL>(raw, n_l, wf_buf[(l + 1) & 1]);
+      const Wf w = plane_chunk_stats<T, V, U, FULL>(raw, n_l, wf_buf[it++ & 1]);
       if (threadIdx.x == 0) {
         fb[l][0] = w.mean;
         fb[l][1] = w.m2;
+        cl_publish(tagged + (g.row * S + l) * 2, w.mean, w.m2, tag);
       }
     }
     __syncthreads();
@@ -265,24 +301,28 @@ __device__ __forceinline__ float2 plane_chunk_sums(const Pack<T, V> (&rx)[U], co
 }
 
 // (sum dy, sum dy * xh) of a whole plane computed by the calling workgroup alone: the pair of
-// every chunk as its workgroup computes it, added up as the gathering wave adds them.  The
-// chunks pass through rx / rd (the caller reloads its own afterwards).  The result is valid in
-// wave 0; contains barriers.
+// every chunk, as found at `pairs` or else computed as its workgroup computes it (and published
+// there), added up as the gathering wave adds them.  The chunks pass through rx / rd (the caller
+// reloads its own afterwards).  The result is valid in wave 0; contains barriers.
 template <typename T, int V, int U, bool FULL>
 __device__ __forceinline__ float2 plane_sums_alone(const T* xr, const T* dr, float mean, float rstd, int S, int n_vec,
                                                    int chunk_vec, Pack<T, V> (&rx)[U], Pack<T, V> (&rd)[U],
-                                                   float2 (&sum_buf)[2][16], float (&fb)[kPlaneMaxChunks][2]) {
+                                                   float2 (&sum_buf)[2][16], float (&fb)[kPlaneMaxChunks][2],
+                                                   int (&have)[kPlaneMaxChunks], cl_word* pairs, unsigned tag) {
   const int lane = threadIdx.x & (kWave - 1);
-  __syncthreads();  // fb and the block sums of whatever came before have been read
+  plane_look(pairs, S, tag, have, fb);  // (only the chunks whose pairs have not arrived: see there)
+  int it = 0;
   for (int l = 0; l < S; ++l) {
+    if (have[l]) continue;  // uniform
     const int n_l = plane_chunk_vectors(l, S, n_vec, chunk_vec);
     const int64_t o = static_cast<int64_t>(l) * chunk_vec * V;
     plane_load<T, V, U, FULL, true>(xr + o, n_l, rx);
     plane_load<T, V, U, FULL, true>(dr + o, n_l, rd);
-    const float2 t = plane_chunk_sums<T, V, U, FULL>(rx, rd, n_l, mean, rstd, sum_buf[l & 1]);
+    const float2 t = plane_chunk_sums<T, V, U, FULL>(rx, rd, n_l, mean, rstd, sum_buf[it++ & 1]);
     if (threadIdx.x == 0) {
       fb[l][0] = t.x;
       fb[l][1] = t.y;
+      cl_publish(pairs + 2 * l, t.x, t.y, tag);
     }
   }
   __syncthreads();
@@ -315,6 +355,7 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
                  unsigned tag, int max_polls, PlaneFold fold) {
   __shared__ float2 sum_buf[2][16];
   __shared__ float fb[kPlaneMaxChunks][2];
+  __shared__ int have[kPlaneMaxChunks];
   __shared__ float inst[kWave][2];
   __shared__ float sm_s1, sm_s2;
   __shared__ int sm_fail, sm_fail_fold;
@@ -358,7 +399,8 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
   __syncthreads();
   if (sm_fail) {
     // On its own (see the forward): dy and x are intact, dx != dy.
-    const float2 t = plane_sums_alone<T, V, U, FULL>(xr, dr, mean, rstd, S, n_vec, chunk_vec, rx, rd, sum_buf, fb);
+    const float2 t = plane_sums_alone<T, V, U, FULL>(xr, dr, mean, rstd, S, n_vec, chunk_vec, rx, rd, sum_buf, fb,
+                                                     have, tagged + g.row * S * 2, tag);
     if (threadIdx.x == 0) {
       sm_s1 = t.x;
       sm_s2 = t.y;
@@ -412,7 +454,8 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
       for (int m = 0; m < N; ++m) {
         const int64_t row = static_cast<int64_t>(m) * C + c;
         const float2 t = plane_sums_alone<T, V, U, FULL>(x + row * D, dy + row * D, mean_in[row], rstd_in[row], S,
-                                                         n_vec, chunk_vec, rx, rd, sum_buf, fb);
+                                                         n_vec, chunk_vec, rx, rd, sum_buf, fb, have,
+                                                         tagged + row * S * 2, tag);
         if (threadIdx.x == 0) {
           inst[m][0] = t.y;
           inst[m][1] = t.x;
