@@ -91,6 +91,37 @@ __device__ __forceinline__ bool cl_single_place(int64_t N, int S, int xm_tiles, 
   return unit < N * xm_tiles;
 }
 
+// Start of a workgroup's fallback: which slabs of instance n have published the partials of all
+// the channels of this tile (have[l] = 1)?  One look per (slab, channel), 256 at a time.  The
+// fallback then computes, and publishes for its peers, only the other slabs: when the workgroups
+// of an instance cannot be resident together, the first ones to give up do the missing slabs once
+// and the late ones find everything there, instead of every workgroup redoing the whole instance.
+// Contains barriers; have is valid for every thread afterwards.
+__device__ __forceinline__ void cl_look(const cl_word* tagged, int64_t n, int S, int C, int c_base, int cap_here,
+                                        unsigned tag, int (&have)[kClSingleMaxSlabs]) {
+  __syncthreads();  // whatever read have before is done
+  if (threadIdx.x < kClSingleMaxSlabs) have[threadIdx.x] = 1;
+  __syncthreads();
+  const int lc = threadIdx.x & (kClSingleMaxCap - 1);
+  for (int l = threadIdx.x / kClSingleMaxCap; l < S; l += kClThreads / kClSingleMaxCap) {
+    if (lc < cap_here) {
+      const cl_word* pair = tagged + ((n * S + l) * C + c_base + lc) * 2;
+      const cl_word w0 = cl_peek(pair);
+      const cl_word w1 = cl_peek(pair + 1);
+      if (static_cast<unsigned>(w0 >> 32) != tag || static_cast<unsigned>(w1 >> 32) != ~tag) have[l] = 0;
+    }
+  }
+  __syncthreads();
+}
+// Polls that a workgroup allows for values it has published itself (or has just seen) to show up
+// in its own device-scope loads: they are on their way, this only bounds the wait.
+constexpr int kClOwnPolls = 1 << 16;
+// The wait for such values.  Should they not show up after all, the result is marked (NaN) rather
+// than computed from whatever the words held.
+__device__ __forceinline__ void cl_wait_own(const cl_word* pair, bool want, unsigned tag, float& a, float& b) {
+  if (!cl_wait_pair(pair, want, tag, kClOwnPolls, a, b)) a = b = __builtin_nanf("");
+}
+
 // ------------------------------------------------------------------------------ forward
 // tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std).
 // Grid: see cl_single_place; tile of at most 64 channels.
@@ -106,7 +137,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
               float* __restrict__ rstd_out, int64_t N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
               float eps, unsigned tag, int max_polls, int xm_tiles) {
   __shared__ float lds[V * kClThreads];
-  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap];
+  __shared__ int have[kClSingleMaxSlabs];
   __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
   __shared__ int sm_fail;
   const int CV = C / V;
@@ -178,49 +209,39 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
   }
   __syncthreads();
   if (sm_fail) {
-    // On its own: the partials of every slab of the instance, computed as their workgroups
-    // compute them, folded as their owners fold them.  The slabs pass through the registers of
-    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).  Two
-    // rounds, each for half of the tile's channels: fb holds S x cap / 2 pairs (the LDS this
-    // kernel asks for decides how many workgroups a CU takes, and this path hardly ever runs).
-    const int hw = cap / 2;
-    for (int hf = 0; hf < 2; ++hf) {
-      for (int l = 0; l < S; ++l) {
-        const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
-        cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
-        float mm[V], qq[V];
-        __syncthreads();  // the previous round's block sums (and fold) have been read
-        cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
-        if (g.ch_ok && g.slot == 0) {
-          const int lc0 = g.coff - c_base;
+    // On its own: the partials of every slab of the instance that have not arrived, computed as
+    // their workgroups compute them and published like theirs; then the finals of every channel
+    // of the tile, folded as their owners fold them.  The slabs pass through the registers of
+    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).
+    cl_look(tagged, g.n, S, C, c_base, cap_here, tag, have);
+    for (int l = 0; l < S; ++l) {
+      if (have[l]) continue;  // uniform
+      const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
+      cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
+      float mm[V], qq[V];
+      __syncthreads();  // the previous round's block sums have been read
+      cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
+      if (g.ch_ok && g.slot == 0) {
+        cl_word* o = tagged + ((g.n * S + l) * C + g.coff) * 2;
 #pragma unroll
-          for (int i = 0; i < V; ++i) {
-            const int lh = lc0 + i - hf * hw;
-            if (lh >= 0 && lh < hw) {
-              fb[(l * hw + lh) * 2] = mm[i];
-              fb[(l * hw + lh) * 2 + 1] = qq[i];
-            }
-          }
-        }
+        for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, mm[i], qq[i], tag);
       }
-      __syncthreads();
-      for (int lc = hf * hw + wave; lc < cap_here && lc < (hf + 1) * hw; lc += kClThreads / kWave) {
-        const int c = c_base + lc;
-        const int lh = lc - hf * hw;
-        const float pm = lane < S ? fb[(lane * hw + lh) * 2] : 0.f;
-        const float pq = lane < S ? fb[(lane * hw + lh) * 2 + 1] : 0.f;
-        float mu, q;
-        cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
-        if (lane == 0) {
-          const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
-          sm_mean[lc] = mu;
-          sm_sc[lc] = gamma[c] * rs;
-          sm_bt[lc] = beta[c];
-          if (lc % S == g.s) {  // an owner still serves its peers
-            cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
-            mean_out[g.n * C + c] = mu;
-            rstd_out[g.n * C + c] = rs;
-          }
+    }
+    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
+      const int c = c_base + lc;
+      float pm, pq;
+      cl_wait_own(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pm, pq);
+      float mu, q;
+      cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
+      if (lane == 0) {
+        const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
+        sm_mean[lc] = mu;
+        sm_sc[lc] = gamma[c] * rs;
+        sm_bt[lc] = beta[c];
+        if (lc % S == g.s) {  // an owner still serves its peers
+          cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
+          mean_out[g.n * C + c] = mu;
+          rstd_out[g.n * C + c] = rs;
         }
       }
     }
@@ -257,7 +278,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
               unsigned tag, int max_polls, int xm_tiles, float* __restrict__ o0, float* __restrict__ o1,
               int64_t o_stride) {
   __shared__ float lds[2 * V * kClThreads];
-  __shared__ float fb[kClSingleMaxSlabs * kClSingleMaxCap * 2];
+  __shared__ int have[kClSingleMaxSlabs];
   __shared__ float sm_mu[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_ca[kClSingleMaxCap], sm_cb[kClSingleMaxCap];
   __shared__ float inst[kClSingleMaxOwned][kWave][2];
   __shared__ int sm_fail, sm_fail_dev;
@@ -343,11 +364,12 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     if (fail && lane == 0) sm_fail = 1;
   }
   __syncthreads();
-  // The sums of every slab of instance n2 for this workgroup's tile, as their workgroups compute
-  // them, into fb[slab][channel][2].  The slabs pass through the registers of the workgroup's own
-  // slab (x and dy are intact: dx aliases neither), which the caller loads again if it still
-  // needs it.
-  auto recompute_instance = [&](int64_t n2) {
+  // On its own, for instance n2 and this workgroup's tile: the sums of every slab that have not
+  // arrived, computed as their workgroups compute them and published like theirs.  The slabs pass
+  // through the registers of the workgroup's own slab (x and dy are intact: dx aliases neither),
+  // which the caller loads again if it still needs it.
+  auto ensure_instance = [&](int64_t n2) {
+    cl_look(tagged, n2, S, C, c_base, cap_here, tag, have);
     float mu2[V], rs2[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) mu2[i] = rs2[i] = 0.f;
@@ -356,6 +378,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       load_f32<V>(rstd_in + n2 * C + g.coff, rs2);
     }
     for (int l = 0; l < S; ++l) {
+      if (have[l]) continue;  // uniform
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, true, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
       cl_load_slab<T, V, U, true, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
@@ -363,22 +386,27 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       __syncthreads();  // the previous round's block sums have been read
       cl_resident_sums<T, V, U>(rx, rd, ok, mu2, rs2, TPP, lds, a2);
       if (g.ch_ok && g.slot == 0) {
-        const int lc0 = g.coff - c_base;
+        cl_word* o = tagged + ((n2 * S + l) * C + g.coff) * 2;
 #pragma unroll
-        for (int i = 0; i < V; ++i) {
-          fb[(l * cap + lc0 + i) * 2] = a2[i];
-          fb[(l * cap + lc0 + i) * 2 + 1] = a2[V + i];
-        }
+        for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, a2[i], a2[V + i], tag);
       }
     }
     __syncthreads();
   };
+  // The sums of channel c of instance n2 from its slabs' sums (all of them are there or on their
+  // way after ensure_instance): a lane per slab, the whole wave must call.
+  auto fold_slabs = [&](int64_t n2, int c, float& b, float& a) {
+    float pb, pa;
+    cl_wait_own(tagged + ((n2 * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pb, pa);
+    b = group_sum<kWave>(lane < S ? pb : 0.f);
+    a = group_sum<kWave>(lane < S ? pa : 0.f);
+  };
   if (sm_fail) {
-    recompute_instance(g.n);
+    ensure_instance(g.n);
     for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
       const int c = c_base + lc;
-      const float b = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2] : 0.f);
-      const float a = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f);
+      float b, a;
+      fold_slabs(g.n, c, b, a);
       if (lane == 0) {
         constants(lc, gamma[c], mean_in[g.n * C + c], rstd_in[g.n * C + c], b, a);
         if (lc % S == g.s) {  // an owner still serves its peers
@@ -442,14 +470,15 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   }
   __syncthreads();
   if (sm_fail_dev) {
-    // every instance's sums for the owned channels, recomputed here
+    // every instance's sums for the owned channels, from its slabs' sums (what has not arrived
+    // of those is computed here)
     for (int n2 = 0; n2 < N; ++n2) {
-      recompute_instance(n2);
+      ensure_instance(n2);
       int k = 0;
       for (int lc = g.s; lc < cap_here; lc += S, ++k) {
         if (wave == 0) {
-          const float b = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2] : 0.f);
-          const float a = group_sum<kWave>(lane < S ? fb[(lane * cap + lc) * 2 + 1] : 0.f);
+          float b, a;
+          fold_slabs(n2, c_base + lc, b, a);
           if (lane == 0) {
             inst[k][n2][0] = b;
             inst[k][n2][1] = a;

@@ -64,13 +64,13 @@ struct Tuning {
   TuneInt cl_single{1};
   TuneInt cl_single_xm{1};  //   also on the XCD-major grid (any batch size, any number of workgroups)
   TuneInt cl_single_occ{1};  //   on that grid, when the launch does not fit the chip: the kernels compiled for more workgroups per CU
-  TuneInt cl_single_polls{2000};
+  TuneInt cl_single_polls{300};
   TuneInt affine_fold{1};      // channel-first backward, a workgroup per plane: dgamma / dbeta folded over the batch in the row kernel
   TuneInt affine_fold_polls{2000};  //   polls before a workgroup recomputes its peers' plane sums (0: at once)
   // channel-first planes too long for a workgroup: the chunks of a plane on the workgroups of one
   // XCD, statistics exchanged while they run, one pass (plane_single_kernels.hip.h); and its polls
   TuneInt plane_single{1};
-  TuneInt plane_single_polls{2000};
+  TuneInt plane_single_polls{500};
   TuneInt plane_nt_min_mb{256};  // forward: non-temporal loads of x from this many MiB (what no cache level retains anyway)
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,

@@ -367,11 +367,11 @@ def test_channels_last_single_launch(coracle, N, C, S, dtype):
         check(alone, "single launch, poll limit 0")
         for n_, a, b in zip(names, normal, alone):
             assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
-        assert L.atexn_set_tuning(b"cl_single_polls", 2000) == 0
+        assert L.atexn_set_tuning(b"cl_single_polls", 300) == 0
         assert L.atexn_set_tuning(b"cl_single", 0) == 0
         check(run(), "two stages")
     finally:
-        L.atexn_set_tuning(b"cl_single_polls", 2000)
+        L.atexn_set_tuning(b"cl_single_polls", 300)
         L.atexn_set_tuning(b"cl_single", 1)
 
 
@@ -537,11 +537,11 @@ def test_channel_first_planes_across_workgroups(coracle, N, C, S, dtype):
         alone = run()
         for n_, a, b in zip(names, normal, alone):
             assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
-        assert L.atexn_set_tuning(b"plane_single_polls", 2000) == 0
+        assert L.atexn_set_tuning(b"plane_single_polls", 500) == 0
         assert L.atexn_set_tuning(b"plane_single", 0) == 0
         check(run(), "two stages")
     finally:
-        L.atexn_set_tuning(b"plane_single_polls", 2000)
+        L.atexn_set_tuning(b"plane_single_polls", 500)
         L.atexn_set_tuning(b"plane_single", 1)
 
 
