@@ -86,6 +86,8 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
       char* w = static_cast<char*>(ws);
       cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
       cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
+      unsigned* claims = reinterpret_cast<unsigned*>(w + p.off_claims);
+      unsigned* trouble = exchange_trouble_word();
       const unsigned tag = next_call_tag();
       const int polls = tuning().cl_single_polls;
       const dim3 sgrid = p.single_xm ? dim3(static_cast<unsigned>(p.xm_grid), 1, 1) : grid;
@@ -96,8 +98,8 @@ int cl_fwd_v(const T* x, const float* gamma, const float* beta, int64_t N, int64
 #define ATEXN_CL_FWD_SINGLE(U_, FULL_)                                                          \
   do {                                                                                          \
     auto fn = occ ? cl_fwd_single<T, V, U_, FULL_, true> : cl_fwd_single<T, V, U_, FULL_, false>; \
-    fn<<<sgrid, kClThreads, 0, st>>>(x, tagged, finals, gamma, beta, y, mean, rstd, N, D, Ci, p.S, \
-                                     p.tpp_shift, p.slab_len, eps, tag, polls, xm_tiles);       \
+    fn<<<sgrid, kClThreads, 0, st>>>(x, tagged, finals, claims, gamma, beta, y, mean, rstd, N, D, Ci, p.S, \
+                                     p.tpp_shift, p.slab_len, eps, tag, polls, xm_tiles, trouble); \
   } while (0)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_FWD_SINGLE(4, true);
@@ -207,6 +209,8 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       cl_word* tagged = reinterpret_cast<cl_word*>(w + p.off_tagged);
       cl_word* finals = reinterpret_cast<cl_word*>(w + p.off_finals);
       cl_word* finals_dev = reinterpret_cast<cl_word*>(w + p.off_finals_dev);
+      unsigned* claims = reinterpret_cast<unsigned*>(w + p.off_claims);
+      unsigned* trouble = exchange_trouble_word();
       const unsigned tag = next_call_tag();
       const int polls = tuning().cl_single_polls;
       const int Ni = static_cast<int>(N);
@@ -226,9 +230,9 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
 #define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
   do {                                                                                          \
     auto fn = occ ? cl_bwd_single<T, V, U_, FULL_, true> : cl_bwd_single<T, V, U_, FULL_, false>; \
-    fn<<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, finals_dev, dx, dgamma, \
+    fn<<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, finals_dev, claims, dx, dgamma, \
                                      dbeta, Ni, D, Ci, p.S, p.tpp_shift, p.slab_len, tag, polls, \
-                                     xm_tiles, o0, o1, o_stride);                               \
+                                     xm_tiles, o0, o1, o_stride, trouble);             \
   } while (0)
       if (cl_slabs_full(p, C, D)) {
         if (p.U == 4) ATEXN_CL_BWD_SINGLE(4, true);

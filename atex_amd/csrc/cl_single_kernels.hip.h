@@ -91,11 +91,17 @@ __device__ __forceinline__ bool cl_single_place(int64_t N, int S, int xm_tiles, 
   return unit < N * xm_tiles;
 }
 
-// Start of a workgroup's fallback: which slabs of instance n have published the partials of all
-// the channels of this tile (have[l] = 1)?  One look per (slab, channel), 256 at a time.  The
-// fallback then computes, and publishes for its peers, only the other slabs: when the workgroups
-// of an instance cannot be resident together, the first ones to give up do the missing slabs once
-// and the late ones find everything there, instead of every workgroup redoing the whole instance.
+// A workgroup's fallback (a wait of its has run out) starts with a look: which slabs of instance n
+// have published the partials of all the channels of this tile (have[l] = 1)?  One look per
+// (slab, channel), 256 at a time.  The missing slabs then get computed, each once, by the
+// workgroups that have given up: round by round a workgroup looks, claims ONE missing slab that
+// nobody has claimed yet (cl_claim_missing: a compare-and-swap of the call's tag into the slab's
+// claim word), computes its partials as the slab's own workgroup would, publishes them and looks
+// again; when nothing is left to claim, whatever is still missing is in the hands of a running
+// workgroup and only has to be waited for.  (When the workgroups of an instance cannot be
+// resident together because another kernel fills part of the chip, the resident ones thus share
+// out the slabs of the absent ones instead of each redoing the whole instance; the absent ones,
+// once started, find everything published, publish their own again with the same bits and go on.)
 // Contains barriers; have is valid for every thread afterwards.
 __device__ __forceinline__ void cl_look(const cl_word* tagged, int64_t n, int S, int C, int c_base, int cap_here,
                                         unsigned tag, int (&have)[kClSingleMaxSlabs]) {
@@ -113,8 +119,30 @@ __device__ __forceinline__ void cl_look(const cl_word* tagged, int64_t n, int S,
   }
   __syncthreads();
 }
-// Polls that a workgroup allows for values it has published itself (or has just seen) to show up
-// in its own device-scope loads: they are on their way, this only bounds the wait.
+// One round of that: -1 when no missing slab is left to claim, else the slab this workgroup is to
+// compute.  claims: the claim words of the instance's slabs for this tile.  Contains barriers.
+__device__ __forceinline__ int cl_claim_missing(unsigned* claims, int S, int s_self, unsigned tag,
+                                                const int (&have)[kClSingleMaxSlabs]) {
+  __shared__ int sm_pick;
+  if (threadIdx.x == 0) {
+    int pick = -1;
+    for (int i = 1; i <= S && pick < 0; ++i) {
+      const int l = (s_self + i) % S;
+      if (have[l]) continue;
+      unsigned cur = __hip_atomic_load(claims + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (cur != tag && __hip_atomic_compare_exchange_strong(claims + l, &cur, tag, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                                             __HIP_MEMORY_SCOPE_AGENT)) {
+        pick = l;
+      }
+    }
+    sm_pick = pick;
+  }
+  __syncthreads();
+  return sm_pick;
+}
+// Polls that a workgroup allows for values that it has published itself, has just seen, or knows
+// to be in the hands of a running workgroup to show up in its device-scope loads: they are on
+// their way, this only bounds the wait.
 constexpr int kClOwnPolls = 1 << 16;
 // The wait for such values.  Should they not show up after all, the result is marked (NaN) rather
 // than computed from whatever the words held.
@@ -122,8 +150,14 @@ __device__ __forceinline__ void cl_wait_own(const cl_word* pair, bool want, unsi
   if (!cl_wait_pair(pair, want, tag, kClOwnPolls, a, b)) a = b = __builtin_nanf("");
 }
 
+// Channel tiles of the launch, on either grid.
+__device__ __forceinline__ int gridDim_tiles(int xm_tiles) {
+  return xm_tiles == 0 ? static_cast<int>(gridDim.z) : xm_tiles;
+}
+
 // ------------------------------------------------------------------------------ forward
-// tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std).
+// tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std);
+// claims: [N][tiles][S] claim words.
 // Grid: see cl_single_place; tile of at most 64 channels.
 // OCC: compiled for four workgroups per CU instead of two (128 VGPRs, a few values in scratch
 // memory): an XCD then has the workgroups of two instances in flight, one loading while the
@@ -132,10 +166,11 @@ __device__ __forceinline__ void cl_wait_own(const cl_word* pair, bool want, unsi
 // a launch that fits the chip anyway loses a little (config 3: 9.97 -> 10.4 us) and keeps OCC off.
 template <typename T, int V, int U, bool FULL, bool OCC>
 __global__ void __launch_bounds__(kClThreads, OCC ? 4 : 2)
-cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const float* __restrict__ gamma,
+cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigned* claims,
+              const float* __restrict__ gamma,
               const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
               float* __restrict__ rstd_out, int64_t N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
-              float eps, unsigned tag, int max_polls, int xm_tiles) {
+              float eps, unsigned tag, int max_polls, int xm_tiles, unsigned* trouble) {
   __shared__ float lds[V * kClThreads];
   __shared__ int have[kClSingleMaxSlabs];
   __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
@@ -177,8 +212,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
     for (int lc = g.s; lc < cap_here; lc += S) {
       const int c = c_base + lc;
       float pm, pq;
-      if (!cl_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls,
-                        pm, pq)) {
+      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, trouble, pm, pq)) {
         fail = true;
         break;
       }
@@ -195,7 +229,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
     if (!fail) {
       float fm, frs;
       const bool want = lane < cap_here;
-      if (cl_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, fm, frs)) {
+      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, trouble, fm, frs)) {
         if (want) {
           sm_mean[lane] = fm;
           sm_sc[lane] = gmc * frs;
@@ -213,13 +247,14 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, const f
     // their workgroups compute them and published like theirs; then the finals of every channel
     // of the tile, folded as their owners fold them.  The slabs pass through the registers of
     // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).
-    cl_look(tagged, g.n, S, C, c_base, cap_here, tag, have);
-    for (int l = 0; l < S; ++l) {
-      if (have[l]) continue;  // uniform
+    unsigned* my_claims = claims + (g.n * gridDim_tiles(xm_tiles) + g.ct) * S;
+    for (int round = 0; round < S; ++round) {
+      cl_look(tagged, g.n, S, C, c_base, cap_here, tag, have);
+      const int l = cl_claim_missing(my_claims, S, g.s, tag, have);
+      if (l < 0) break;  // uniform
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
       float mm[V], qq[V];
-      __syncthreads();  // the previous round's block sums have been read
       cl_resident_stats<T, V, U>(raw, ok, 1.0f / static_cast<float>(h.p1 - h.p0), TPP, lds, mm, qq);
       if (g.ch_ok && g.slot == 0) {
         cl_word* o = tagged + ((g.n * S + l) * C + g.coff) * 2;
@@ -273,10 +308,10 @@ template <typename T, int V, int U, bool FULL, bool OCC>
 __global__ void __launch_bounds__(kClThreads, OCC ? 3 : 2)
 cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
               const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
-              cl_word* finals, cl_word* finals_dev, T* __restrict__ dx, float* __restrict__ dgamma,
+              cl_word* finals, cl_word* finals_dev, unsigned* claims, T* __restrict__ dx, float* __restrict__ dgamma,
               float* __restrict__ dbeta, int N, int64_t D, int C, int S, int tpp_shift, int64_t slab_len,
               unsigned tag, int max_polls, int xm_tiles, float* __restrict__ o0, float* __restrict__ o1,
-              int64_t o_stride) {
+              int64_t o_stride, unsigned* trouble) {
   __shared__ float lds[2 * V * kClThreads];
   __shared__ int have[kClSingleMaxSlabs];
   __shared__ float sm_mu[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_ca[kClSingleMaxCap], sm_cb[kClSingleMaxCap];
@@ -335,8 +370,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     for (int lc = g.s; lc < cap_here; lc += S) {
       const int c = c_base + lc;
       float pb, pa;
-      if (!cl_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls,
-                        pb, pa)) {
+      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, trouble, pb, pa)) {
         fail = true;
         break;
       }
@@ -355,7 +389,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     if (!fail) {
       float fb_, fa_;
       const bool want = lane < cap_here;
-      if (cl_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, fb_, fa_)) {
+      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, trouble, fb_, fa_)) {
         if (want) constants(lane, gmc, muc, rsc, fb_, fa_);
       } else {
         fail = true;
@@ -369,7 +403,6 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   // through the registers of the workgroup's own slab (x and dy are intact: dx aliases neither),
   // which the caller loads again if it still needs it.
   auto ensure_instance = [&](int64_t n2) {
-    cl_look(tagged, n2, S, C, c_base, cap_here, tag, have);
     float mu2[V], rs2[V];
 #pragma unroll
     for (int i = 0; i < V; ++i) mu2[i] = rs2[i] = 0.f;
@@ -377,13 +410,15 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       load_f32<V>(mean_in + n2 * C + g.coff, mu2);
       load_f32<V>(rstd_in + n2 * C + g.coff, rs2);
     }
-    for (int l = 0; l < S; ++l) {
-      if (have[l]) continue;  // uniform
+    unsigned* my_claims = claims + (n2 * gridDim_tiles(xm_tiles) + g.ct) * S;
+    for (int round = 0; round < S; ++round) {
+      cl_look(tagged, n2, S, C, c_base, cap_here, tag, have);
+      const int l = cl_claim_missing(my_claims, S, g.s, tag, have);
+      if (l < 0) break;  // uniform
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, true, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
       cl_load_slab<T, V, U, true, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
       float a2[2 * V];
-      __syncthreads();  // the previous round's block sums have been read
       cl_resident_sums<T, V, U>(rx, rd, ok, mu2, rs2, TPP, lds, a2);
       if (g.ch_ok && g.slot == 0) {
         cl_word* o = tagged + ((n2 * S + l) * C + g.coff) * 2;
@@ -454,6 +489,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       const int c = c_base + lc;
       float pb = eb, pa = ea;
       if (!(early && lc == g.s) &&
+          // (patiently in any case: the other instances do not depend on this workgroup)
           !cl_wait_pair(finals_dev + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2, lane < N, tag,
                         max_polls, pb, pa)) {
         fail = true;

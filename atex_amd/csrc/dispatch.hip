@@ -61,6 +61,32 @@ bool exchange_allowed(void* st) {
   return status == hipStreamCaptureStatusNone;
 }
 
+namespace {
+// tag of the last call on this device in which a patient wait for a peer's results ran out
+__device__ unsigned g_exchange_trouble;
+}  // namespace
+
+unsigned* exchange_trouble_word() {
+  static std::atomic<unsigned*> cached[64];
+  static std::atomic<bool> failed[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) {
+    (void)hipGetLastError();
+    return nullptr;
+  }
+  unsigned* p = cached[dev].load(std::memory_order_acquire);
+  if (p != nullptr || failed[dev].load(std::memory_order_relaxed)) return p;
+  void* q = nullptr;
+  if (hipGetSymbolAddress(&q, HIP_SYMBOL(g_exchange_trouble)) != hipSuccess || q == nullptr) {
+    (void)hipGetLastError();
+    failed[dev].store(true, std::memory_order_relaxed);
+    return nullptr;
+  }
+  // (racing threads look the same address up: the stores agree)
+  cached[dev].store(static_cast<unsigned*>(q), std::memory_order_release);
+  return static_cast<unsigned*>(q);
+}
+
 int cu_count() {
   static std::atomic<int> cached[64];
   int dev = 0;

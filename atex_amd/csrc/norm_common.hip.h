@@ -422,6 +422,39 @@ __device__ __forceinline__ bool cl_wait_pair(const cl_word* pair, bool want, uns
   return false;
 }
 
+// How patient the waits of a call are.  The kernels whose workgroups exchange results need the
+// workgroups of one instance / plane resident together; where another kernel fills whole CUs they
+// never are, every wait runs out, and what costs the time is the waiting (the workgroups that give
+// up do the missing work between them).  `trouble` is a word of device memory that holds the tag
+// of the last call in which a patient wait ran out.  A wait polls kExchangeHastyPolls times
+// first, which is mostly enough when the peers are resident; only then does it read the word (a
+// call on a GPU of its own seldom touches it).  For kExchangeTroubleCalls calls after the one
+// recorded there it gives up at once, which costs a little redundant work when the peers were
+// merely slow; after that a call waits patiently again and finds out whether the GPU is still
+// shared.  Results do not depend on any of this (whatever a workgroup computes for a peer has the
+// peer's bits).
+constexpr int kExchangePatientPolls = 100;  // poll limits from here on count as patient
+constexpr int kExchangeHastyPolls = 24;
+constexpr unsigned kExchangeTroubleCalls = 256;
+// cl_wait_pair under that rule.  All 64 lanes of the wave must call it; the result is the same
+// in all of them.  trouble == nullptr or a limit below kExchangePatientPolls: the plain wait.
+__device__ __forceinline__ bool exchange_wait_pair(const cl_word* pair, bool want, unsigned tag, int max_polls,
+                                                   unsigned* trouble, float& a, float& b) {
+  a = b = 0.f;
+  const bool adaptive = trouble != nullptr && max_polls >= kExchangePatientPolls;
+  for (int poll = 0; poll < max_polls; ++poll) {
+    if (cl_try_pair(pair, want, tag, a, b)) return true;
+    if (adaptive && poll == kExchangeHastyPolls - 1) {
+      const unsigned seen = __hip_atomic_load(trouble, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (tag - seen < kExchangeTroubleCalls) return false;
+    }
+  }
+  if (adaptive && (threadIdx.x & (kWave - 1)) == 0) {
+    __hip_atomic_store(trouble, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  return false;
+}
+
 // Loops over strided indices are written in batches of B whose loads are all issued before
 // the first is consumed: the compiler does not move a load above the bounds check of the
 // iteration before it, so a plain loop would pay one memory latency per iteration.

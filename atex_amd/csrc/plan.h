@@ -147,6 +147,7 @@ struct RowsPlan {
   int ps_S = 0, ps_chunk_vec = 0, ps_grid = 0;
   bool ps_full = false;  // every thread of every workgroup holds 8 vectors
   size_t off_ps_tagged = 0;
+  size_t off_ps_claims = 0;  // a word per chunk: who computes it when its workgroup is not there
   // backward: the planes' sums folded over the batch inside the kernel (tagged pairs per plane at
   // off_ps_fold) instead of by a col_reduce launch: the planes of a channel must share an XCD (C a
   // multiple of the XCD count, or a single instance), at most 64 instances
@@ -260,6 +261,8 @@ inline void plan_plane_single(RowsPlan& p, RowsKind kind, int V, int64_t n_rows,
       p.ps_full = n_vec % S2 == 0 && p.ps_chunk_vec == per_wg;
       p.off_ps_tagged = bytes;
       bytes += align256(size_t(16) * size_t(n_rows) * size_t(S2));
+      p.off_ps_claims = bytes;
+      bytes += align256(size_t(4) * size_t(n_rows) * size_t(S2));
       if (kind == RowsKind::kBwdAffine && t.affine_fold && p.part_rows <= 64 &&
           (C % kPlanXcdCount == 0 || p.part_rows == 1)) {
         p.ps_fold = true;
@@ -550,6 +553,7 @@ struct ClPlan {
   // fallback, in the same workspace.
   bool single = false;
   size_t off_tagged = 0, off_finals = 0, off_finals_dev = 0;
+  size_t off_claims = 0;  // a word per (instance, tile, slab): who computes it when its workgroup is not there
   // The same kernels on a one-dimensional XCD-major grid (cl_single_place) for launches that do
   // not meet the conditions on N and on the number of workgroups: any batch size, any number of
   // instances; an instance's slabs must fit one XCD (two workgroups per CU).  The backward then
@@ -715,7 +719,8 @@ inline ClPlan plan_cl_with(bool bwd, int V, int64_t N, int64_t C, int64_t D, int
     p.off_tagged = 0;
     p.off_finals = align256(size_t(16) * size_t(N) * size_t(p.S) * size_t(C));
     p.off_finals_dev = p.off_finals + align256(size_t(16) * size_t(N) * size_t(C));
-    p.ws_bytes = std::max(p.ws_bytes, p.off_finals_dev + align256(size_t(16) * size_t(N) * size_t(C)));
+    p.off_claims = p.off_finals_dev + align256(size_t(16) * size_t(N) * size_t(C));
+    p.ws_bytes = std::max(p.ws_bytes, p.off_claims + align256(size_t(4) * size_t(N) * size_t(p.CT) * size_t(p.S)));
     if (p.single_xm) {  // (the finals_dev section is not used; the per-instance sums take its place)
       p.off_xm_part = p.off_finals_dev;
     }

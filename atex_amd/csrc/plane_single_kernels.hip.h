@@ -154,31 +154,65 @@ __device__ __forceinline__ void plane_merge_stats(float pm, float pq, int lane, 
   m2 = group_sum<kWave>(in ? pq + w * (d * d) : 0.f);
 }
 
-// Start of a workgroup's fallback: wave 0 looks once, a lane per chunk, at the pairs of the plane
-// at `pairs`, keeps those that have arrived in fb and notes which have (have[l]); the fallback
-// then computes, and publishes for its peers, only the others.  (When the workgroups of a plane
-// cannot be resident together, the first ones to give up thus do the missing chunks once, and
-// the late ones find everything there, instead of every workgroup redoing the whole plane.)
-// Contains a barrier; have / fb are valid for every thread afterwards.
-__device__ __forceinline__ void plane_look(const cl_word* pairs, int S, unsigned tag, int (&have)[kPlaneMaxChunks],
-                                           float (&fb)[kPlaneMaxChunks][2]) {
-  __syncthreads();  // whatever read have / fb before is done
+// A workgroup's fallback (its wait for the pairs of a plane has run out): the chunks whose pairs
+// are missing get computed, each once, by the workgroups that have given up.  Round by round a
+// workgroup looks, a lane per chunk, at what has arrived (plane_look), claims ONE missing chunk
+// that nobody has claimed yet (a compare-and-swap on the chunk's claim word: the call's tag),
+// computes its pair as the chunk's own workgroup would, publishes it, and looks again; when
+// nothing is left to claim, whatever is still missing is in the hands of a running workgroup
+// and only has to be waited for.  (When the workgroups of a plane cannot be resident together
+// because another kernel fills part of the chip, the resident ones thus share out the chunks of
+// the absent ones instead of each redoing the whole plane; the absent ones, once started, find
+// their pairs published, publish them again with the same bits and go on.)
+__device__ __forceinline__ void plane_look(const cl_word* pairs, int S, unsigned tag, int (&have)[kPlaneMaxChunks]) {
+  __syncthreads();  // whatever read have before is done
   if (threadIdx.x < kWave) {
     const int lane = threadIdx.x;
     bool ok = false;
-    float a = 0.f, b = 0.f;
     if (lane < S) {
       const cl_word w0 = cl_peek(pairs + 2 * lane);
       const cl_word w1 = cl_peek(pairs + 2 * lane + 1);
       ok = static_cast<unsigned>(w0 >> 32) == tag && static_cast<unsigned>(w1 >> 32) == ~tag;
-      a = __builtin_bit_cast(float, static_cast<unsigned>(w0));
-      b = __builtin_bit_cast(float, static_cast<unsigned>(w1));
     }
     have[lane] = ok ? 1 : 0;
-    fb[lane][0] = a;
-    fb[lane][1] = b;
   }
   __syncthreads();
+}
+__device__ __forceinline__ bool plane_try_claim(unsigned* word, unsigned tag) {
+  unsigned cur = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if (cur == tag) return false;
+  return __hip_atomic_compare_exchange_strong(word, &cur, tag, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+                                              __HIP_MEMORY_SCOPE_AGENT);
+}
+// compute(l) returns the pair of chunk l in every thread (it contains barriers and is called by
+// the whole workgroup).  s_self: where this workgroup starts looking for a chunk to claim.
+template <typename F>
+__device__ __forceinline__ void plane_fill_missing(cl_word* pairs, unsigned* claims, int S, int s_self, unsigned tag,
+                                                   int (&have)[kPlaneMaxChunks], F&& compute) {
+  __shared__ int sm_pick;
+  for (int round = 0; round < S; ++round) {
+    plane_look(pairs, S, tag, have);
+    if (threadIdx.x == 0) {
+      int pick = -1;
+      for (int i = 1; i <= S && pick < 0; ++i) {
+        const int l = (s_self + i) % S;
+        if (!have[l] && plane_try_claim(claims + l, tag)) pick = l;
+      }
+      sm_pick = pick;
+    }
+    __syncthreads();
+    const int l = sm_pick;
+    if (l < 0) break;  // uniform
+    const float2 t = compute(l);
+    if (threadIdx.x == 0) cl_publish(pairs + 2 * l, t.x, t.y, tag);
+  }
+}
+// Polls that a workgroup allows for pairs that are in the hands of running workgroups (or its
+// own) to show up: they are on their way, this only bounds the wait.  Should they not show up
+// after all, the result is marked (NaN) rather than computed from whatever the words held.
+constexpr int kPlaneOwnPolls = 1 << 16;
+__device__ __forceinline__ void plane_wait_own(const cl_word* pair, bool want, unsigned tag, float& a, float& b) {
+  if (!cl_wait_pair(pair, want, tag, kPlaneOwnPolls, a, b)) a = b = __builtin_nanf("");
 }
 
 // ------------------------------------------------------------------------------ forward
@@ -187,12 +221,11 @@ __device__ __forceinline__ void plane_look(const cl_word* pairs, int S, unsigned
 // anyway; the fallback then keeps a few values in scratch memory)
 template <typename T, int V, int U, bool FULL, bool NT>
 __global__ void __launch_bounds__(kPlaneThreads, FULL ? 8 : 4)
-plane_fwd_single(const T* __restrict__ x, cl_word* tagged, const float* __restrict__ gamma,
+plane_fwd_single(const T* __restrict__ x, cl_word* tagged, unsigned* claims, const float* __restrict__ gamma,
                  const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
                  float* __restrict__ rstd_out, int64_t n_rows, int n_vec, int S, int chunk_vec, int C, float eps,
-                 unsigned tag, int max_polls) {
+                 unsigned tag, int max_polls, unsigned* trouble) {
   __shared__ Wf wf_buf[2][16];
-  __shared__ float fb[kPlaneMaxChunks][2];
   __shared__ int have[kPlaneMaxChunks];
   __shared__ float sm_mean, sm_rstd;
   __shared__ int sm_fail;
@@ -217,7 +250,7 @@ plane_fwd_single(const T* __restrict__ x, cl_word* tagged, const float* __restri
   for (int k = 0; k < U; ++k) forget_derived(raw[k]);
   if (wave == 0) {
     float pm, pq;
-    if (cl_wait_pair(tagged + (g.row * S + (lane < S ? lane : 0)) * 2, lane < S, tag, max_polls, pm, pq)) {
+    if (exchange_wait_pair(tagged + (g.row * S + (lane < S ? lane : 0)) * 2, lane < S, tag, max_polls, trouble, pm, pq)) {
       float mu, q;
       plane_merge_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
       if (lane == 0) {
@@ -230,28 +263,19 @@ plane_fwd_single(const T* __restrict__ x, cl_word* tagged, const float* __restri
   }
   __syncthreads();
   if (sm_fail) {
-    // On its own: the pair of every chunk of the plane that has not arrived, computed as its
-    // workgroup computes it (and published: the workgroup may turn up late, its peers may be
-    // looking).  The chunks pass through the registers of the workgroup's own chunk, which is
-    // loaded again at the end (x is intact: y != x).
-    plane_look(tagged + g.row * S * 2, S, tag, have, fb);
+    // See plane_fill_missing.  The chunks pass through the registers of the workgroup's own
+    // chunk, which is loaded again at the end (x is intact: y != x).
     int it = 1;
-    for (int l = 0; l < S; ++l) {
-      if (have[l]) continue;  // uniform
+    plane_fill_missing(tagged + g.row * S * 2, claims + g.row * S, S, g.s, tag, have, [&](int l) {
       const int n_l = plane_chunk_vectors(l, S, n_vec, chunk_vec);
       plane_load<T, V, U, FULL, NT>(xr + static_cast<int64_t>(l) * chunk_vec * V, n_l, raw);
       const Wf w = plane_chunk_stats<T, V, U, FULL>(raw, n_l, wf_buf[it++ & 1]);
-      if (threadIdx.x == 0) {
-        fb[l][0] = w.mean;
-        fb[l][1] = w.m2;
-        cl_publish(tagged + (g.row * S + l) * 2, w.mean, w.m2, tag);
-      }
-    }
-    __syncthreads();
+      return make_float2(w.mean, w.m2);
+    });
     if (wave == 0) {
-      float mu, q;
-      plane_merge_stats(lane < S ? fb[lane][0] : 0.f, lane < S ? fb[lane][1] : 0.f, lane, S, n_full, n_last, inv_d,
-                        mu, q);
+      float pm, pq, mu, q;
+      plane_wait_own(tagged + (g.row * S + (lane < S ? lane : 0)) * 2, lane < S, tag, pm, pq);
+      plane_merge_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
       if (lane == 0) {
         sm_mean = mu;
         sm_rstd = rsqrtf(__builtin_fmaf(q, inv_d, eps));
@@ -300,34 +324,28 @@ __device__ __forceinline__ float2 plane_chunk_sums(const Pack<T, V> (&rx)[U], co
   return block_sum2(s1, s2 * rstd, buf, kPlaneThreads / kWave);
 }
 
-// (sum dy, sum dy * xh) of a whole plane computed by the calling workgroup alone: the pair of
-// every chunk, as found at `pairs` or else computed as its workgroup computes it (and published
-// there), added up as the gathering wave adds them.  The chunks pass through rx / rd (the caller
-// reloads its own afterwards).  The result is valid in wave 0; contains barriers.
+// (sum dy, sum dy * xh) of a whole plane when the wait for its chunks' pairs has run out: what is
+// missing gets computed (plane_fill_missing; the chunks pass through rx / rd, the caller reloads
+// its own afterwards), then the pairs are added up as the gathering wave adds them.  The result
+// is valid in wave 0; contains barriers.
 template <typename T, int V, int U, bool FULL>
-__device__ __forceinline__ float2 plane_sums_alone(const T* xr, const T* dr, float mean, float rstd, int S, int n_vec,
-                                                   int chunk_vec, Pack<T, V> (&rx)[U], Pack<T, V> (&rd)[U],
-                                                   float2 (&sum_buf)[2][16], float (&fb)[kPlaneMaxChunks][2],
-                                                   int (&have)[kPlaneMaxChunks], cl_word* pairs, unsigned tag) {
+__device__ __forceinline__ float2 plane_sums_alone(const T* xr, const T* dr, float mean, float rstd, int S, int s_self,
+                                                   int n_vec, int chunk_vec, Pack<T, V> (&rx)[U], Pack<T, V> (&rd)[U],
+                                                   float2 (&sum_buf)[2][16], int (&have)[kPlaneMaxChunks],
+                                                   cl_word* pairs, unsigned* claims, unsigned tag) {
   const int lane = threadIdx.x & (kWave - 1);
-  plane_look(pairs, S, tag, have, fb);  // (only the chunks whose pairs have not arrived: see there)
   int it = 0;
-  for (int l = 0; l < S; ++l) {
-    if (have[l]) continue;  // uniform
+  plane_fill_missing(pairs, claims, S, s_self, tag, have, [&](int l) {
     const int n_l = plane_chunk_vectors(l, S, n_vec, chunk_vec);
     const int64_t o = static_cast<int64_t>(l) * chunk_vec * V;
     plane_load<T, V, U, FULL, true>(xr + o, n_l, rx);
     plane_load<T, V, U, FULL, true>(dr + o, n_l, rd);
-    const float2 t = plane_chunk_sums<T, V, U, FULL>(rx, rd, n_l, mean, rstd, sum_buf[it++ & 1]);
-    if (threadIdx.x == 0) {
-      fb[l][0] = t.x;
-      fb[l][1] = t.y;
-      cl_publish(pairs + 2 * l, t.x, t.y, tag);
-    }
-  }
-  __syncthreads();
-  const float a = group_sum<kWave>(lane < S ? fb[lane < S ? lane : 0][0] : 0.f);
-  const float b = group_sum<kWave>(lane < S ? fb[lane < S ? lane : 0][1] : 0.f);
+    return plane_chunk_sums<T, V, U, FULL>(rx, rd, n_l, mean, rstd, sum_buf[it++ & 1]);
+  });
+  float pa = 0.f, pb = 0.f;
+  if (threadIdx.x < kWave) plane_wait_own(pairs + 2 * (lane < S ? lane : 0), lane < S, tag, pa, pb);
+  const float a = group_sum<kWave>(lane < S ? pa : 0.f);
+  const float b = group_sum<kWave>(lane < S ? pb : 0.f);
   return make_float2(a, b);
 }
 
@@ -351,10 +369,9 @@ template <typename T, int V, int U, bool FULL>
 __global__ void __launch_bounds__(kPlaneThreads, 4)
 plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
                  const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
-                 T* __restrict__ dx, float* __restrict__ part, int64_t n_rows, int n_vec, int S, int chunk_vec, int C,
-                 unsigned tag, int max_polls, PlaneFold fold) {
+                 unsigned* claims, T* __restrict__ dx, float* __restrict__ part, int64_t n_rows, int n_vec, int S, int chunk_vec, int C,
+                 unsigned tag, int max_polls, PlaneFold fold, unsigned* trouble) {
   __shared__ float2 sum_buf[2][16];
-  __shared__ float fb[kPlaneMaxChunks][2];
   __shared__ int have[kPlaneMaxChunks];
   __shared__ float inst[kWave][2];
   __shared__ float sm_s1, sm_s2;
@@ -385,7 +402,7 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
   }
   if (wave == 0) {
     float pa, pb;
-    if (cl_wait_pair(tagged + (g.row * S + (lane < S ? lane : 0)) * 2, lane < S, tag, max_polls, pa, pb)) {
+    if (exchange_wait_pair(tagged + (g.row * S + (lane < S ? lane : 0)) * 2, lane < S, tag, max_polls, trouble, pa, pb)) {
       const float a = group_sum<kWave>(lane < S ? pa : 0.f);
       const float b = group_sum<kWave>(lane < S ? pb : 0.f);
       if (lane == 0) {
@@ -399,8 +416,8 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
   __syncthreads();
   if (sm_fail) {
     // On its own (see the forward): dy and x are intact, dx != dy.
-    const float2 t = plane_sums_alone<T, V, U, FULL>(xr, dr, mean, rstd, S, n_vec, chunk_vec, rx, rd, sum_buf, fb,
-                                                     have, tagged + g.row * S * 2, tag);
+    const float2 t = plane_sums_alone<T, V, U, FULL>(xr, dr, mean, rstd, S, g.s, n_vec, chunk_vec, rx, rd, sum_buf,
+                                                     have, tagged + g.row * S * 2, claims + g.row * S, tag);
     if (threadIdx.x == 0) {
       sm_s1 = t.x;
       sm_s2 = t.y;
@@ -444,6 +461,7 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
     bool ok = false;
     float pb = 0.f, pa = 0.f;
     if (wave == 0) {
+      // (patiently in any case: the planes waited for belong to workgroups started long ago)
       ok = cl_wait_pair(fold.tagged + (static_cast<int64_t>(lane < N ? lane : 0) * C + c) * 2, lane < N, tag, max_polls,
                         pb, pa);
       if (lane == 0 && !ok) sm_fail_fold = 1;
@@ -454,8 +472,8 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
       for (int m = 0; m < N; ++m) {
         const int64_t row = static_cast<int64_t>(m) * C + c;
         const float2 t = plane_sums_alone<T, V, U, FULL>(x + row * D, dy + row * D, mean_in[row], rstd_in[row], S,
-                                                         n_vec, chunk_vec, rx, rd, sum_buf, fb, have,
-                                                         tagged + row * S * 2, tag);
+                                                         g.s, n_vec, chunk_vec, rx, rd, sum_buf, have,
+                                                         tagged + row * S * 2, claims + row * S, tag);
         if (threadIdx.x == 0) {
           inst[m][0] = t.y;
           inst[m][1] = t.x;

@@ -164,8 +164,10 @@ int rows_fwd_v(const T* x, const float* gamma, const float* beta, int64_t n_rows
       const bool nt = n_rows * D * int64_t(sizeof(T)) >= int64_t(tuning().plane_nt_min_mb) << 20;
       auto fn = p.ps_full ? (nt ? plane_fwd_single<T, V, kPlanPlaneVpt, true, true> : plane_fwd_single<T, V, kPlanPlaneVpt, true, false>)
                           : (nt ? plane_fwd_single<T, V, kPlanPlaneVpt, false, true> : plane_fwd_single<T, V, kPlanPlaneVpt, false, false>);
-      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(x, tagged, gamma, beta, y, mean, rstd, n_rows, n_vec, p.ps_S,
-                                              p.ps_chunk_vec, C, eps, next_call_tag(), tuning().plane_single_polls);
+      unsigned* claims = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + p.off_ps_claims);
+      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(x, tagged, claims, gamma, beta, y, mean, rstd, n_rows, n_vec, p.ps_S,
+                                              p.ps_chunk_vec, C, eps, next_call_tag(), tuning().plane_single_polls,
+                                              exchange_trouble_word());
       ATEXN_CHECK_LAUNCH("plane_fwd_single");
       return ATEXN_OK;
     }
@@ -359,8 +361,10 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
       auto fn = p.ps_full ? plane_bwd_single<T, V, kPlanPlaneVpt, true> : plane_bwd_single<T, V, kPlanPlaneVpt, false>;
       PlaneFold pf{nullptr, dgamma, dbeta, p.part_rows};
       if (p.ps_fold) pf.tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_fold);
-      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, dx, part, n_rows, n_vec, p.ps_S,
-                                              p.ps_chunk_vec, C, next_call_tag(), tuning().plane_single_polls, pf);
+      unsigned* claims = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + p.off_ps_claims);
+      fn<<<p.ps_grid, kPlaneThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, claims, dx, part, n_rows, n_vec, p.ps_S,
+                                              p.ps_chunk_vec, C, next_call_tag(), tuning().plane_single_polls, pf,
+                                              exchange_trouble_word());
       ATEXN_CHECK_LAUNCH("plane_bwd_single");
       if (p.ps_fold) return ATEXN_OK;
       return launch_col_reduce(part, dgamma, dbeta, p.part_rows, W, st);

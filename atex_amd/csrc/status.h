@@ -30,6 +30,11 @@ unsigned next_call_tag();
 // The results are the same; the time is not.  The variable is read once, at the first call.
 bool exchange_allowed(void* st);
 
+// The current device's word for exchange_polls / exchange_gave_up (norm_common.hip.h): a static
+// device variable of the library, looked up once per device.  nullptr if that fails (the kernels
+// then always wait patiently).
+unsigned* exchange_trouble_word();
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 
 #define ATEXN_REQUIRE(cond, ...)                                                  \

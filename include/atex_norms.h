@@ -23,15 +23,17 @@
  *   - the saved statistics are the mean and the INVERSE STANDARD DEVIATION
  *     rsqrt(biased_variance + epsilon) (reference: cc/kernels/norm_util.h:253-258);
  *   - `stream` is a hipStream_t passed as void* (NULL = the default stream); every call is
- *     asynchronous on it, re-entrant, allocates nothing and keeps no device state
- *     (atexn_layer_norm_bwd_static is the one exception, see there); the library has no
+ *     asynchronous on it, re-entrant, allocates nothing and keeps no device state that a
+ *     result depends on (atexn_layer_norm_bwd_static is the one exception, see there; besides,
+ *     one 4-byte word per device remembers the last call whose workgroups waited for each other
+ *     in vain, and only makes the next calls give such waits up sooner); the library has no
  *     process-wide settings: launch plans depend on the sizes and the device alone.  One
  *     environment variable is read, once, at the first call: ATEXN_NO_EXCHANGE=1 keeps every
  *     InstanceNorm call on kernels that need no group of workgroups resident on the GPU
  *     together (two launches per direction instead of one for some shapes; same results up to
  *     the order of a few float32 additions in the statistics, same workspace sizes) -- for
  *     processes that keep other kernels running on the same GPU all the time, under which
- *     the one-launch kernels are correct but many times slower;
+ *     the one-launch kernels are correct but two to four times slower than the two launches;
  *   - the device the stream belongs to must be the calling thread's current device: launch
  *     plans and workspace sizes are made for the current device's compute-unit count;
  *   - data pointers need only the alignment of their element type (2 or 4 bytes): the

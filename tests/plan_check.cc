@@ -89,10 +89,13 @@ static void check_rows(RowsKind kind, bool layer_norm, int vec, int64_t n_rows, 
                p.ws_bytes >= p.off_ps_tagged + size_t(16) * size_t(n_rows) * size_t(p.ps_S),
            "plane single: workspace");
     if (kind == RowsKind::kBwdAffine) EXPECT(p.off_ps_tagged >= p.off_part + sizeof(float) * 2 * size_t(n_rows), "plane single: tagged pairs over the plane sums");
+    EXPECT(p.off_ps_claims % 256 == 0 && p.off_ps_claims >= p.off_ps_tagged + size_t(16) * size_t(n_rows) * size_t(p.ps_S) &&
+               p.ws_bytes >= p.off_ps_claims + size_t(4) * size_t(n_rows) * size_t(p.ps_S),
+           "plane single: claim words");
     if (p.ps_fold) {
       EXPECT(kind == RowsKind::kBwdAffine && p.part_rows >= 1 && p.part_rows <= 64 && (C % 8 == 0 || p.part_rows == 1),
              "plane fold: N=%d C=%d", p.part_rows, C);
-      EXPECT(p.off_ps_fold % 256 == 0 && p.off_ps_fold >= p.off_ps_tagged + size_t(16) * size_t(n_rows) * size_t(p.ps_S) &&
+      EXPECT(p.off_ps_fold % 256 == 0 && p.off_ps_fold >= p.off_ps_claims + size_t(4) * size_t(n_rows) * size_t(p.ps_S) &&
                  p.ws_bytes >= p.off_ps_fold + size_t(16) * size_t(n_rows),
              "plane fold: workspace");
     }
@@ -251,7 +254,8 @@ static void check_cl(bool bwd, int V, int64_t N, int64_t C, int64_t D, int cus) 
     }
     EXPECT(p.off_tagged % 256 == 0 && p.off_finals >= p.off_tagged + size_t(16) * N * p.S * C &&
                p.off_finals_dev >= p.off_finals + size_t(16) * N * C &&
-               p.ws_bytes >= p.off_finals_dev + size_t(16) * N * C,
+               p.off_claims % 256 == 0 && p.off_claims >= p.off_finals_dev + size_t(16) * N * C &&
+               p.ws_bytes >= p.off_claims + size_t(4) * N * p.CT * p.S,
            "single: workspace sections");
   }
 }
