@@ -23,6 +23,11 @@ int atexn_set_tuning(const char* name, int value);
 int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C, int64_t D,
                              char* out, size_t out_bytes);
 
+/* Writes the current device's record of "the last call whose workgroups waited for each other in
+ * vain": recent != 0 makes it this moment (the exchange kernels of the next 256 calls give a wait
+ * up after a few polls), recent == 0 makes it long ago (patient waits).  Synchronous. */
+int atexn_bench_mark_exchange_trouble(int recent);
+
 #ifdef __cplusplus
 }
 #endif

@@ -293,6 +293,15 @@ int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C
   }
   return n < 0 ? 0 : (static_cast<size_t>(n) < out_bytes ? n : static_cast<int>(out_bytes) - 1);
 }
+
+int atexn_bench_mark_exchange_trouble(int recent) {
+  unsigned* word = exchange_trouble_word();
+  ATEXN_REQUIRE(word != nullptr, "no record of waits on this device");
+  const unsigned value = next_call_tag() - (recent ? 0u : 0x40000000u);
+  const hipError_t e = hipMemcpy(word, &value, sizeof(value), hipMemcpyHostToDevice);
+  if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "hipMemcpy: %s", hipGetErrorString(e));
+  return ATEXN_OK;
+}
 #endif  // ATEXN_BENCH_BUILD
 
 /* ------------------------------------------------------------------ kernel level */

@@ -75,10 +75,11 @@ SIGNATURES = {
     "atexn_fused_instance_norm_grad_workspace_bytes": (_sz, [_tp, ctypes.c_char_p]),
     "atexn_fused_instance_norm_grad": (_i, [_tp, _tp, _tp, _tp, _tp, ctypes.c_char_p, _tp, _tp, _tp, _vp, _sz, _vp]),
 }
-# the two extra entry points of the benchmark build (csrc/bench_hooks.h)
+# the extra entry points of the benchmark build (csrc/bench_hooks.h)
 BENCH_SIGNATURES = {
     "atexn_set_tuning": (_i, [ctypes.c_char_p, _i]),
     "atexn_bench_describe_bwd": (_i, [_i, _i, _i, _i64, _i64, _i64, ctypes.c_char_p, _sz]),
+    "atexn_bench_mark_exchange_trouble": (_i, [_i]),
 }
 BENCH_LIB_PATH = LIB_PATH.replace(".so", "_bench.so")
 _bench_lib = None

@@ -367,12 +367,22 @@ def test_channels_last_single_launch(coracle, N, C, S, dtype):
         check(alone, "single launch, poll limit 0")
         for n_, a, b in zip(names, normal, alone):
             assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
+        for polls in (1, 3, 8):  # some workgroups give up, others find what they wait for
+            assert L.atexn_set_tuning(b"cl_single_polls", polls) == 0
+            for n_, a, b in zip(names, normal, run()):
+                assert torch.equal(_bits(a), _bits(b)), f"poll limit {polls} differs from the normal run in {n_}"
         assert L.atexn_set_tuning(b"cl_single_polls", 300) == 0
+        # as after a call whose waits ran out: the waits of the next calls are cut short
+        assert L.atexn_bench_mark_exchange_trouble(1) == 0
+        for n_, a, b in zip(names, normal, run()):
+            assert torch.equal(_bits(a), _bits(b)), f"short waits differ from the normal run in {n_}"
+        assert L.atexn_bench_mark_exchange_trouble(0) == 0
         assert L.atexn_set_tuning(b"cl_single", 0) == 0
         check(run(), "two stages")
     finally:
         L.atexn_set_tuning(b"cl_single_polls", 300)
         L.atexn_set_tuning(b"cl_single", 1)
+        L.atexn_bench_mark_exchange_trouble(0)
 
 
 def test_channels_last_single_launch_in_place_takes_two_stages(capi, coracle):
@@ -537,12 +547,22 @@ def test_channel_first_planes_across_workgroups(coracle, N, C, S, dtype):
         alone = run()
         for n_, a, b in zip(names, normal, alone):
             assert torch.equal(_bits(a), _bits(b)), f"poll limit 0 differs from the normal run in {n_}"
+        for polls in (1, 3, 8):  # some workgroups give up, others find what they wait for
+            assert L.atexn_set_tuning(b"plane_single_polls", polls) == 0
+            for n_, a, b in zip(names, normal, run()):
+                assert torch.equal(_bits(a), _bits(b)), f"poll limit {polls} differs from the normal run in {n_}"
         assert L.atexn_set_tuning(b"plane_single_polls", 500) == 0
+        # as after a call whose waits ran out: the waits of the next calls are cut short
+        assert L.atexn_bench_mark_exchange_trouble(1) == 0
+        for n_, a, b in zip(names, normal, run()):
+            assert torch.equal(_bits(a), _bits(b)), f"short waits differ from the normal run in {n_}"
+        assert L.atexn_bench_mark_exchange_trouble(0) == 0
         assert L.atexn_set_tuning(b"plane_single", 0) == 0
         check(run(), "two stages")
     finally:
         L.atexn_set_tuning(b"plane_single_polls", 500)
         L.atexn_set_tuning(b"plane_single", 1)
+        L.atexn_bench_mark_exchange_trouble(0)
 
 
 def test_channel_first_planes_across_workgroups_in_place(capi, coracle):
