@@ -502,6 +502,47 @@ def streaming_reference(case, steps, warmup):
         "note": "torch elementwise copy (1r+1w) and add (2r+1w) on the same rotating tensors"}
 
 
+def torch_ops_reference(case, steps, warmup):
+    """What the stock PyTorch-ROCm operators take on the same tensors and rotation: aten's
+    native_layer_norm / native_group_norm(groups = C) and their backward operators, called
+    directly (no autograd graph), event-timed like the library's calls.  gamma / beta are cast to
+    the storage dtype, which those operators require.  Channels-last InstanceNorm has no aten
+    kernel (group_norm wants channel-first memory), so that layout reports None."""
+    torch = case.torch
+    if case.op == "in" and case.layout == 1:
+        return None
+    tdt = case.sets[0]["x"].dtype
+    gamma, beta = case.gamma.to(tdt), case.beta.to(tdt)
+    try:
+        if case.op == "ln":
+            N, D = case.dims
+            fwd = lambda i: torch.native_layer_norm(case.sets[i % case.n_sets]["x"], [D], gamma, beta, 1e-3)
+            _, mean, rstd = fwd(0)
+            bwd = lambda i: torch.ops.aten.native_layer_norm_backward(
+                case.sets[i % case.n_sets]["dy"], case.sets[i % case.n_sets]["x"], [D], mean, rstd, gamma, beta,
+                [True, True, True])
+        else:
+            N, C, D, _ = case.dims
+            fwd = lambda i: torch.native_group_norm(case.sets[i % case.n_sets]["x"], gamma, beta, N, C, D, C, 1e-3)
+            _, mean, rstd = fwd(0)
+            bwd = lambda i: torch.ops.aten.native_group_norm_backward(
+                case.sets[i % case.n_sets]["dy"], case.sets[i % case.n_sets]["x"], mean, rstd, gamma, N, C, D, C,
+                [True, True, True])
+
+        def step(i):
+            fwd(i)
+            bwd(i)
+
+        ms_step = case.time_loop(step, steps, warmup)
+        ms_fwd = case.time_loop(fwd, steps, warmup)
+        ms_bwd = case.time_loop(bwd, steps, warmup)
+    except Exception as e:  # a comparison, never fatal
+        return {"error": str(e)[:200]}
+    return {"fwd_us": ms_fwd * 1e3, "bwd_us": ms_bwd * 1e3, "fwd_bwd_us": ms_step * 1e3,
+            "note": "aten native_layer_norm / native_group_norm(groups=C) and their backward operators, "
+                    "PyTorch-ROCm as installed, same rotating tensors"}
+
+
 # the benchmark configurations beside the default case and the targets, on the default run's line
 CONFIG_CASES = ("ln_cfg0", "ln_128_f16", "ln_128_bf16", "ln_4096_f16", "ln_4096_bf16", "ln_12288_f16",
                 "ln_12288_bf16", "in3d_ndhwc", "in3d_ncdhw")
@@ -512,9 +553,11 @@ def steps_for(name, steps):
     return max(10, steps // 10) if "3d" in name else steps
 
 
-def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=False):
+def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=False, torch_ops=False):
     op, dtype, dims = CASES[name]
     m, case = measure(name, steps, warmup, extras=not cold_only)
+    if torch_ops:
+        m["torch_ops"] = torch_ops_reference(case, steps, warmup)
     out = {
         "metric": "LN/IN fwd+bwd achieved HBM GB/s",
         "value": m["value"],
@@ -537,6 +580,8 @@ def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=F
         "streaming_reference": m.get("streaming_reference"),
         "roofline": m["roofline"],
     }
+    if torch_ops:
+        out["torch_ops"] = m["torch_ops"]
     del case
     if with_targets:
         # the second target shape, on the same driver-run line
@@ -588,6 +633,9 @@ def main():
                     help="only the rotating-buffer (cold) legs: no hot-cache loop and no HIP-graph replay (and no "
                          "torch copy / add for the targets and configurations of the default run); what a "
                          "rocprofv3 kernel trace of this file should average over")
+    ap.add_argument("--torch-ops", action="store_true",
+                    help="also time PyTorch-ROCm's own layer_norm / group_norm(groups=C) operators, forward and "
+                         "backward, on the same tensors (the case itself only, not the targets / configurations)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
                          "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
@@ -613,12 +661,13 @@ def main():
         for name in CASES:
             if name in SWEEP_ONLY_CASES:
                 continue
-            r = run_case(name, steps_for(name, args.steps), args.warmup, with_cpu=False, cold_only=args.cold_only)
+            r = run_case(name, steps_for(name, args.steps), args.warmup, with_cpu=False, cold_only=args.cold_only,
+                         torch_ops=args.torch_ops)
             print(json.dumps(r), flush=True)
         return
     print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu,
                               with_targets=args.case == DEFAULT_CASE and not args.no_targets,
-                              cold_only=args.cold_only)), flush=True)
+                              cold_only=args.cold_only, torch_ops=args.torch_ops)), flush=True)
     if args.copy_calibration:
         src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
         dst = torch.empty_like(src)
