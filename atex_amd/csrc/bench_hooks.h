@@ -28,6 +28,10 @@ int atexn_bench_describe_bwd(int op, int dtype, int layout, int64_t N, int64_t C
  * up after a few polls), recent == 0 makes it long ago (patient waits).  Synchronous. */
 int atexn_bench_mark_exchange_trouble(int recent);
 
+/* How many exchange-kernel calls ago that record was last written by a kernel (or by the function
+ * above), saturated at INT_MAX; -1 when it cannot be read.  Synchronises the device. */
+int atexn_bench_exchange_trouble_age(void);
+
 #ifdef __cplusplus
 }
 #endif

@@ -302,6 +302,18 @@ int atexn_bench_mark_exchange_trouble(int recent) {
   if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "hipMemcpy: %s", hipGetErrorString(e));
   return ATEXN_OK;
 }
+
+int atexn_bench_exchange_trouble_age(void) {
+  unsigned* word = exchange_trouble_word();
+  unsigned value = 0;
+  if (word == nullptr || hipDeviceSynchronize() != hipSuccess ||
+      hipMemcpy(&value, word, sizeof(value), hipMemcpyDeviceToHost) != hipSuccess) {
+    (void)hipGetLastError();
+    return -1;
+  }
+  const unsigned age = next_call_tag() - value;
+  return age > 0x7fffffffu ? 0x7fffffff : static_cast<int>(age);
+}
 #endif  // ATEXN_BENCH_BUILD
 
 /* ------------------------------------------------------------------ kernel level */

@@ -443,11 +443,12 @@ __device__ __forceinline__ bool exchange_wait_pair(const cl_word* pair, bool wan
   a = b = 0.f;
   const bool adaptive = trouble != nullptr && max_polls >= kExchangePatientPolls;
   for (int poll = 0; poll < max_polls; ++poll) {
+    // (the record is fetched along with the poll's own loads: one round trip, not two)
+    const bool decide = adaptive && poll == kExchangeHastyPolls - 1;
+    unsigned seen = 0;
+    if (decide) seen = __hip_atomic_load(trouble, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     if (cl_try_pair(pair, want, tag, a, b)) return true;
-    if (adaptive && poll == kExchangeHastyPolls - 1) {
-      const unsigned seen = __hip_atomic_load(trouble, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (tag - seen < kExchangeTroubleCalls) return false;
-    }
+    if (decide && tag - seen < kExchangeTroubleCalls) return false;
   }
   if (adaptive && (threadIdx.x & (kWave - 1)) == 0) {
     __hip_atomic_store(trouble, tag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

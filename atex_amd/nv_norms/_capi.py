@@ -80,6 +80,7 @@ BENCH_SIGNATURES = {
     "atexn_set_tuning": (_i, [ctypes.c_char_p, _i]),
     "atexn_bench_describe_bwd": (_i, [_i, _i, _i, _i64, _i64, _i64, ctypes.c_char_p, _sz]),
     "atexn_bench_mark_exchange_trouble": (_i, [_i]),
+    "atexn_bench_exchange_trouble_age": (_i, []),
 }
 BENCH_LIB_PATH = LIB_PATH.replace(".so", "_bench.so")
 _bench_lib = None
