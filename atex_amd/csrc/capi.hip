@@ -150,7 +150,7 @@ int atexn_abi_version(void) { return kAbiVersion; }
 int atexn_set_tuning(const char* name, int value) {
   ATEXN_REQUIRE(name != nullptr && value >= 0, "bad tuning request");
   ATEXN_REQUIRE(value >= 1 || !strcmp(name, "reverse_second_pass") || !strcmp(name, "cl_fused") ||
-                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "cl_single_xm") || !strcmp(name, "cl_single_occ") || !strcmp(name, "plane_single") || !strcmp(name, "plane_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
+                    !strcmp(name, "cl_fold_cap") || !strcmp(name, "cl_single") || !strcmp(name, "affine_fold") || !strcmp(name, "affine_fold_polls") || !strcmp(name, "cl_single_polls") || !strcmp(name, "cl_single_xm") || !strcmp(name, "cl_single_occ") || !strcmp(name, "plane_single") || !strcmp(name, "plane_single_occ") || !strcmp(name, "plane_single_polls") || !strcmp(name, "bwd_lds_rows") || !strcmp(name, "staged_rows") || !strcmp(name, "cl_narrow_tiles") || !strcmp(name, "cl_fused_split"),
                 "value must be >= 1");
   Tuning& t = tuning();
   if (!strcmp(name, "fwd_waves_per_cu")) t.fwd_waves_per_cu = value;
@@ -217,6 +217,9 @@ int atexn_set_tuning(const char* name, int value) {
     t.plane_single = value;
   } else if (!strcmp(name, "plane_single_polls")) {
     t.plane_single_polls = value;
+  } else if (!strcmp(name, "plane_single_occ")) {
+    ATEXN_REQUIRE(value == 0 || value == 1, "plane_single_occ must be 0 or 1");
+    t.plane_single_occ = value;
   } else if (!strcmp(name, "plane_nt_min_mb")) {
     t.plane_nt_min_mb = value;
   } else if (!strcmp(name, "cl_single")) {

@@ -203,6 +203,15 @@ __device__ __forceinline__ unsigned cl_slab_offset(const ClGeom& g, int C, int u
   return static_cast<unsigned>(g.slot + u * g.ppb) * static_cast<unsigned>(C) + static_cast<unsigned>(g.coff);
 }
 
+// A copy of the geometry whose per-thread fields the compiler treats as new values: a load
+// through it, on a path that is seldom taken, computes its addresses there instead of keeping
+// those of the kernel's first load alive (sixteen registers) all the way through the common path.
+__device__ __forceinline__ ClGeom cl_geom_again(const ClGeom& g) {
+  ClGeom h = g;
+  asm volatile("" : "+v"(h.slot), "+v"(h.coff));
+  return h;
+}
+
 // FULL: the host has checked that every slab of the launch has exactly U pixels per slot and that
 // every channel tile is complete, so every lane's every vector is valid: ok[] are compile-time
 // constants and the masks they feed disappear from the arithmetic (a third of the instructions

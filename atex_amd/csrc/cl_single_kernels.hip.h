@@ -280,7 +280,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
         }
       }
     }
-    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, g, C, raw, ok);
+    cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, cl_geom_again(g), C, raw, ok);
     __syncthreads();
   }
   if (g.ch_ok) {
@@ -455,8 +455,9 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
         }
       }
     }
-    cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g, C, rx, ok);
-    cl_load_slab<T, V, U, true, FULL>(dy + (g.n * D + g.p0) * C, g, C, rd, ok);
+    const ClGeom g2 = cl_geom_again(g);
+    cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g2, C, rx, ok);
+    cl_load_slab<T, V, U, true, FULL>(dy + (g.n * D + g.p0) * C, g2, C, rd, ok);
     __syncthreads();
   }
   // The owners of instance 0 also fold the instances' sums into dgamma / dbeta (below, after

@@ -71,6 +71,8 @@ struct Tuning {
   // XCD, statistics exchanged while they run, one pass (plane_single_kernels.hip.h); and its polls
   TuneInt plane_single{1};
   TuneInt plane_single_polls{500};
+  // 1: plane_bwd_single built for three workgroups per CU when a plane has more than 32 chunks
+  TuneInt plane_single_occ{1};
   TuneInt plane_nt_min_mb{256};  // forward: non-temporal loads of x from this many MiB (what no cache level retains anyway)
   TuneInt bwd_wave_groups{1};  // LayerNorm backward, 129..512 vectors per row: rows on 2 / 4 waves
   // Block-wide resident rows: longest row (in vectors) that uses 2 vectors per thread (more,

@@ -72,12 +72,17 @@ __device__ __forceinline__ int plane_chunk_vectors(int l, int S, int n_vec, int 
 // the same x comes round again before the memory-side cache has let go of it (134 MB per tensor,
 // three buffer sets in rotation: 40 -> 47 us whatever the number of chunks): the host asks for it
 // from 256 MiB.
-template <typename T, int V, int U, bool FULL, bool NT>
+// AGAIN: a load on a path that is seldom taken computes its addresses there, from a thread
+// index that the compiler treats as a new value, instead of keeping the addresses of the kernel's
+// first load alive all the way through the common path.
+template <typename T, int V, int U, bool FULL, bool NT, bool AGAIN = false>
 __device__ __forceinline__ void plane_load(const T* p, int n_here, Pack<T, V> (&raw)[U]) {
+  unsigned tid = threadIdx.x;
+  if constexpr (AGAIN) asm volatile("" : "+v"(tid));
 #pragma unroll
   for (int k = 0; k < U; ++k) {
     // (a 32-bit element offset from the chunk's start, which is the same for the whole workgroup)
-    const unsigned i = threadIdx.x + static_cast<unsigned>(k * kPlaneThreads);
+    const unsigned i = tid + static_cast<unsigned>(k * kPlaneThreads);
     const T* q = p + i * static_cast<unsigned>(V);
     if constexpr (FULL) {
       raw[k] = NT ? load_pack_last<T, V>(q) : load_pack<T, V>(q);
@@ -102,14 +107,30 @@ template <typename T, int V, int U, bool FULL>
 __device__ __forceinline__ Wf plane_chunk_stats(Pack<T, V> (&raw)[U], int n_here, Wf* buf) {
   Wf w;
   if constexpr (FULL) {
-    float f[U * V];
+    // wf_push over the thread's U * V elements, written out so that the second pass converts
+    // the elements again rather than keeping U * V floats alive beside the raw vectors (bf16
+    // has no mixed-precision arithmetic that would take the raw halves as they are: it came to
+    // 109 registers, or 98 spilled ones under the bound of 64)
+    float s = 0.f;
 #pragma unroll
     for (int k = 0; k < U; ++k) {
 #pragma unroll
-      for (int i = 0; i < V; ++i) f[k * V + i] = to_f32(raw[k].v[i]);
+      for (int i = 0; i < V; ++i) s += to_f32(raw[k].v[i]);
+    }
+    const float mb = s * (1.0f / (U * V));
+#pragma unroll
+    for (int k = 0; k < U; ++k) forget_derived(raw[k]);
+    float q = 0.f;
+#pragma unroll
+    for (int k = 0; k < U; ++k) {
+#pragma unroll
+      for (int i = 0; i < V; ++i) {
+        const float d = to_f32(raw[k].v[i]) - mb;
+        q += d * d;
+      }
     }
     w = Wf{0.f, 0.f, 0.f};
-    wf_push<U * V>(w, f);
+    wf_push_batch(w, mb, q, static_cast<float>(U * V));
   } else {
     // the thread's first nv vectors are inside the chunk
     const int nv = plane_valid<U, FULL>(n_here);
@@ -220,7 +241,7 @@ __device__ __forceinline__ void plane_wait_own(const cl_word* pair, bool want, u
 // (FULL: built for four workgroups per CU, 64 VGPRs, which the path that every launch takes needs
 // anyway; the fallback then keeps a few values in scratch memory)
 template <typename T, int V, int U, bool FULL, bool NT>
-__global__ void __launch_bounds__(kPlaneThreads, FULL ? 8 : 4)
+__global__ void __launch_bounds__(kPlaneThreads, FULL ? (__is_same(T, bf16_t) ? 6 : 8) : 4)
 plane_fwd_single(const T* __restrict__ x, cl_word* tagged, unsigned* claims, const float* __restrict__ gamma,
                  const float* __restrict__ beta, T* __restrict__ y, float* __restrict__ mean_out,
                  float* __restrict__ rstd_out, int64_t n_rows, int n_vec, int S, int chunk_vec, int C, float eps,
@@ -281,7 +302,7 @@ plane_fwd_single(const T* __restrict__ x, cl_word* tagged, unsigned* claims, con
         sm_rstd = rsqrtf(__builtin_fmaf(q, inv_d, eps));
       }
     }
-    plane_load<T, V, U, FULL, NT>(xr + static_cast<int64_t>(g.s) * chunk_vec * V, n_here, raw);
+    plane_load<T, V, U, FULL, NT, true>(xr + static_cast<int64_t>(g.s) * chunk_vec * V, n_here, raw);
     __syncthreads();
   }
   const float mean = sm_mean, rstd = sm_rstd;
@@ -365,8 +386,14 @@ struct PlaneFold {
 // tagged: [n_rows][S] pairs (sum dy, sum dy * xh) of the chunks; part: the planes' sums for the
 // column reduction over the batch that follows (layout as in rows_bwd_resident) when fold.tagged
 // is null.
-template <typename T, int V, int U, bool FULL>
-__global__ void __launch_bounds__(kPlaneThreads, 4)
+// OCC: built for three workgroups per CU instead of two (80 registers, a few of them spilled; the
+// addresses of the loads are computed again where the fallback loads the chunk again, which the
+// build for two is better off without).  It pays when a plane has so many chunks that the two
+// workgroups per CU of an XCD all belong to one plane and move in step, load - exchange - store:
+// [2, 32, 128^3] fp16 (64 chunks) 147.4 -> 143.1 us; with two chunks per plane
+// ([16, 64, 256, 256]) it loses, 71.0 -> 73.1 us.
+template <typename T, int V, int U, bool FULL, bool OCC>
+__global__ void __launch_bounds__(kPlaneThreads, OCC ? 6 : 4)
 plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
                  const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
                  unsigned* claims, T* __restrict__ dx, float* __restrict__ part, int64_t n_rows, int n_vec, int S, int chunk_vec, int C,
@@ -422,8 +449,8 @@ plane_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float*
       sm_s1 = t.x;
       sm_s2 = t.y;
     }
-    plane_load<T, V, U, FULL, true>(xr + off, n_here, rx);
-    plane_load<T, V, U, FULL, true>(dr + off, n_here, rd);
+    plane_load<T, V, U, FULL, true, OCC>(xr + off, n_here, rx);
+    plane_load<T, V, U, FULL, true, OCC>(dr + off, n_here, rd);
     __syncthreads();
   }
   const float s1 = sm_s1, s2 = sm_s2;

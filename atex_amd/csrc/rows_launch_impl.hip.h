@@ -358,7 +358,11 @@ int rows_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, c
     if (p.plane_single && static_cast<const void*>(dx) != static_cast<const void*>(dy) && exchange_allowed(st)) {
       cl_word* tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_tagged);
       const int n_vec = static_cast<int>(D / V);
-      auto fn = p.ps_full ? plane_bwd_single<T, V, kPlanPlaneVpt, true> : plane_bwd_single<T, V, kPlanPlaneVpt, false>;
+      // (three workgroups per CU when the two of an XCD's CUs would all hold chunks of one plane)
+      const bool occ = p.ps_full && tuning().plane_single_occ && p.ps_S > 32;
+      auto fn = occ         ? plane_bwd_single<T, V, kPlanPlaneVpt, true, true>
+                : p.ps_full ? plane_bwd_single<T, V, kPlanPlaneVpt, true, false>
+                            : plane_bwd_single<T, V, kPlanPlaneVpt, false, false>;
       PlaneFold pf{nullptr, dgamma, dbeta, p.part_rows};
       if (p.ps_fold) pf.tagged = reinterpret_cast<cl_word*>(static_cast<char*>(ws) + p.off_ps_fold);
       unsigned* claims = reinterpret_cast<unsigned*>(static_cast<char*>(ws) + p.off_ps_claims);

@@ -543,6 +543,12 @@ def test_channel_first_planes_across_workgroups(coracle, N, C, S, dtype):
         again = run()
         for n_, a, b in zip(names, normal, again):
             assert torch.equal(_bits(a), _bits(b)), f"second run differs in {n_}"
+        # the backward's build for three workgroups per CU (planes of more than 32 chunks) against
+        # the one for two: the same arithmetic
+        assert L.atexn_set_tuning(b"plane_single_occ", 0) == 0
+        for n_, a, b in zip(names, normal, run()):
+            assert torch.equal(_bits(a), _bits(b)), f"the build for two workgroups per CU differs in {n_}"
+        assert L.atexn_set_tuning(b"plane_single_occ", 1) == 0
         assert L.atexn_set_tuning(b"plane_single_polls", 0) == 0
         alone = run()
         for n_, a, b in zip(names, normal, alone):
@@ -562,6 +568,7 @@ def test_channel_first_planes_across_workgroups(coracle, N, C, S, dtype):
     finally:
         L.atexn_set_tuning(b"plane_single_polls", 500)
         L.atexn_set_tuning(b"plane_single", 1)
+        L.atexn_set_tuning(b"plane_single_occ", 1)
         L.atexn_bench_mark_exchange_trouble(0)
 
 
