@@ -223,10 +223,12 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
       float* o1 = N == 1 ? dbeta : xpart + C;
       const int64_t o_stride = N == 1 ? 0 : 2 * C;
       if (p.single_xm && !p.xm_fold) finals_dev = nullptr;
-      // (the backward only with at most 32 slabs per instance: with 64, three workgroups per CU
-      // are one and a half instances per XCD and the registers moved to scratch memory cost as
-      // much: [16, 128^2, 64] fp16 25.4 -> 26.4 us, [128, 64^2, 64] 49.6 -> 43.9 us)
-      const bool occ = p.single_xm && !p.xm_resident && p.S <= 32 && tuning().cl_single_occ;
+      // (the backward, which runs three workgroups per CU as it is, only with more than 32 slabs
+      // per instance and more than two instances per XCD: [64, 128^2, 64] fp16 94 -> 87 us; with
+      // fewer slabs it loses, [128, 64^2, 64] 44.0 -> 46.8 us, [32, 128^2, 32] 23.1 -> 23.8 us, and
+      // with two instances per XCD the step does, [16, 128^2, 64] 39.1 -> 40.2 us)
+      const bool occ = p.single_xm && !p.xm_resident && p.S > 32 && static_cast<int64_t>(Ni) * p.CT > 16 &&
+                       tuning().cl_single_occ;
 #define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
   do {                                                                                          \
     auto fn = occ ? cl_bwd_single<T, V, U_, FULL_, true> : cl_bwd_single<T, V, U_, FULL_, false>; \

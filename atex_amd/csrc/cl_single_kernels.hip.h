@@ -304,8 +304,11 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
 // whose workgroups are not all on the chip together): the owners leave the instances' sums at
 // o0[n * o_stride + c] (sum dy * xh) and o1[n * o_stride + c] (sum dy) instead: dgamma / dbeta
 // themselves for a single instance, partial rows for a col_reduce launch otherwise.
+// OCC: built for four workgroups per CU (128 registers, a dozen of the 16-bit kernel's 138 in
+// scratch memory), so that an XCD holds two instances of 64 slabs at a time; the plain build
+// already runs three per CU.
 template <typename T, int V, int U, bool FULL, bool OCC>
-__global__ void __launch_bounds__(kClThreads, OCC ? 3 : 2)
+__global__ void __launch_bounds__(kClThreads, OCC ? 4 : 2)
 cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __restrict__ gamma,
               const float* __restrict__ mean_in, const float* __restrict__ rstd_in, cl_word* tagged,
               cl_word* finals, cl_word* finals_dev, unsigned* claims, T* __restrict__ dx, float* __restrict__ dgamma,

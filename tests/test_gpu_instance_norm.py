@@ -307,7 +307,10 @@ def _bits(t):
                                    # the XCD-major grid: batches that are no multiples of 8, more
                                    # workgroups than the chip holds, a single instance, many instances
                                    (4, 64, 16384), (16, 64, 16384), (2, 128, 4096), (1, 64, 8192), (3, 24, 5000),
-                                   (100, 64, 2048), (5, 256, 4096)])
+                                   (100, 64, 2048), (5, 256, 4096),
+                                   # more than two instances of 64 slabs per XCD: the backward built
+                                   # for four workgroups per CU
+                                   (20, 64, 16384)])
 def test_channels_last_single_launch(coracle, N, C, S, dtype):
     """Register-resident slabs whose instance fits one XCD: statistics and their use run as ONE
     launch per direction whose workgroups exchange tagged partials while they run (every
@@ -362,6 +365,11 @@ def test_channels_last_single_launch(coracle, N, C, S, dtype):
         again = run()
         for n_, a, b in zip(names, normal, again):
             assert torch.equal(_bits(a), _bits(b)), f"second run differs in {n_}"
+        # the builds for more workgroups per CU against the plain ones: the same arithmetic
+        assert L.atexn_set_tuning(b"cl_single_occ", 0) == 0
+        for n_, a, b in zip(names, normal, run()):
+            assert torch.equal(_bits(a), _bits(b)), f"the plain build differs in {n_}"
+        assert L.atexn_set_tuning(b"cl_single_occ", 1) == 0
         assert L.atexn_set_tuning(b"cl_single_polls", 0) == 0
         alone = run()
         check(alone, "single launch, poll limit 0")
@@ -382,6 +390,7 @@ def test_channels_last_single_launch(coracle, N, C, S, dtype):
     finally:
         L.atexn_set_tuning(b"cl_single_polls", 300)
         L.atexn_set_tuning(b"cl_single", 1)
+        L.atexn_set_tuning(b"cl_single_occ", 1)
         L.atexn_bench_mark_exchange_trouble(0)
 
 
