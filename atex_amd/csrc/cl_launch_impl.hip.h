@@ -231,7 +231,8 @@ int cl_bwd_v(const T* dy, const T* x, const float* gamma, const float* mean, con
                        tuning().cl_single_occ;
 #define ATEXN_CL_BWD_SINGLE(U_, FULL_)                                                          \
   do {                                                                                          \
-    auto fn = occ ? cl_bwd_single<T, V, U_, FULL_, true> : cl_bwd_single<T, V, U_, FULL_, false>; \
+    /* (ragged slabs keep the plain build: under the bound of 128 registers theirs spills 96) */ \
+    auto fn = occ ? cl_bwd_single<T, V, U_, FULL_, FULL_> : cl_bwd_single<T, V, U_, FULL_, false>; \
     fn<<<sgrid, kClThreads, 0, st>>>(dy, x, gamma, mean, rstd, tagged, finals, finals_dev, claims, dx, dgamma, \
                                      dbeta, Ni, D, Ci, p.S, p.tpp_shift, p.slab_len, tag, polls, \
                                      xm_tiles, o0, o1, o_stride, trouble);             \

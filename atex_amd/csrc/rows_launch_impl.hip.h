@@ -74,7 +74,9 @@ BwdResidentFn<T, V, AFF> bwd_variant(int rb, bool exact, bool ragged) {
       }
       return rb == 1 ? rows_bwd_resident<T, V, TPR, VPT, 1, false, AFF, true> : nullptr;
     }
-    if constexpr (TPR != 0 && TPR <= 64) {
+    // (the planner batches backward rows only with one vector per lane: with two or three the
+    // batched kernels need more than 256 registers)
+    if constexpr (TPR != 0 && TPR <= 64 && VPT == 1) {
       if (rb == 2) return exact ? rows_bwd_resident<T, V, TPR, VPT, 2, true, AFF> : rows_bwd_resident<T, V, TPR, VPT, 2, false, AFF>;
     }
     if (rb == 1 && exact) return rows_bwd_resident<T, V, TPR, VPT, 1, true, AFF>;
