@@ -98,10 +98,15 @@ CASES = {
     # kernels on their XCD-major grid
     "in_16x128x128x64_cl": ("in", "f16", (16, 64, 128 * 128, False)),
     "in_64x128x128x64_cl": ("in", "f16", (64, 64, 128 * 128, False)),
+    # the InstanceNorm configurations in bf16 (the configurations name fp16; the ops take both)
+    "in2d_nhwc_bf16": ("in", "bf16", (8, 64, 128 * 128, False)),
+    "in2d_nchw_bf16": ("in", "bf16", (8, 64, 128 * 128, True)),
+    "in3d_ndhwc_bf16": ("in", "bf16", (2, 32, 128 ** 3, False)),
+    "in3d_ncdhw_bf16": ("in", "bf16", (2, 32, 128 ** 3, True)),
 }
 # cases that `--case all` leaves out (single-purpose sweeps and the reference's benchmark table)
 SWEEP_ONLY_CASES = frozenset(
-    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "in_16x", "in_64x", "ln_8192x", "ln_4096x")) or n.endswith("_f32")])
+    [n for n in CASES if n.startswith(("lnref_", "inref_", "in_1x", "in_16x", "in_64x", "ln_8192x", "ln_4096x")) or n.endswith("_f32") or (n.startswith("in") and n.endswith("_bf16"))])
 DEFAULT_CASE = "ln_bert"
 # the two shapes the throughput target is stated on, reported on the default run's line
 TARGET_CASES = ("ln_bert", "in2d_nhwc", "in2d_nchw")
