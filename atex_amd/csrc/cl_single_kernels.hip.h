@@ -155,6 +155,17 @@ __device__ __forceinline__ int gridDim_tiles(int xm_tiles) {
   return xm_tiles == 0 ? static_cast<int>(gridDim.z) : xm_tiles;
 }
 
+// Whether the waits of a kernel adapt to a shared GPU (exchange_wait_pair).  The kernels of small
+// slabs (four vectors per thread) do not: their launches are a few microseconds long, of which
+// the adaptive wait's code - never its read of the record - cost 0.4 of 14 in a forward + backward
+// step ([8, 64^2, 64], [2, 16^3, 128], [4, 64^2, 32] fp16), and the 300 polls that a wait on a
+// shared GPU then runs to are bounded by the same few workgroups.  With eight vectors per thread
+// the cost is within the noise (config 3: 20.35 against 20.5 us).
+template <int U>
+__device__ __forceinline__ constexpr bool cl_single_adapts() {
+  return U >= 8;
+}
+
 // ------------------------------------------------------------------------------ forward
 // tagged: [N][S][C] pairs (mean, m2) of the slabs; finals: [N][C] pairs (mean, inverse std);
 // claims: [N][tiles][S] claim words.
@@ -185,6 +196,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
   const int c_base = g.ct * cap;
   const int cap_here = C - c_base < cap ? C - c_base : cap;
   const int lane = threadIdx.x & (kWave - 1);
+  unsigned* const record = cl_single_adapts<U>() ? trouble : nullptr;
   const int wave = threadIdx.x / kWave;
   const float inv_d = 1.0f / static_cast<float>(D);
   const float n_full = static_cast<float>(slab_len);
@@ -212,7 +224,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
     for (int lc = g.s; lc < cap_here; lc += S) {
       const int c = c_base + lc;
       float pm, pq;
-      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, trouble, pm, pq)) {
+      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, record, pm, pq)) {
         fail = true;
         break;
       }
@@ -229,7 +241,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
     if (!fail) {
       float fm, frs;
       const bool want = lane < cap_here;
-      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, trouble, fm, frs)) {
+      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, record, fm, frs)) {
         if (want) {
           sm_mean[lane] = fm;
           sm_sc[lane] = gmc * frs;
@@ -330,6 +342,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
   const int c_base = g.ct * cap;
   const int cap_here = C - c_base < cap ? C - c_base : cap;
   const int lane = threadIdx.x & (kWave - 1);
+  unsigned* const record = cl_single_adapts<U>() ? trouble : nullptr;
   const int wave = threadIdx.x / kWave;
   const float inv_d = 1.0f / static_cast<float>(D);
   if (threadIdx.x == 0) sm_fail = sm_fail_dev = 0;
@@ -373,7 +386,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     for (int lc = g.s; lc < cap_here; lc += S) {
       const int c = c_base + lc;
       float pb, pa;
-      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, trouble, pb, pa)) {
+      if (!exchange_wait_pair(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, max_polls, record, pb, pa)) {
         fail = true;
         break;
       }
@@ -392,7 +405,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     if (!fail) {
       float fb_, fa_;
       const bool want = lane < cap_here;
-      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, trouble, fb_, fa_)) {
+      if (exchange_wait_pair(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, max_polls, record, fb_, fa_)) {
         if (want) constants(lane, gmc, muc, rsc, fb_, fa_);
       } else {
         fail = true;
