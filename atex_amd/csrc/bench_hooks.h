@@ -32,6 +32,13 @@ int atexn_bench_mark_exchange_trouble(int recent);
  * above), saturated at INT_MAX; -1 when it cannot be read.  Synchronises the device. */
 int atexn_bench_exchange_trouble_age(void);
 
+/* Launches, on `stream`, a kernel that does nothing but hold `workgroups` whole compute units
+ * (1024 threads and 158 of the CU's 160 KB of LDS each) for about `milliseconds` (at most 100): what a large kernel
+ * of another library does to the exchange kernels when it runs beside them on the same GPU.
+ * Every wave leaves when the time is up, or after a fixed number of loop passes whatever the
+ * clock says.  For the tests and measurements of that situation. */
+int atexn_bench_occupy(int workgroups, double milliseconds, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -306,6 +306,38 @@ int atexn_bench_mark_exchange_trouble(int recent) {
   return ATEXN_OK;
 }
 
+namespace {
+// Holds a whole CU per workgroup (its LDS) until the wall clock (100 MHz) has advanced by `ticks`
+// or `max_passes` loop passes are over, whichever comes first: it cannot outstay its bound.
+__global__ void __launch_bounds__(1024) occupy_kernel(long long ticks, int max_passes, int* sink) {
+  extern __shared__ int occupy_pad[];
+  const long long t0 = wall_clock64();
+  int v = threadIdx.x;
+  for (int pass = 0; pass < max_passes && wall_clock64() - t0 < ticks; ++pass) {
+    v = v * 1664525 + 1013904223;
+    __builtin_amdgcn_s_sleep(20);
+  }
+  occupy_pad[threadIdx.x] = v;
+  if (sink != nullptr && v == 0x7fffffff) sink[0] = occupy_pad[0];
+}
+}  // namespace
+
+int atexn_bench_occupy(int workgroups, double milliseconds, void* stream) {
+  ATEXN_REQUIRE(workgroups >= 1 && workgroups <= 1024, "1 to 1024 workgroups");
+  ATEXN_REQUIRE(milliseconds > 0.0 && milliseconds <= 100.0, "at most 100 milliseconds");
+  constexpr int kLds = 158 * 1024;  // of a CU's 160 KB: no workgroup of another kernel fits beside it
+  hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(occupy_kernel),
+                                     hipFuncAttributeMaxDynamicSharedMemorySize, kLds);
+  if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "hipFuncSetAttribute: %s", hipGetErrorString(e));
+  // a pass is a sleep of about 0.6 us: the cap is some ten times the time asked for
+  const int max_passes = static_cast<int>(milliseconds * 20000.0) + 1000;
+  occupy_kernel<<<workgroups, 1024, kLds, static_cast<hipStream_t>(stream)>>>(
+      static_cast<long long>(milliseconds * 1e5), max_passes, nullptr);
+  e = hipGetLastError();
+  if (e != hipSuccess) return set_error(ATEXN_LAUNCH_ERROR, "occupy_kernel: %s", hipGetErrorString(e));
+  return ATEXN_OK;
+}
+
 int atexn_bench_exchange_trouble_age(void) {
   unsigned* word = exchange_trouble_word();
   unsigned value = 0;

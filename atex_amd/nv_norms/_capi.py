@@ -81,6 +81,7 @@ BENCH_SIGNATURES = {
     "atexn_bench_describe_bwd": (_i, [_i, _i, _i, _i64, _i64, _i64, ctypes.c_char_p, _sz]),
     "atexn_bench_mark_exchange_trouble": (_i, [_i]),
     "atexn_bench_exchange_trouble_age": (_i, []),
+    "atexn_bench_occupy": (_i, [_i, ctypes.c_double, _vp]),
 }
 BENCH_LIB_PATH = LIB_PATH.replace(".so", "_bench.so")
 _bench_lib = None

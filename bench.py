@@ -548,6 +548,58 @@ def torch_ops_reference(case, steps, warmup):
                     "PyTorch-ROCm as installed, same rotating tensors"}
 
 
+def shared_gpu_reference(name, occupier_wgs=128, hold_ms=20.0, reps=7):
+    """One InstanceNorm case beside a kernel that holds whole CUs (atexn_bench_occupy of the
+    benchmark build, on a second stream, started first): single forward and backward calls, with
+    the kernels whose workgroups exchange results and with the two-launch kernels.  The first
+    exchange call pays for waits that run out; the later ones give such waits up early."""
+    global USE_BENCH_LIB_EVERYWHERE
+    op, dtype, dims = CASES[name]
+    if op != "in":
+        return None
+    torch = torch_mod()
+    L = bench_lib()
+    if L is None:
+        return {"error": "needs the benchmark build of the library"}
+    saved = USE_BENCH_LIB_EVERYWHERE
+    USE_BENCH_LIB_EVERYWHERE = True
+    out = {"occupier": f"{occupier_wgs} workgroups x 1024 threads x 158 KB of LDS, held for {hold_ms:g} ms on a second stream"}
+    try:
+        case = GpuCase(op, dtype, dims)
+        side = torch.cuda.Stream()
+
+        def one(fn, i):
+            torch.cuda.synchronize()
+            if L.atexn_bench_occupy(occupier_wgs, hold_ms, side.cuda_stream) != 0:
+                raise RuntimeError(L.atexn_last_error().decode())
+            torch.cuda._sleep(400000)  # the occupier gets its CUs first
+            e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+            e0.record()
+            fn(i)
+            e1.record()
+            torch.cuda.synchronize()
+            return e0.elapsed_time(e1) * 1e3
+
+        for knob, label in ((1, "exchange"), (0, "two_launch")):
+            for nm in (b"cl_single", b"plane_single", b"affine_fold"):
+                L.atexn_set_tuning(nm, knob)
+            L.atexn_bench_mark_exchange_trouble(0)
+            case.fwd(0)
+            case.bwd(0)
+            f = [one(case.fwd, i) for i in range(reps)]
+            L.atexn_bench_mark_exchange_trouble(0)
+            b = [one(case.bwd, i) for i in range(reps)]
+            out[label] = {"fwd_first_us": f[0], "fwd_us": float(np.median(f[1:])),
+                          "bwd_first_us": b[0], "bwd_us": float(np.median(b[1:]))}
+        del case
+    finally:
+        for nm in (b"cl_single", b"plane_single", b"affine_fold"):
+            L.atexn_set_tuning(nm, 1)
+        L.atexn_bench_mark_exchange_trouble(0)
+        USE_BENCH_LIB_EVERYWHERE = saved
+    return out
+
+
 # the benchmark configurations beside the default case and the targets, on the default run's line
 CONFIG_CASES = ("ln_cfg0", "ln_128_f16", "ln_128_bf16", "ln_4096_f16", "ln_4096_bf16", "ln_12288_f16",
                 "ln_12288_bf16", "in3d_ndhwc", "in3d_ncdhw")
@@ -558,7 +610,8 @@ def steps_for(name, steps):
     return max(10, steps // 10) if "3d" in name else steps
 
 
-def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=False, torch_ops=False):
+def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=False, torch_ops=False,
+             shared_gpu=0):
     op, dtype, dims = CASES[name]
     m, case = measure(name, steps, warmup, extras=not cold_only)
     if torch_ops:
@@ -588,6 +641,9 @@ def run_case(name, steps, warmup, with_cpu=True, with_targets=False, cold_only=F
     if torch_ops:
         out["torch_ops"] = m["torch_ops"]
     del case
+    if shared_gpu:
+        torch_mod().cuda.empty_cache()
+        out["shared_gpu"] = shared_gpu_reference(name, occupier_wgs=shared_gpu)
     if with_targets:
         # the second target shape, on the same driver-run line
         out["targets"] = {}
@@ -641,6 +697,9 @@ def main():
     ap.add_argument("--torch-ops", action="store_true",
                     help="also time PyTorch-ROCm's own layer_norm / group_norm(groups=C) operators, forward and "
                          "backward, on the same tensors (the case itself only, not the targets / configurations)")
+    ap.add_argument("--shared-gpu", type=int, default=0, metavar="WORKGROUPS",
+                    help="InstanceNorm cases: also time single calls while a busy kernel of the benchmark build "
+                         "holds that many whole CUs on a second stream (e.g. 128: half the chip)")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="after the case, run 5 elementwise negations of a 64 MiB tensor into "
                          "another (torch's neg kernel: reads 64 MiB, writes 64 MiB): a kernel of "
@@ -667,12 +726,13 @@ def main():
             if name in SWEEP_ONLY_CASES:
                 continue
             r = run_case(name, steps_for(name, args.steps), args.warmup, with_cpu=False, cold_only=args.cold_only,
-                         torch_ops=args.torch_ops)
+                         torch_ops=args.torch_ops, shared_gpu=args.shared_gpu)
             print(json.dumps(r), flush=True)
         return
     print(json.dumps(run_case(args.case, args.steps, args.warmup, with_cpu=not args.no_cpu,
                               with_targets=args.case == DEFAULT_CASE and not args.no_targets,
-                              cold_only=args.cold_only, torch_ops=args.torch_ops)), flush=True)
+                              cold_only=args.cold_only, torch_ops=args.torch_ops,
+                              shared_gpu=args.shared_gpu)), flush=True)
     if args.copy_calibration:
         src = torch.randn(32 << 20, device="cuda:0", dtype=torch.float16)  # 64 MiB
         dst = torch.empty_like(src)

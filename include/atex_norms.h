@@ -32,8 +32,9 @@
  *     InstanceNorm call on kernels that need no group of workgroups resident on the GPU
  *     together (two launches per direction instead of one for some shapes; same results up to
  *     the order of a few float32 additions in the statistics, same workspace sizes) -- for
- *     processes that keep other kernels running on the same GPU all the time, under which
- *     the one-launch kernels are correct but two to four times slower than the two launches;
+ *     processes that keep other kernels running on more than half of the GPU's compute units
+ *     all the time, under which the one-launch kernels are correct but two to five times slower
+ *     than the two launches;
  *   - the device the stream belongs to must be the calling thread's current device: launch
  *     plans and workspace sizes are made for the current device's compute-unit count;
  *   - data pointers need only the alignment of their element type (2 or 4 bytes): the
