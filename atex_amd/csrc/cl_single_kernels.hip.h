@@ -124,18 +124,31 @@ __device__ __forceinline__ void cl_look(const cl_word* tagged, int64_t n, int S,
 __device__ __forceinline__ int cl_claim_missing(unsigned* claims, int S, int s_self, unsigned tag,
                                                 const int (&have)[kClSingleMaxSlabs]) {
   __shared__ int sm_pick;
-  if (threadIdx.x == 0) {
-    int pick = -1;
-    for (int i = 1; i <= S && pick < 0; ++i) {
-      const int l = (s_self + i) % S;
-      if (have[l]) continue;
-      unsigned cur = __hip_atomic_load(claims + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (cur != tag && __hip_atomic_compare_exchange_strong(claims + l, &cur, tag, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
-                                                             __HIP_MEMORY_SCOPE_AGENT)) {
-        pick = l;
-      }
+  if (threadIdx.x < kWave) {
+    // a lane per slab looks at its claim word; the candidates are then tried in turn, starting
+    // behind the workgroup's own slab (so that the workgroups spread over the missing ones)
+    const int lane = threadIdx.x;
+    const int l = (s_self + 1 + lane) % S;  // lane i: the i-th slab behind this one (i < S)
+    bool open_ = false;
+    if (lane < S && !have[l]) {
+      open_ = __hip_atomic_load(claims + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != tag;
     }
-    sm_pick = pick;
+    unsigned long long cand = __ballot(open_);
+    int pick = -1;
+    while (cand != 0 && pick < 0) {  // uniform over the wave
+      const int first = __builtin_ctzll(cand);
+      int got = 0;
+      if (lane == first) {
+        unsigned cur = __hip_atomic_load(claims + l, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        got = cur != tag && __hip_atomic_compare_exchange_strong(claims + l, &cur, tag, __ATOMIC_RELAXED,
+                                                                 __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)
+                  ? 1 : 0;
+      }
+      got = __shfl(got, first, kWave);
+      if (got) pick = (s_self + 1 + first) % S;
+      cand &= cand - 1;
+    }
+    if (lane == 0) sm_pick = pick;
   }
   __syncthreads();
   return sm_pick;
@@ -184,6 +197,7 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
               float eps, unsigned tag, int max_polls, int xm_tiles, unsigned* trouble) {
   __shared__ float lds[V * kClThreads];
   __shared__ int have[kClSingleMaxSlabs];
+  __shared__ int mine[kClSingleMaxSlabs];
   __shared__ float sm_mean[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_bt[kClSingleMaxCap];
   __shared__ int sm_fail;
   const int CV = C / V;
@@ -255,15 +269,22 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
   }
   __syncthreads();
   if (sm_fail) {
-    // On its own: the partials of every slab of the instance that have not arrived, computed as
-    // their workgroups compute them and published like theirs; then the finals of every channel
-    // of the tile, folded as their owners fold them.  The slabs pass through the registers of
-    // the workgroup's own slab, which is loaded again at the end (x is intact: y != x).
+    // The partials of every slab of the instance that have not arrived get computed as their
+    // workgroups compute them and published like theirs, each by one of the workgroups that have
+    // given up.  Whoever publishes a slab's partials also does its workgroup's duty as an owner:
+    // it folds the channels that the slab owns and publishes their finals (the absent workgroup,
+    // once it runs, does both again, to the same bits).  So every channel's finals come from a
+    // running workgroup, and all that is left is to wait for them.  The slabs pass through the
+    // registers of the workgroup's own slab, which is loaded again at the end (x is intact:
+    // y != x).
     unsigned* my_claims = claims + (g.n * gridDim_tiles(xm_tiles) + g.ct) * S;
+    int n_mine = 0;  // uniform
     for (int round = 0; round < S; ++round) {
       cl_look(tagged, g.n, S, C, c_base, cap_here, tag, have);
       const int l = cl_claim_missing(my_claims, S, g.s, tag, have);
       if (l < 0) break;  // uniform
+      if (threadIdx.x == 0) mine[n_mine] = l;
+      ++n_mine;
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, false, FULL>(x + (h.n * D + h.p0) * C, h, C, raw, ok);
       float mm[V], qq[V];
@@ -274,22 +295,31 @@ cl_fwd_single(const T* __restrict__ x, cl_word* tagged, cl_word* finals, unsigne
         for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, mm[i], qq[i], tag);
       }
     }
-    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
-      const int c = c_base + lc;
-      float pm, pq;
-      cl_wait_own(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pm, pq);
-      float mu, q;
-      cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
-      if (lane == 0) {
-        const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
-        sm_mean[lc] = mu;
-        sm_sc[lc] = gamma[c] * rs;
-        sm_bt[lc] = beta[c];
-        if (lc % S == g.s) {  // an owner still serves its peers
+    __syncthreads();  // mine is written
+    for (int k = -1; k < n_mine; ++k) {
+      const int sk = k < 0 ? g.s : mine[k];
+      for (int lc = sk + wave * S; lc < cap_here; lc += (kClThreads / kWave) * S) {
+        const int c = c_base + lc;
+        float pm, pq;
+        cl_wait_own(tagged + ((g.n * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pm, pq);
+        float mu, q;
+        cl_fold_lanes_stats(pm, pq, lane, S, n_full, n_last, inv_d, mu, q);
+        if (lane == 0) {
+          const float rs = rsqrtf(__builtin_fmaf(q, inv_d, eps));
           cl_publish(finals + (g.n * C + c) * 2, mu, rs, tag);
           mean_out[g.n * C + c] = mu;
           rstd_out[g.n * C + c] = rs;
         }
+      }
+    }
+    if (wave == 0) {
+      float fm, frs;
+      const bool want = lane < cap_here;
+      cl_wait_own(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, fm, frs);
+      if (want) {
+        sm_mean[lane] = fm;
+        sm_sc[lane] = gmc * frs;
+        sm_bt[lane] = btc;
       }
     }
     cl_load_slab<T, V, U, false, FULL>(x + (g.n * D + g.p0) * C, cl_geom_again(g), C, raw, ok);
@@ -329,6 +359,7 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
               int64_t o_stride, unsigned* trouble) {
   __shared__ float lds[2 * V * kClThreads];
   __shared__ int have[kClSingleMaxSlabs];
+  __shared__ int mine[kClSingleMaxSlabs];
   __shared__ float sm_mu[kClSingleMaxCap], sm_sc[kClSingleMaxCap], sm_ca[kClSingleMaxCap], sm_cb[kClSingleMaxCap];
   __shared__ float inst[kClSingleMaxOwned][kWave][2];
   __shared__ int sm_fail, sm_fail_dev;
@@ -414,10 +445,37 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
     if (fail && lane == 0) sm_fail = 1;
   }
   __syncthreads();
+  // The sums of channel c of instance n2 from its slabs' sums (all of them are there or on their
+  // way after ensure_instance): a lane per slab, the whole wave must call.
+  auto fold_slabs = [&](int64_t n2, int c, float& b, float& a) {
+    float pb, pa;
+    cl_wait_own(tagged + ((n2 * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pb, pa);
+    b = group_sum<kWave>(lane < S ? pb : 0.f);
+    a = group_sum<kWave>(lane < S ? pa : 0.f);
+  };
+  // The owner's duty for slab sk of instance n2: the sums of the channels that the slab owns,
+  // published for the instance's workgroups and for the fold over the batch.
+  auto owner_duty = [&](int64_t n2, int sk) {
+    for (int lc = sk + wave * S; lc < cap_here; lc += (kClThreads / kWave) * S) {
+      const int c = c_base + lc;
+      float b, a;
+      fold_slabs(n2, c, b, a);
+      if (lane == 0) {
+        cl_publish(finals + (n2 * C + c) * 2, b, a, tag);
+        if (finals_dev != nullptr) {
+          cl_publish_device(finals_dev + (n2 * C + c) * 2, b, a, tag);
+        } else {
+          o0[n2 * o_stride + c] = b;
+          o1[n2 * o_stride + c] = a;
+        }
+      }
+    }
+  };
   // On its own, for instance n2 and this workgroup's tile: the sums of every slab that have not
   // arrived, computed as their workgroups compute them and published like theirs.  The slabs pass
   // through the registers of the workgroup's own slab (x and dy are intact: dx aliases neither),
   // which the caller loads again if it still needs it.
+  int n_mine = 0;  // slabs of the instance that ensure_instance computed here (uniform); they are in mine[]
   auto ensure_instance = [&](int64_t n2) {
     float mu2[V], rs2[V];
 #pragma unroll
@@ -427,10 +485,13 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       load_f32<V>(rstd_in + n2 * C + g.coff, rs2);
     }
     unsigned* my_claims = claims + (n2 * gridDim_tiles(xm_tiles) + g.ct) * S;
+    n_mine = 0;
     for (int round = 0; round < S; ++round) {
       cl_look(tagged, n2, S, C, c_base, cap_here, tag, have);
       const int l = cl_claim_missing(my_claims, S, g.s, tag, have);
       if (l < 0) break;  // uniform
+      if (threadIdx.x == 0) mine[n_mine] = l;
+      ++n_mine;
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, true, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
       cl_load_slab<T, V, U, true, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
@@ -442,34 +503,23 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
         for (int i = 0; i < V; ++i) cl_publish(o + 2 * i, a2[i], a2[V + i], tag);
       }
     }
-    __syncthreads();
-  };
-  // The sums of channel c of instance n2 from its slabs' sums (all of them are there or on their
-  // way after ensure_instance): a lane per slab, the whole wave must call.
-  auto fold_slabs = [&](int64_t n2, int c, float& b, float& a) {
-    float pb, pa;
-    cl_wait_own(tagged + ((n2 * S + (lane < S ? lane : 0)) * C + c) * 2, lane < S, tag, pb, pa);
-    b = group_sum<kWave>(lane < S ? pb : 0.f);
-    a = group_sum<kWave>(lane < S ? pa : 0.f);
+    __syncthreads();  // mine is written
+    // whoever publishes a slab's sums also does its workgroup's duty as an owner (the absent
+    // workgroup, once it runs, does both again, to the same bits): every channel's sums thus
+    // come from a running workgroup
+    for (int k = 0; k < n_mine; ++k) owner_duty(n2, mine[k]);
   };
   if (sm_fail) {
+    // What is missing of the instance's sums, this workgroup's own duty as an owner (again, if
+    // the wait that ran out was the one for the sums of the instance), and then all that is left
+    // is to wait for every channel's sums: they come from running workgroups.
     ensure_instance(g.n);
-    for (int lc = wave; lc < cap_here; lc += kClThreads / kWave) {
-      const int c = c_base + lc;
-      float b, a;
-      fold_slabs(g.n, c, b, a);
-      if (lane == 0) {
-        constants(lc, gamma[c], mean_in[g.n * C + c], rstd_in[g.n * C + c], b, a);
-        if (lc % S == g.s) {  // an owner still serves its peers
-          cl_publish(finals + (g.n * C + c) * 2, b, a, tag);
-          if (finals_dev != nullptr) {
-            cl_publish_device(finals_dev + (g.n * C + c) * 2, b, a, tag);
-          } else {
-            o0[g.n * o_stride + c] = b;
-            o1[g.n * o_stride + c] = a;
-          }
-        }
-      }
+    owner_duty(g.n, g.s);
+    if (wave == 0) {
+      float fb_, fa_;
+      const bool want = lane < cap_here;
+      cl_wait_own(finals + (g.n * C + c_base + (want ? lane : 0)) * 2, want, tag, fb_, fa_);
+      if (want) constants(lane, gmc, muc, rsc, fb_, fa_);
     }
     const ClGeom g2 = cl_geom_again(g);
     cl_load_slab<T, V, U, true, FULL>(x + (g.n * D + g.p0) * C, g2, C, rx, ok);

@@ -33,7 +33,7 @@
  *     together (two launches per direction instead of one for some shapes; same results up to
  *     the order of a few float32 additions in the statistics, same workspace sizes) -- for
  *     processes that keep other kernels running on more than half of the GPU's compute units
- *     all the time, under which the one-launch kernels are correct but two to five times slower
+ *     all the time, under which the one-launch kernels are correct but two to three times slower
  *     than the two launches;
  *   - the device the stream belongs to must be the calling thread's current device: launch
  *     plans and workspace sizes are made for the current device's compute-unit count;
