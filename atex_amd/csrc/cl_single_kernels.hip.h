@@ -25,10 +25,12 @@
 //
 // Nothing here can hang: every wait is a bounded number of polls.  A workgroup whose wait runs
 // out (its peers are not resident: another kernel holds the CUs; or the placement assumption
-// does not hold on this device) stops relying on anyone and recomputes, with the same code and
-// therefore to the same bits, the partials of every slab of its instance from x itself.  That
-// is why the host keeps callers that pass y == x (dx == dy) on the two-stage kernels: a peer may
-// already have overwritten its part of x by then.
+// does not hold on this device) stops relying on workgroups that may not be running: together
+// with the others that have given up it computes, with the same code and therefore to the same
+// bits, the partials of the slabs that are missing, from x itself, and does the duty of their
+// workgroups as owners (below, at cl_look); from then on it only waits for running workgroups.
+// That is why the host keeps callers that pass y == x (dx == dy) on the two-stage kernels: a
+// peer may already have overwritten its part of x by then.
 //
 // Counterpart in the reference: the single-kernel channels-last variant that keeps an instance
 // in one block's shared memory (fused_instance_norm_op.cu:1066-1165); it stops at D <= 372.
@@ -102,6 +104,8 @@ __device__ __forceinline__ bool cl_single_place(int64_t N, int S, int xm_tiles, 
 // resident together because another kernel fills part of the chip, the resident ones thus share
 // out the slabs of the absent ones instead of each redoing the whole instance; the absent ones,
 // once started, find everything published, publish their own again with the same bits and go on.)
+// Whoever publishes a slab's partials also does its workgroup's duty as an owner (step 2 above)
+// for the channels that the slab owns, so every channel's finals come from a running workgroup.
 // Contains barriers; have is valid for every thread afterwards.
 __device__ __forceinline__ void cl_look(const cl_word* tagged, int64_t n, int S, int C, int c_base, int cap_here,
                                         unsigned tag, int (&have)[kClSingleMaxSlabs]) {
