@@ -157,6 +157,13 @@ __device__ __forceinline__ int cl_claim_missing(unsigned* claims, int S, int s_s
   __syncthreads();
   return sm_pick;
 }
+// The first slab whose partials have not been seen (-1: none); the same in every thread.
+__device__ __forceinline__ int cl_first_missing(int S, const int (&have)[kClSingleMaxSlabs]) {
+  for (int l = 0; l < S; ++l) {
+    if (!have[l]) return l;
+  }
+  return -1;
+}
 // Polls that a workgroup allows for values that it has published itself, has just seen, or knows
 // to be in the hands of a running workgroup to show up in its device-scope loads: they are on
 // their way, this only bounds the wait.
@@ -489,13 +496,21 @@ cl_bwd_single(const T* __restrict__ dy, const T* __restrict__ x, const float* __
       load_f32<V>(rstd_in + n2 * C + g.coff, rs2);
     }
     unsigned* my_claims = claims + (n2 * gridDim_tiles(xm_tiles) + g.ct) * S;
+    // Another instance's workgroups sit on another XCD: what they publish with plain stores is
+    // not to be seen from here before their L2 lets go of it, and what is published from here
+    // they do not see either.  So for another instance (the fold over the batch, below) nothing
+    // is claimed and no claim is honoured: whatever this workgroup cannot see it computes itself,
+    // for its own use.
+    const bool same_xcd = n2 == g.n;
     n_mine = 0;
     for (int round = 0; round < S; ++round) {
       cl_look(tagged, n2, S, C, c_base, cap_here, tag, have);
-      const int l = cl_claim_missing(my_claims, S, g.s, tag, have);
+      const int l = same_xcd ? cl_claim_missing(my_claims, S, g.s, tag, have) : cl_first_missing(S, have);
       if (l < 0) break;  // uniform
-      if (threadIdx.x == 0) mine[n_mine] = l;
-      ++n_mine;
+      if (same_xcd) {
+        if (threadIdx.x == 0) mine[n_mine] = l;
+        ++n_mine;
+      }
       const ClGeom h = cl_geom_of_slab(g, l, D, slab_len);
       cl_load_slab<T, V, U, true, FULL>(x + (n2 * D + h.p0) * C, h, C, rx, ok);
       cl_load_slab<T, V, U, true, FULL>(dy + (n2 * D + h.p0) * C, h, C, rd, ok);
