@@ -121,9 +121,9 @@ MEASURED_TRAFFIC = {
     "ln_4096_f16": 412.22e6,            # rows_bwd_resident
     "ln_12288_f16": 176.84e6,           # rows_bwd_resident (151.0 MB of rows + 25.2 MB of partial rows)
     "in2d_nchw": 50.58e6,               # rows_bwd_resident (row-affine, plane sums folded in the kernel)
-    "in2d_nhwc": 51.68e6,               # cl_bwd_single
+    "in2d_nhwc": 51.71e6,               # cl_bwd_single
     "in3d_ndhwc": 536.94e6 + 805.87e6,  # cl_bwd_sums + cl_bwd_apply
-    "in3d_ncdhw": 813.26e6,             # plane_bwd_single (plane sums folded in the kernel)
+    "in3d_ncdhw": 813.19e6,             # plane_bwd_single (plane sums folded in the kernel)
 }
 ESIZE = {"f32": 4, "f16": 2, "bf16": 2}
 
